@@ -1,0 +1,67 @@
+"""The Python entry point: load a model folder, generate, or step by hand.
+
+It mirrors the reference's library demo (examples/generate.rs:12-44: load, make
+caches, loop {forward, pick, stop?, append}) with its runner's option names
+(src/bin/runner.rs:24-123), for batches of prompts given as token ids.
+"""
+from __future__ import annotations
+
+from typing import Sequence
+
+import torch
+
+from .engine import Engine, GenerationResult, StepEntry, generate as _generate
+from .parts import load_model, random_model
+from .sampling import DEFAULT_SEED, SamplingParams
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           "f32": torch.float32}
+
+
+def as_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        return dtype
+    try:
+        return _DTYPES[str(dtype).lower()]
+    except KeyError:
+        raise ValueError(f"dtype {dtype!r}: expected bfloat16 or float32") from None
+
+
+class Model:
+    """A loaded model with a cache sized for ``max_batch`` sequences of ``max_seq_len`` tokens."""
+
+    def __init__(self, decoder, max_batch: int = 8, max_seq_len: int = 4096, max_tokens: int | None = None):
+        self.decoder = decoder
+        self.config = getattr(decoder, "config", None)
+        max_seq_len = min(max_seq_len, decoder.spec.max_positions)
+        page = 32
+        per_seq = -(-max_seq_len // page) * page
+        self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
+        self.engine = Engine(decoder, self.cache)
+
+    @classmethod
+    def load(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **cache_options) -> "Model":
+        return cls(load_model(model_dir, as_dtype(dtype), device), **cache_options)
+
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", **cache_options) -> "Model":
+        """Random weights made in memory from a config.json dict or a typed configuration."""
+        return cls(random_model(config, seed, as_dtype(dtype), device), **cache_options)
+
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 600, temperature: float = 0.0,
+                 top_k: int = 0, top_p: float = 1.0, repetition_penalty: float = 1.0, seed: int = DEFAULT_SEED,
+                 stop_token_ids: Sequence[int] = (), ignore_eos: bool = False, max_batch: int | None = None,
+                 on_token=None) -> GenerationResult:
+        params = SamplingParams(temperature, top_k, top_p, repetition_penalty, seed)
+        return _generate(self.engine, prompts, max_new_tokens, params, stop_token_ids, ignore_eos, max_batch, on_token)
+
+    def step(self, entries) -> torch.Tensor:
+        """``entries``: ``(slot, tokens, want)`` triples; float32 logits at the wanted places."""
+        return self.engine.step([e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries])
+
+
+def generate(model_dir: str, prompts, dtype="bfloat16", **options) -> list:
+    """One call from a folder to generated token ids."""
+    longest = max(len(p) for p in prompts) + options.get("max_new_tokens", 600)
+    model = Model.load(model_dir, dtype, max_batch=min(len(prompts), 64), max_seq_len=longest)
+    return model.generate(prompts, **options).tokens

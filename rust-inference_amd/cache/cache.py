@@ -1,0 +1,184 @@
+"""The cache: what live sequences keep between steps.
+
+A model's mixers say what they need per cache entry: keys and values for every
+token (optionally only a window of them), or a state of fixed size per sequence.
+Entries with the same key/value geometry form a group with storage and a page
+pool of its own; every state entry has an arena of its own, one row per slot.
+A sequence holds one slot from its first step to its end, and the slot addresses
+all of these.  Lengths are per slot: sequences of a batch advance by different
+numbers of tokens.
+
+The reference keeps one page table per layer and advances every sequence by the
+same count (src/kvcache.rs:106-135, :185-187); here one table serves all layers
+of a group and is sent to the device once per step.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import torch
+
+from ..errors import CacheError
+from .pages import PagePool, UNMAPPED
+from .slots import SlotAllocator
+
+PAGE_SIZE = 32   # tokens per page, as in the reference (src/kvcache.rs:12)
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values of ``kv_heads`` heads of ``head_dim`` for every token, or for
+    the last ``window`` tokens only."""
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A tensor of fixed shape per sequence, zero when the sequence starts."""
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+class KVGroup:
+    """Storage for all cache entries that share one key/value geometry.
+
+    ``k_pages[e]`` and ``v_pages[e]`` are ``[num_pages, kv_heads, page_size, head_dim]``
+    for entry ``e`` of the group (the reference's layout: src/kvcache.rs:42-50,
+    :145-147); one page number means the same page in every entry.
+    """
+
+    def __init__(self, need: KVNeed, entries: list[int], num_pages: int, num_slots: int,
+                 max_pages_per_slot: int, page_size: int, dtype, device, allocate: bool):
+        self.need, self.entries, self.page_size = need, list(entries), page_size
+        self.pool = PagePool(num_pages, page_size, num_slots, max_pages_per_slot, need.window)
+        self.index_of = {e: i for i, e in enumerate(self.entries)}
+        shape = (len(self.entries), num_pages, need.kv_heads, page_size, need.head_dim)
+        self.k_pages = torch.zeros(shape, dtype=dtype, device=device) if allocate else None
+        self.v_pages = torch.zeros(shape, dtype=dtype, device=device) if allocate else None
+
+    def table_rows(self, slots: Sequence[int], width: int) -> list[list[int]]:
+        return [self.pool.tables[s][:width] for s in slots]
+
+
+@dataclass
+class KVView:
+    """What a mixer gets for its cache entry in a step."""
+    group_index: int
+    k_pages: torch.Tensor
+    v_pages: torch.Tensor
+    page_size: int
+    window: Optional[int]
+
+
+class Cache:
+    def __init__(self, needs: Sequence[object], num_slots: int, max_tokens: int, max_seq_len: int,
+                 dtype=torch.bfloat16, device="cpu", page_size: int = PAGE_SIZE, allocate: bool = True):
+        """``needs[e]`` is the need of cache entry ``e`` (None for an entry nothing
+        uses).  ``max_tokens`` is the most tokens all live sequences hold together,
+        each sequence's count rounded up to whole pages; ``max_seq_len`` is the most
+        one sequence may hold."""
+        if max_tokens < 1 or max_seq_len < 1:
+            raise CacheError("max_tokens and max_seq_len must be positive")
+        self.page_size, self.num_slots = page_size, num_slots
+        self.max_seq_len = max_seq_len
+        self.device, self.dtype = device, dtype
+        self.slots = SlotAllocator(num_slots)
+        self.lengths = [0] * num_slots
+        self.max_pages_per_slot = -(-max_seq_len // page_size)
+        num_pages = -(-max_tokens // page_size)
+        self.needs = list(needs)
+        self.groups: list[KVGroup] = []
+        self._kv_of_entry: dict[int, tuple[int, int]] = {}
+        self._state: dict[int, torch.Tensor] = {}
+        by_need: dict[KVNeed, list[int]] = {}
+        for e, need in enumerate(self.needs):
+            if isinstance(need, KVNeed):
+                by_need.setdefault(need, []).append(e)
+            elif isinstance(need, StateNeed):
+                self._state[e] = torch.zeros((num_slots, *need.shape), dtype=need.dtype, device=device)
+            elif need is not None:
+                raise CacheError(f"cache entry {e}: unknown need {need!r}")
+        for need, entries in by_need.items():
+            g = KVGroup(need, entries, num_pages, num_slots, self.max_pages_per_slot, page_size, dtype, device, allocate)
+            for e in entries:
+                self._kv_of_entry[e] = (len(self.groups), g.index_of[e])
+            self.groups.append(g)
+
+    # ---- slots
+    def acquire(self) -> int:
+        slot = self.slots.acquire()
+        self.lengths[slot] = 0
+        for arena in self._state.values():
+            arena[slot].zero_()
+        return slot
+
+    def release(self, slot: int) -> None:
+        self.slots.release(slot)
+        for g in self.groups:
+            g.pool.release(slot)
+        self.lengths[slot] = 0
+
+    def length(self, slot: int) -> int:
+        self.slots.check_held(slot)
+        return self.lengths[slot]
+
+    # ---- steps
+    def reserve(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
+        """Map pages for the tokens a step is about to write.  Either every sequence
+        gets its pages or the cache is left as it was."""
+        if len(set(slots)) != len(slots):
+            raise CacheError("a slot appears twice in one step")
+        for s, n in zip(slots, new_tokens):
+            self.slots.check_held(s)
+            if n < 1:
+                raise CacheError(f"slot {s}: a step needs at least one token")
+            if self.lengths[s] + n > self.max_seq_len:
+                raise CacheError(f"slot {s} would reach {self.lengths[s] + n} tokens, "
+                                 f"the cache holds {self.max_seq_len} per sequence")
+        for g in self.groups:
+            want = sum(g.pool.pages_needed(s, self.lengths[s], n) for s, n in zip(slots, new_tokens))
+            if want > g.pool.free_count:
+                raise CacheError(f"cache out of pages: the step needs {want} more, {g.pool.free_count} of "
+                                 f"{g.pool.num_pages} are free ({g.page_size} tokens each)")
+        for g in self.groups:
+            for s, n in zip(slots, new_tokens):
+                g.pool.reserve(s, self.lengths[s], n)
+
+    def commit(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
+        """The step has written its tokens: advance the lengths, drop what fell out of a window."""
+        for s, n in zip(slots, new_tokens):
+            self.lengths[s] += n
+            for g in self.groups:
+                g.pool.trim_behind_window(s, self.lengths[s])
+
+    # ---- views for mixers
+    def kv(self, entry: int) -> KVView:
+        gi, ei = self._kv_of_entry[entry]
+        g = self.groups[gi]
+        return KVView(gi, g.k_pages[ei], g.v_pages[ei], g.page_size, g.need.window)
+
+    def state(self, entry: int) -> torch.Tensor:
+        return self._state[entry]
+
+    def has_state(self, entry: int) -> bool:
+        return entry in self._state
+
+    # ---- accounting
+    def free_pages(self) -> list[int]:
+        return [g.pool.free_count for g in self.groups]
+
+    def check_consistent(self) -> None:
+        for g in self.groups:
+            g.pool.check_consistent()
+            for s in range(self.num_slots):
+                if not self.slots.is_held(s) and g.pool.pages_of(s):
+                    raise CacheError(f"slot {s} is free but still holds pages")
+        held = len(self.slots.held_slots())
+        if held + self.slots.free_count != self.num_slots:
+            raise CacheError("a slot is lost")
+
+
+__all__ = ["Cache", "KVNeed", "StateNeed", "KVGroup", "KVView", "PAGE_SIZE", "UNMAPPED"]

@@ -1,0 +1,63 @@
+// C interface of the kernel library.  Every function returns 0 on success; on a
+// non-zero return ri_last_error() holds the reason and nothing was launched.
+// Pointers are device pointers unless said otherwise; `stream` is a hipStream_t.
+// dtype arguments take RiDtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* ri_last_error(void);
+int ri_abi_version(void);
+
+// out[t, :] = table[ids[t], :] as float32.  ids are int32 and must be < vocab (checked by the caller).
+int ri_embed_gather(float* out, const void* table, int table_dtype, const int32_t* ids,
+                    int tokens, int dim, void* stream);
+
+// r = residual[src] (+ pending[src]); if rows == NULL: src = row and residual[row] = r is written back;
+// else src = rows[row] and nothing is written back.  out[row] = r * rsqrt(mean(r^2) + eps) * gain.
+// residual float32, pending of pending_dtype (may be NULL), gain float32, out of out_dtype.
+int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype,
+                   const float* gain, float eps, const int32_t* rows, int n_rows, int dim, void* stream);
+
+// Plain residual add on gathered rows, no norm: out[row] = residual[src] + pending[src], float32.
+int ri_add_rows(float* out, const float* residual, const void* pending, int pending_dtype,
+                const int32_t* rows, int n_rows, int dim, void* stream);
+
+// Per-head RMSNorm of q and k (gains may be NULL: no norm), rotate-half position encoding of the first
+// rot_dim elements of each head (inv_freq NULL: none), in place for q, and write of k and v into the pages.
+// qkv: [tokens, (heads + 2 kv_heads) * head_dim] of act_dtype.  tok_pos/tok_seq: int32 [tokens].
+// page_table: int32 [seqs, table_width].  k_pages/v_pages: [pages, kv_heads, page_size, head_dim] of cache_dtype.
+int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
+                             const float* inv_freq, int rot_dim, const int32_t* tok_pos, const int32_t* tok_seq,
+                             const int32_t* page_table, int table_width, void* k_pages, void* v_pages,
+                             int cache_dtype, int tokens, int heads, int kv_heads, int head_dim, int page_size,
+                             int num_pages, void* stream);
+
+// Causal grouped-query attention of each new token over its sequence's pages (any number of new tokens
+// per sequence).  q is read from qkv rows (row stride q_stride elements); out: [tokens, heads * head_dim].
+// window <= 0: all keys 0..pos; else keys max(0, pos - window + 1)..pos.
+int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const void* k_pages, const void* v_pages,
+                 int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
+                 int table_width, int tokens, int heads, int kv_heads, int head_dim, int page_size, int window,
+                 float scale, void* stream);
+
+// out[M, N] (float32) = x[M, K] (float32) . w[N, K]^T, w float32 or bfloat16; true 32-bit arithmetic.
+int ri_gemm_f32(float* out, const float* x, const void* w, int w_dtype, int m, int n, int k, void* stream);
+
+// out[M, N] (out_dtype) = x[M, K] . w[N, K]^T for bfloat16 x and w, float32 accumulation, M <= 8.
+// swiglu != 0: w is [2 * N, K] = gate rows then up rows and out[m, n] = silu(gate) * up.
+int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
+                 void* stream);
+
+// out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
+int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);
+
+// ids[r] = first index of the maximum of logits[r, :] (float32).
+int ri_argmax(int32_t* ids, const float* logits, int rows, int vocab, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

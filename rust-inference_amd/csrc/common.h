@@ -1,0 +1,88 @@
+// Shared device helpers for the gfx950 kernels: number formats, 64-lane reductions,
+// launch checking.  Everything here is written for CDNA4 wavefronts of 64 lanes.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define RI_WAVE 64
+
+// dtype codes of the C interface
+enum RiDtype { RI_F32 = 0, RI_BF16 = 1 };
+
+typedef uint16_t bf16_t;   // bfloat16 carried as its bits
+
+// A bfloat16 is the upper half of a 32-bit float (the reference: src/dtype.rs:75-77).
+__device__ __forceinline__ float bf16_to_f32(bf16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// Round to nearest, ties to even; a NaN stays a quiet NaN (the reference: src/dtype.rs:82-89).
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (bf16_t)((u >> 16) | 0x0040u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+__device__ __forceinline__ void from_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ void from_f32(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// Sum over the 64 lanes of a wavefront; every lane gets the result.  The order of
+// the additions is fixed, so the result does not depend on anything but the inputs.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = RI_WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, RI_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = RI_WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, RI_WAVE));
+    return v;
+}
+
+// Sum over a workgroup of up to 1024 threads (a multiple of 64).  `scratch` is an LDS
+// array of at least 16 floats.  All threads get the result.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
+    const int nwaves = (blockDim.x + RI_WAVE - 1) / RI_WAVE;
+    v = wave_sum(v);
+    __syncthreads();                      // scratch may still be read from an earlier call
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < nwaves; ++w) total += scratch[w];
+    return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
+    const int nwaves = (blockDim.x + RI_WAVE - 1) / RI_WAVE;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = -INFINITY;
+    for (int w = 0; w < nwaves; ++w) total = fmaxf(total, scratch[w]);
+    return total;
+}
+
+// ---- host side: error text of the last refused or failed call (per thread)
+void ri_set_error(const char* fmt, ...);
+
+#define RI_REQUIRE(cond, ...)                 \
+    do {                                      \
+        if (!(cond)) {                        \
+            ri_set_error(__VA_ARGS__);        \
+            return 1;                         \
+        }                                     \
+    } while (0)
+
+#define RI_LAUNCH_CHECK(name)                                                   \
+    do {                                                                        \
+        hipError_t e_ = hipGetLastError();                                      \
+        if (e_ != hipSuccess) {                                                 \
+            ri_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+            return 2;                                                           \
+        }                                                                       \
+    } while (0)

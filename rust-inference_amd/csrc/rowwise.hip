@@ -1,0 +1,169 @@
+// Row-wise kernels: embedding gather, fused residual add + RMSNorm, SwiGLU, argmax.
+// One workgroup per row; all statistics in float32.
+#include "api.h"
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+// out[t, :] = table[ids[t], :] (the reference: src/cuda/kernels.cu:90-95), widened to float32
+// because the residual stream is kept in 32-bit.
+template <typename TW>
+__global__ void embed_gather_kernel(float* __restrict__ out, const TW* __restrict__ table,
+                                    const int32_t* __restrict__ ids, int dim) {
+    const int t = blockIdx.x;
+    const TW* row = table + (size_t)ids[t] * dim;
+    float* o = out + (size_t)t * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) o[d] = to_f32(row[d]);
+}
+
+extern "C" int ri_embed_gather(float* out, const void* table, int table_dtype, const int32_t* ids,
+                               int tokens, int dim, void* stream) {
+    RI_REQUIRE(tokens > 0 && dim > 0, "embed_gather: tokens %d, dim %d", tokens, dim);
+    RI_REQUIRE(table_dtype == RI_F32 || table_dtype == RI_BF16, "embed_gather: table dtype %d", table_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    if (table_dtype == RI_F32)
+        embed_gather_kernel<float><<<tokens, 256, 0, s>>>(out, (const float*)table, ids, dim);
+    else
+        embed_gather_kernel<bf16_t><<<tokens, 256, 0, s>>>(out, (const bf16_t*)table, ids, dim);
+    RI_LAUNCH_CHECK("embed_gather");
+    return 0;
+}
+
+// ------------------------------------------------------------------ residual add + RMSNorm
+// r = residual + pending is the new residual stream; out = r * (1 / sqrt(mean(r^2) + eps)) * gain,
+// multiplied in that order (the reference: src/ops/norm.rs:7-10, :25-30, :53-58).  The sum stays in
+// float32 and is not rounded before the variance is taken.
+template <typename TP, typename TO>
+__global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ residual, const TP* __restrict__ pending,
+                                   const float* __restrict__ gain, float eps, const int32_t* __restrict__ rows,
+                                   int dim) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[row] : row) * dim;
+    const bool write_back = rows == nullptr;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float v = residual[src + d];
+        if (pending) v += to_f32(pending[src + d]);
+        if (write_back && pending) residual[src + d] = v;
+        ss += v * v;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)dim + eps);
+    TO* o = out + (size_t)row * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float v = residual[src + d];                       // written by this same thread when write_back
+        if (pending && !write_back) v += to_f32(pending[src + d]);
+        from_f32(o + d, v * inv * gain[d]);
+    }
+}
+
+template <typename TP>
+static void launch_add_rmsnorm(void* out, int out_dtype, float* residual, const TP* pending, const float* gain,
+                               float eps, const int32_t* rows, int n_rows, int dim, hipStream_t s) {
+    if (out_dtype == RI_F32)
+        add_rmsnorm_kernel<TP, float><<<n_rows, 256, 0, s>>>((float*)out, residual, pending, gain, eps, rows, dim);
+    else
+        add_rmsnorm_kernel<TP, bf16_t><<<n_rows, 256, 0, s>>>((bf16_t*)out, residual, pending, gain, eps, rows, dim);
+}
+
+extern "C" int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype,
+                              const float* gain, float eps, const int32_t* rows, int n_rows, int dim, void* stream) {
+    RI_REQUIRE(n_rows > 0 && dim > 0, "add_rmsnorm: rows %d, dim %d", n_rows, dim);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "add_rmsnorm: out dtype %d", out_dtype);
+    RI_REQUIRE(pending_dtype == RI_F32 || pending_dtype == RI_BF16, "add_rmsnorm: pending dtype %d", pending_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    if (pending_dtype == RI_F32)
+        launch_add_rmsnorm<float>(out, out_dtype, residual, (const float*)pending, gain, eps, rows, n_rows, dim, s);
+    else
+        launch_add_rmsnorm<bf16_t>(out, out_dtype, residual, (const bf16_t*)pending, gain, eps, rows, n_rows, dim, s);
+    RI_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+}
+
+template <typename TP>
+__global__ void add_rows_kernel(float* __restrict__ out, const float* __restrict__ residual,
+                                const TP* __restrict__ pending, const int32_t* __restrict__ rows, int dim) {
+    const int row = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[row] : row) * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float v = residual[src + d];
+        if (pending) v += to_f32(pending[src + d]);
+        out[(size_t)row * dim + d] = v;
+    }
+}
+
+extern "C" int ri_add_rows(float* out, const float* residual, const void* pending, int pending_dtype,
+                           const int32_t* rows, int n_rows, int dim, void* stream) {
+    RI_REQUIRE(n_rows > 0 && dim > 0, "add_rows: rows %d, dim %d", n_rows, dim);
+    hipStream_t s = (hipStream_t)stream;
+    if (pending_dtype == RI_F32)
+        add_rows_kernel<float><<<n_rows, 256, 0, s>>>(out, residual, (const float*)pending, rows, dim);
+    else if (pending_dtype == RI_BF16)
+        add_rows_kernel<bf16_t><<<n_rows, 256, 0, s>>>(out, residual, (const bf16_t*)pending, rows, dim);
+    else
+        RI_REQUIRE(false, "add_rows: pending dtype %d", pending_dtype);
+    RI_LAUNCH_CHECK("add_rows");
+    return 0;
+}
+
+// ------------------------------------------------------------------ SwiGLU
+// silu(z) = z / (1 + exp(-z)) (the reference: src/ops/elementwise.rs:9-12); gate = silu(gate) * up.
+__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
+
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ y, int inter) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= inter) return;
+    const T* row = y + (size_t)t * 2 * inter;
+    from_f32(out + (size_t)t * inter + i, silu(to_f32(row[i])) * to_f32(row[inter + i]));
+}
+
+extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream) {
+    RI_REQUIRE(tokens > 0 && inter > 0, "swiglu: tokens %d, inter %d", tokens, inter);
+    RI_REQUIRE(tokens <= 65535, "swiglu: %d tokens exceed one launch (65535)", tokens);
+    dim3 grid((inter + 255) / 256, tokens);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == RI_F32)
+        swiglu_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)y, inter);
+    else if (dtype == RI_BF16)
+        swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, inter);
+    else
+        RI_REQUIRE(false, "swiglu: dtype %d", dtype);
+    RI_LAUNCH_CHECK("swiglu");
+    return 0;
+}
+
+// ------------------------------------------------------------------ argmax
+// First index of the row maximum: of equal values the lower index wins
+// (the reference: src/ops/reduce.rs:18-25, src/cuda/kernels.cu:182, :189).  A NaN never wins.
+__device__ __forceinline__ void better(float& v, int& i, float ov, int oi) {
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+
+__global__ void argmax_kernel(int32_t* __restrict__ ids, const float* __restrict__ logits, int vocab) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const float* row = logits + (size_t)blockIdx.x * vocab;
+    float v = -INFINITY;
+    int idx = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) better(v, idx, row[i], i);
+    for (int m = RI_WAVE / 2; m > 0; m >>= 1) {
+        float ov = __shfl_xor(v, m, RI_WAVE);
+        int oi = __shfl_xor(idx, m, RI_WAVE);
+        better(v, idx, ov, oi);
+    }
+    const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
+    if (lane == 0) { sv[wave] = v; si[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x / RI_WAVE); ++w) better(v, idx, sv[w], si[w]);
+        ids[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
+    }
+}
+
+extern "C" int ri_argmax(int32_t* ids, const float* logits, int rows, int vocab, void* stream) {
+    RI_REQUIRE(rows > 0 && vocab > 0, "argmax: rows %d, vocab %d", rows, vocab);
+    argmax_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(ids, logits, vocab);
+    RI_LAUNCH_CHECK("argmax");
+    return 0;
+}

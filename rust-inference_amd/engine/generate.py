@@ -1,0 +1,170 @@
+"""The generation loop above the step function.
+
+Requests (prompts as token ids) are served in batches: the sequences of a batch
+start together with their prompts in one step, then take one token each per step;
+a sequence that ends leaves the batch and gives its slot and pages back at once,
+and the steps after it no longer carry it.  When a batch has ended the next one
+starts, on the same cache, until every request is served.
+
+Per sequence the loop is the reference's (src/bin/runner.rs:287-313): the first
+token comes from the prompt's logits and counts toward ``max_new_tokens``; a stop
+token is tested before it is put out, is not part of the output and is never fed
+back; the last token allowed is put out but not fed.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Sequence
+
+from ..errors import CacheError, ShapeError
+from ..sampling import SamplingParams, SequenceSampler, sample_batch
+from .step import StepEntry
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_tokens: int = 0           # tokens produced by decode steps (the reference's `generated - 1`)
+    decode_seconds: float = 0.0
+    decode_steps: int = 0
+    batches: int = 0
+
+    @property
+    def prefill_tokens_per_second(self) -> float:
+        return self.prompt_tokens / self.prefill_seconds if self.prefill_seconds > 0 else 0.0
+
+    @property
+    def decode_tokens_per_second(self) -> float:
+        return self.decode_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+
+@dataclass
+class GenerationResult:
+    tokens: list                     # per request, the generated token ids (stop token not included)
+    finish_reasons: list             # per request: "stop" or "length"
+    stats: GenerationStats = field(default_factory=GenerationStats)
+
+
+def pages_for(prompt_len: int, max_new_tokens: int, page_size: int) -> int:
+    """Pages a sequence can come to hold: the last generated token is never fed, so the
+    cache sees ``prompt_len + max_new_tokens - 1`` tokens at most."""
+    held = prompt_len + max(max_new_tokens, 1) - 1
+    return -(-held // page_size)
+
+
+def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, page_size: int, total_pages: int,
+                 num_slots: int, max_seq_len: int, max_batch: int | None = None) -> list[range]:
+    """Cut the requests, in order, into batches that fit the cache: at most
+    ``num_slots`` (and ``max_batch``) sequences whose pages fit together."""
+    limit = min(num_slots, max_batch) if max_batch else num_slots
+    batches, start, used = [], 0, 0
+    for i, n in enumerate(prompt_lens):
+        if n < 1:
+            raise ShapeError(f"request {i} has an empty prompt")                       # src/bin/runner.rs:235-237
+        if n + max(max_new_tokens, 1) - 1 > max_seq_len:
+            raise CacheError(f"request {i}: {n} prompt tokens and {max_new_tokens} new ones exceed the "
+                             f"{max_seq_len} tokens a sequence may hold")
+        need = pages_for(n, max_new_tokens, page_size)
+        if need > total_pages:
+            raise CacheError(f"request {i} needs {need} pages, the cache has {total_pages}")
+        if i > start and (i - start >= limit or used + need > total_pages):
+            batches.append(range(start, i))
+            start, used = i, 0
+        used += need
+    if start < len(prompt_lens):
+        batches.append(range(start, len(prompt_lens)))
+    return batches
+
+
+class _Live:
+    """One sequence of the running batch."""
+
+    def __init__(self, request: int, slot: int, prompt, sampler: SequenceSampler):
+        self.request, self.slot, self.prompt, self.sampler = request, slot, prompt, sampler
+        self.out: list[int] = []
+        self.generated = 0
+        self.next_token = None
+        self.reason = None
+
+
+def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sampling: SamplingParams,
+              stop: frozenset, ignore_eos: bool, stats: GenerationStats, on_token=None) -> dict:
+    """Serve one batch to the end; returns request -> (tokens, reason)."""
+    cache = engine.cache
+    live = []
+    try:
+        for r in requests:
+            live.append(_Live(r, cache.acquire(), list(prompts[r]), SequenceSampler(sampling, r, prompts[r])))
+    except Exception:
+        for s in live:
+            cache.release(s.slot)
+        raise
+    done = {}
+    held = {s.slot for s in live}
+    try:
+        t0 = time.perf_counter()
+        logits = engine.step([StepEntry(s.slot, s.prompt, "last") for s in live])
+        picks = sample_batch(logits, [s.sampler for s in live])
+        stats.prompt_tokens += sum(len(s.prompt) for s in live)
+        stats.prefill_seconds += time.perf_counter() - t0      # includes the first sample, as in the reference
+        for s, tok in zip(live, picks):
+            s.next_token, s.generated = int(tok), 1
+        t0 = time.perf_counter()
+        while live:
+            going = []
+            for s in live:
+                if not ignore_eos and s.next_token in stop:
+                    s.reason = "stop"                           # tested before output; not part of it
+                else:
+                    s.out.append(s.next_token)
+                    if on_token is not None:
+                        on_token(s.request, s.next_token)
+                    if s.generated >= max_new_tokens:
+                        s.reason = "length"                     # put out but never fed
+                if s.reason is None:
+                    going.append(s)
+                else:
+                    done[s.request] = (s.out, s.reason)
+                    cache.release(s.slot)                       # slot and pages go back at once
+                    held.discard(s.slot)
+            live = going
+            if not live:
+                break
+            logits = engine.step([StepEntry(s.slot, [s.next_token], "last") for s in live])
+            for s in live:
+                s.sampler.history.append(s.next_token)
+            picks = sample_batch(logits, [s.sampler for s in live])
+            for s, tok in zip(live, picks):
+                s.next_token = int(tok)
+                s.generated += 1
+            stats.decode_tokens += len(live)
+            stats.decode_steps += 1
+        stats.decode_seconds += time.perf_counter() - t0
+    finally:
+        for slot in held:
+            cache.release(slot)
+    return done
+
+
+def generate(engine, prompts: Sequence[Sequence[int]], max_new_tokens: int = 600,
+             sampling: SamplingParams | None = None, stop_token_ids: Sequence[int] = (), ignore_eos: bool = False,
+             max_batch: int | None = None, on_token=None) -> GenerationResult:
+    """Generate for every prompt; results in the order of the prompts."""
+    sampling = sampling or SamplingParams()
+    if max_new_tokens < 1:
+        raise ShapeError("max_new_tokens must be at least 1")
+    cache = engine.cache
+    total_pages = min((g.pool.num_pages for g in cache.groups), default=1 << 30)
+    batches = plan_batches([len(p) for p in prompts], max_new_tokens, cache.page_size, total_pages,
+                           cache.num_slots, cache.max_seq_len, max_batch)
+    stats = GenerationStats()
+    tokens, reasons = [None] * len(prompts), [None] * len(prompts)
+    stop = frozenset(int(t) for t in stop_token_ids)
+    for batch in batches:
+        done = run_batch(engine, list(batch), prompts, max_new_tokens, sampling, stop, ignore_eos, stats, on_token)
+        stats.batches += 1
+        for r, (out, reason) in done.items():
+            tokens[r], reasons[r] = out, reason
+    return GenerationResult(tokens, reasons, stats)

@@ -1,0 +1,136 @@
+"""Building and loading the HIP kernel library.
+
+The sources under ``csrc/`` are compiled for gfx950 with hipcc into one shared
+library beside this file.  ``load()`` takes the library that is there when it was
+built from the present sources, and builds it otherwise (in the package folder, or
+in a temporary folder when that is not writable), printing a line per file so that
+a first call in a fresh checkout shows that it is alive.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+from ..errors import KernelError
+
+ARCH = "gfx950"
+LIB_NAME = "libri_kernels.so"
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
+
+# -packed-fp32-ops off: packed float32 instructions are not to be generated on this hardware pool
+HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-Wno-unused-command-line-argument",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+_lib = None
+
+
+def _say(msg: str) -> None:
+    print(f"[rust-inference_amd] {msg}", file=sys.stderr, flush=True)
+
+
+def sources() -> list[str]:
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def source_hash() -> str:
+    h = hashlib.sha256()
+    for path in sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".h"))):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def _hipcc() -> str:
+    for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise KernelError("hipcc not found: the HIP kernel library cannot be built")
+
+
+def _is_current(lib_path: str) -> bool:
+    stamp = lib_path + ".hash"
+    if not (os.path.exists(lib_path) and os.path.exists(stamp)):
+        return False
+    with open(stamp) as f:
+        return f.read().strip() == source_hash()
+
+
+def _compile_one(hipcc: str, src: str, obj: str, env: dict) -> None:
+    proc = subprocess.run([hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj], capture_output=True, text=True, env=env)
+    if proc.returncode != 0:
+        raise KernelError(f"hipcc failed on {os.path.basename(src)}:\n{proc.stderr[-4000:]}")
+
+
+def build(out_dir: str | None = None, jobs: int | None = None) -> str:
+    """Compile every source for gfx950 and link the library; returns its path."""
+    hipcc = _hipcc()
+    out_dir = out_dir or _HERE
+    os.makedirs(out_dir, exist_ok=True)
+    lib_path = os.path.join(out_dir, LIB_NAME)
+    srcs = sources()
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())          # hipcc wants a HOME for its caches
+    jobs = jobs or min(8, len(srcs), os.cpu_count() or 1)
+    t0 = time.time()
+    _say(f"building {LIB_NAME} for {ARCH}: {len(srcs)} files, {jobs} at a time")
+    with tempfile.TemporaryDirectory(prefix="ri_build_") as tmp:
+        objs = [os.path.join(tmp, os.path.basename(s) + ".o") for s in srcs]
+        done = 0
+
+        def one(pair):
+            nonlocal done
+            _compile_one(hipcc, pair[0], pair[1], env)
+            done += 1
+            _say(f"  compiled {os.path.basename(pair[0])} ({done}/{len(srcs)}, {time.time() - t0:.0f} s)")
+
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            list(pool.map(one, zip(srcs, objs)))
+        tmp_lib = os.path.join(tmp, LIB_NAME)
+        proc = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp_lib],
+                              capture_output=True, text=True, env=env)
+        if proc.returncode != 0:
+            raise KernelError(f"linking {LIB_NAME} failed:\n{proc.stderr[-4000:]}")
+        shutil.move(tmp_lib, lib_path + ".tmp")
+        os.replace(lib_path + ".tmp", lib_path)
+    with open(lib_path + ".hash", "w") as f:
+        f.write(source_hash())
+    _say(f"built {lib_path} in {time.time() - t0:.0f} s")
+    return lib_path
+
+
+def find_or_build() -> str:
+    in_tree = os.path.join(_HERE, LIB_NAME)
+    if _is_current(in_tree):
+        return in_tree
+    if os.access(_HERE, os.W_OK):
+        return build(_HERE)
+    alt = os.path.join(tempfile.gettempdir(), f"ri_kernels_{os.getuid()}_{source_hash()}")
+    alt_lib = os.path.join(alt, LIB_NAME)
+    if _is_current(alt_lib):
+        return alt_lib
+    return build(alt)
+
+
+def load() -> ctypes.CDLL:
+    """The kernel library, loaded once per process.  Raises KernelError when it
+    cannot be had: there is no other implementation to fall back to."""
+    global _lib
+    if _lib is None:
+        path = find_or_build()
+        try:
+            _lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load {path}: {e}") from None
+        _lib.ri_last_error.restype = ctypes.c_char_p
+        _lib.ri_abi_version.restype = ctypes.c_int
+    return _lib

@@ -1,0 +1,192 @@
+"""Python face of the HIP kernels: one function per kernel.
+
+Each wrapper checks on the host that the operands are what the kernel and its
+grid assume (device, dtype, contiguity, shapes) and then launches on torch's
+current stream.  There is no other implementation behind these functions: without
+the library, or on a tensor that is not on the GPU, they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_void_p
+
+import torch
+
+from ..errors import KernelError, ShapeError
+from .build import load
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+_SIGNATURES = {
+    "ri_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "ri_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p],
+    "ri_add_rows": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "ri_qk_norm_rope_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_void_p],
+    "ri_attention": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+}
+
+_fn = {}
+
+
+def _get(name: str):
+    f = _fn.get(name)
+    if f is None:
+        lib = load()
+        try:
+            f = getattr(lib, name)
+        except AttributeError:
+            raise KernelError(f"the kernel library has no {name}: it is older than this package, build it again") from None
+        f.argtypes = _SIGNATURES[name]
+        f.restype = c_int
+        _fn[name] = f
+    return f
+
+
+def _call(name: str, *args) -> None:
+    rc = _get(name)(*args)
+    if rc != 0:
+        raise KernelError(load().ri_last_error().decode())
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def code(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise ShapeError(f"dtype {dtype} is not float32 or bfloat16") from None
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None, shape=None) -> int:
+    """Checks a tensor and returns its device address."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: the kernels run on the GPU only, got "
+                          f"{t.device if isinstance(t, torch.Tensor) else type(t).__name__}")
+    if not t.is_contiguous():
+        raise ShapeError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise ShapeError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ShapeError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+    return t.data_ptr()
+
+
+def _opt(t, name: str, dtype=None, shape=None):
+    return None if t is None else _dev(t, name, dtype, shape)
+
+
+# ---------------------------------------------------------------- row-wise
+def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """float32 rows ``table[ids]``; ids int32 ``[T]``, already checked to be inside the table."""
+    tokens, dim = ids.shape[0], table.shape[1]
+    out = torch.empty((tokens, dim), dtype=torch.float32, device=table.device)
+    _call("ri_embed_gather", _dev(out, "out"), _dev(table, "table"), code(table.dtype),
+          _dev(ids, "ids", torch.int32, (tokens,)), tokens, dim, _stream())
+    return out
+
+
+def add_rmsnorm(residual: torch.Tensor, pending, gain: torch.Tensor, eps: float, out_dtype,
+                rows: torch.Tensor | None = None) -> torch.Tensor:
+    """``residual += pending`` (in place, when ``rows`` is None) and the RMSNorm of the sum.
+    With ``rows`` the sum and norm are taken of those rows only and nothing is written back."""
+    t, dim = residual.shape
+    n = t if rows is None else rows.shape[0]
+    out = torch.empty((n, dim), dtype=out_dtype, device=residual.device)
+    _call("ri_add_rmsnorm", _dev(out, "out"), code(out_dtype), _dev(residual, "residual", torch.float32),
+          _opt(pending, "pending", None, (t, dim)), code(pending.dtype) if pending is not None else F32,
+          _dev(gain, "gain", torch.float32, (dim,)), float(eps), _opt(rows, "rows", torch.int32), n, dim, _stream())
+    return out
+
+
+def add_rows(residual: torch.Tensor, pending, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """float32 ``residual[rows] + pending[rows]`` without a norm."""
+    t, dim = residual.shape
+    n = t if rows is None else rows.shape[0]
+    out = torch.empty((n, dim), dtype=torch.float32, device=residual.device)
+    _call("ri_add_rows", _dev(out, "out"), _dev(residual, "residual", torch.float32),
+          _opt(pending, "pending", None, (t, dim)), code(pending.dtype) if pending is not None else F32,
+          _opt(rows, "rows", torch.int32), n, dim, _stream())
+    return out
+
+
+def swiglu(y: torch.Tensor) -> torch.Tensor:
+    """``silu(y[:, :I]) * y[:, I:]`` for ``y: [T, 2 I]``."""
+    tokens, two_i = y.shape
+    if two_i % 2:
+        raise ShapeError(f"swiglu input has an odd width {two_i}")
+    out = torch.empty((tokens, two_i // 2), dtype=y.dtype, device=y.device)
+    _call("ri_swiglu", _dev(out, "out"), _dev(y, "y"), code(y.dtype), tokens, two_i // 2, _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """int32 index of the first maximum of every row of float32 ``logits``."""
+    rows, vocab = logits.shape
+    ids = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _call("ri_argmax", _dev(ids, "ids"), _dev(logits, "logits", torch.float32), rows, vocab, _stream())
+    return ids
+
+
+# ---------------------------------------------------------------- attention
+def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, k_pages, v_pages,
+                          heads: int, kv_heads: int, head_dim: int) -> None:
+    """In place on ``qkv: [T, (H + 2 Hkv) dh]``: per-head norm and rotation of q and k; k and v go to their pages."""
+    tokens = qkv.shape[0]
+    width = (heads + 2 * kv_heads) * head_dim
+    num_pages, hkv, page_size, dh = k_pages.shape
+    if (hkv, dh) != (kv_heads, head_dim) or v_pages.shape != k_pages.shape:
+        raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv heads "
+                         f"of {head_dim}")
+    half = head_dim // 2
+    _call("ri_qk_norm_rope_kv_write", _dev(qkv, "qkv", None, (tokens, width)), code(qkv.dtype),
+          _opt(q_gain, "q_gain", torch.float32, (head_dim,)), _opt(k_gain, "k_gain", torch.float32, (head_dim,)),
+          float(eps), _opt(inv_freq, "inv_freq", torch.float32, (half,)), head_dim,
+          _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1],
+          _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), code(k_pages.dtype), tokens, heads, kv_heads, head_dim,
+          page_size, num_pages, _stream())
+
+
+def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, kv_heads: int, head_dim: int,
+              window: int | None, scale: float) -> torch.Tensor:
+    """Attention of every new token over its sequence's pages; q is the first ``H dh`` columns of ``qkv``."""
+    tokens, stride = qkv.shape
+    out = torch.empty((tokens, heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    _call("ri_attention", _dev(out, "out"), _dev(qkv, "qkv"), code(qkv.dtype), stride, _dev(k_pages, "k_pages"),
+          _dev(v_pages, "v_pages"), code(k_pages.dtype), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
+          _dev(tok_seq, "tok_seq", torch.int32, (tokens,)), _dev(page_table, "page_table", torch.int32),
+          page_table.shape[1], tokens, heads, kv_heads, head_dim, k_pages.shape[2], int(window or 0), float(scale),
+          _stream())
+    return out
+
+
+# ---------------------------------------------------------------- products
+def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w.T`` in true 32-bit arithmetic; ``x`` float32 ``[M, K]``, ``w`` float32 or bfloat16 ``[N, K]``."""
+    m, k = x.shape
+    n = w.shape[0]
+    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _call("ri_gemm_f32", _dev(out, "out"), _dev(x, "x", torch.float32), _dev(w, "w", None, (n, k)), code(w.dtype),
+          m, n, k, _stream())
+    return out
+
+
+def gemv_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu: bool = False) -> torch.Tensor:
+    """``x @ w.T`` for up to 8 bfloat16 rows; with ``swiglu`` ``w`` is gate rows then up rows and the
+    result is ``silu(gate) * up``."""
+    m, k = x.shape
+    n = w.shape[0] // 2 if swiglu else w.shape[0]
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _call("ri_gemv_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
+          _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
+    return out

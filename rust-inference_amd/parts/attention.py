@@ -1,0 +1,80 @@
+"""Grouped-query attention over the paged cache."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..cache import KVNeed
+from ..errors import ConfigError
+from ..kernels import ops
+from ..weights.loader import GAIN, MATRIX, TensorSpec
+from .base import Mixer
+from .registry import build_part, register_part
+from .spec import PartSpec
+
+
+@register_part("mixer", "attention")
+class GroupedQueryAttention(Mixer):
+    """q/k/v projections (no bias), optional per-head RMSNorm of q and k with one
+    gain of ``head_dim`` shared by all heads, position encoding of q and k, write of
+    k and v into the sequence's pages, causal attention of every new token over its
+    sequence (all keys, or the last ``window``), output projection
+    (the reference: src/models/qwen3.rs:71-100; src/attention.rs:33-150).
+
+    Query head ``h`` reads kv head ``h // (heads / kv_heads)``; the score is
+    ``(q . k) / sqrt(head_dim)``; softmax statistics and the accumulator are float32.
+    The three projections are one product with the row-concatenated weight
+    ``[q; k; v]``: every output row's dot product is the same as with three products.
+    """
+
+    def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, prefix: str, qk_norm: bool = True,
+                 eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None):
+        if heads < 1 or kv_heads < 1 or heads % kv_heads:
+            raise ConfigError(f"{heads} attention heads not divisible by {kv_heads} kv heads")
+        if head_dim % 16:
+            raise ConfigError(f"head_dim {head_dim}: the attention kernels take multiples of 16")
+        if window is not None and window < 1:
+            raise ConfigError(f"window {window} must be positive")
+        self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
+        self.prefix, self.qk_norm, self.eps, self.window = prefix, qk_norm, eps, window
+        self.scale = 1.0 / math.sqrt(head_dim)                      # src/attention.rs:28
+        self.position = build_part("position", position or PartSpec("none"))
+
+    def tensors(self):
+        p, d, dh = self.prefix, self.hidden, self.head_dim
+        t = {
+            p + "q_proj.weight": TensorSpec((self.heads * dh, d), MATRIX),
+            p + "k_proj.weight": TensorSpec((self.kv_heads * dh, d), MATRIX),
+            p + "v_proj.weight": TensorSpec((self.kv_heads * dh, d), MATRIX),
+            p + "o_proj.weight": TensorSpec((d, self.heads * dh), MATRIX),
+        }
+        if self.qk_norm:
+            t[p + "q_norm.weight"] = TensorSpec((dh,), GAIN)
+            t[p + "k_norm.weight"] = TensorSpec((dh,), GAIN)
+        t.update(self.position.tensors())
+        return t
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        p = self.prefix
+        qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
+        self.w_qkv = rt.place_matrix(qkv)
+        self.w_o = rt.place_matrix(weights[p + "o_proj.weight"])
+        self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
+        self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
+        self.position.bind(weights, rt)
+
+    def cache_need(self):
+        return KVNeed(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, ctx, store, page_table):
+        rt = self.rt
+        qkv = rt.linear(x, self.w_qkv)
+        self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
+        ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
+                                  ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
+                                  self.heads, self.kv_heads, self.head_dim)
+        o = ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table,
+                          self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
+        return rt.linear(o, self.w_o)

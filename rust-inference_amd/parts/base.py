@@ -1,0 +1,69 @@
+"""Interfaces of the parts.
+
+Every part: is built from the parameters of its ``PartSpec``; says which tensors
+it wants (``tensors()``: checkpoint name -> ``TensorSpec``); takes them over
+(``bind(weights, runtime)``); and runs on the flattened tokens of a step.  No part
+knows which model it is in.
+"""
+from __future__ import annotations
+
+from ..weights.loader import TensorSpec
+
+
+class Part:
+    def tensors(self) -> dict[str, TensorSpec]:
+        """Checkpoint names and shapes of this part's weights."""
+        return {}
+
+    def bind(self, weights: dict, rt) -> None:
+        """Take the weights (host tensors, as stored) and put what is needed on the device."""
+        self.rt = rt
+
+
+class Norm(Part):
+    """``apply(residual, pending, out_dtype, rows=None)``: adds ``pending`` into the
+    float32 residual stream (in place when ``rows`` is None) and returns the norm of
+    the sum in ``out_dtype``; with ``rows`` only those rows, nothing written back."""
+
+    def apply(self, residual, pending, out_dtype, rows=None):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a sequence.
+
+    ``cache_need()`` says what one cache entry of this mixer holds (a ``KVNeed``, a
+    ``StateNeed`` or None).  ``forward(x, ctx, store, page_table)`` gets the normed
+    tokens ``[T, hidden]``, the step's context, its cache entry's storage (a
+    ``KVView`` or the state arena ``[slots, ...]``) and, for key/value needs, the
+    step's page table of its group; it returns ``[T, hidden]``.  Tokens of a
+    sequence are contiguous and in order (``ctx.cu_seqlens``); a mixer with state
+    reads its slot's row, consumes the sequence's tokens in order and writes the
+    row back.
+    """
+
+    def cache_need(self):
+        return None
+
+    def forward(self, x, ctx, store, page_table):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Token-wise ``[T, hidden] -> [T, hidden]``."""
+
+    def forward(self, x, ctx):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How positions enter a mixer.  ``rotation_table()`` returns the float32 inverse
+    frequencies ``[head_dim / 2]`` for the fused rotate-half kernel, or None when
+    this encoding does not rotate; ``apply(qkv, ctx, heads, kv_heads, head_dim)`` may
+    change q and k in place before the fused kernel for encodings of another kind."""
+
+    def rotation_table(self):
+        return None
+
+    def apply(self, qkv, ctx, heads, kv_heads, head_dim):
+        return None

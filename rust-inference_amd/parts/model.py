@@ -1,0 +1,174 @@
+"""The generic decoder: embedding, layers in schedule order, final norm, output matrix.
+
+Built from a ``ModelSpec``; which parts the layers have is the spec's business.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache import Cache, KVNeed
+from ..config import load_config
+from ..errors import ConfigError, ShapeError
+from ..kernels import ops
+from ..weights.loader import MATRIX, TensorSpec, load_checked
+from ..weights.random_init import random_tensors
+from .base import Part
+from .block import ResidualStream
+from .registry import build_part, part_class, register_part
+from .runtime import Runtime
+from .spec import ModelSpec
+
+
+@register_part("embedding", "table")
+class TokenEmbedding(Part):
+    """``h[t, :] = E[id_t, :]`` without scaling (the reference: src/ops/embedding.rs:10-42)."""
+
+    def __init__(self, vocab: int, dim: int, name: str):
+        self.vocab, self.dim, self.name = vocab, dim, name
+
+    def tensors(self):
+        return {self.name: TensorSpec((self.vocab, self.dim), MATRIX)}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.table = rt.place_matrix(weights[self.name])
+
+    def forward(self, ids):
+        return ops.embed_gather(self.table, ids)
+
+
+@register_part("head", "linear")
+class OutputHead(Part):
+    """``logits = x W^T`` in float32, no scaling or cap.  The matrix is the embedding
+    table when the configuration ties them or the checkpoint has no tensor of this
+    name (the reference: src/models/qwen3.rs:167-171, :286)."""
+
+    def __init__(self, vocab: int, dim: int, name: str, tied: bool):
+        self.vocab, self.dim, self.name, self.tied = vocab, dim, name, tied
+
+    def tensors(self):
+        return {self.name: TensorSpec((self.vocab, self.dim), MATRIX, optional=True)}
+
+    def written_when_random(self) -> bool:
+        return not self.tied
+
+    def bind(self, weights, rt, embedding: TokenEmbedding | None = None):
+        self.rt = rt
+        if self.tied or self.name not in weights:
+            if embedding is None:
+                raise ConfigError(f"{self.name} is absent and there is no embedding to tie it to")
+            self.weight = embedding.table           # the same device tensor: tying costs no memory
+        else:
+            self.weight = rt.place_matrix(weights[self.name])
+
+    def forward(self, x):
+        return self.rt.linear(x, self.weight, out_dtype=torch.float32)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = build_part("embedding", spec.embedding)
+        self.layers = [part_class("arrangement", ls.arrangement)(ls) for ls in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm)
+        self.head = build_part("head", spec.head)
+        self.schedule = list(spec.schedule)
+        for r in self.schedule:
+            if not 0 <= r.layer < len(self.layers):
+                raise ConfigError(f"schedule names layer {r.layer}, the model has {len(self.layers)}")
+        self.rt = None
+
+    # ---- weights
+    def parts(self):
+        yield self.embedding
+        for layer in self.layers:
+            yield from layer.parts()
+        yield self.final_norm
+        yield self.head
+
+    def tensors(self, for_writing: bool = False) -> dict[str, TensorSpec]:
+        out = {}
+        for part in self.parts():
+            if for_writing and part is self.head and not self.head.written_when_random():
+                continue
+            for name, spec in part.tensors().items():
+                if name in out and out[name].shape != spec.shape:
+                    raise ConfigError(f"tensor {name} is wanted with shapes {out[name].shape} and {spec.shape}")
+                out[name] = spec
+        return out
+
+    def bind(self, weights: dict, rt: Runtime) -> "DecoderModel":
+        self.rt = rt
+        self.embedding.bind(weights, rt)
+        for layer in self.layers:
+            for part in layer.parts():
+                part.bind(weights, rt)
+        self.final_norm.bind(weights, rt)
+        self.head.bind(weights, rt, self.embedding)
+        return self
+
+    # ---- cache
+    def cache_needs(self) -> list:
+        """The need of every cache entry the schedule names."""
+        needs = [None] * self.spec.num_cache_entries
+        for r in self.schedule:
+            if r.cache is None:
+                continue
+            need = self.layers[r.layer].mixer.cache_need()
+            if needs[r.cache] is not None and needs[r.cache] != need:
+                raise ConfigError(f"cache entry {r.cache} is used with two different needs")
+            needs[r.cache] = need
+        return needs
+
+    def new_cache(self, max_tokens: int, num_slots: int, max_seq_len: int | None = None, **kw) -> Cache:
+        max_seq_len = min(max_seq_len or self.spec.max_positions, self.spec.max_positions)
+        return Cache(self.cache_needs(), num_slots, max_tokens, max_seq_len, dtype=self.rt.dtype,
+                     device=self.rt.device, **kw)
+
+    # ---- one step
+    def forward(self, ctx, cache: Cache) -> torch.Tensor:
+        """float32 logits ``[n_want, vocab]`` for the wanted rows of this step's tokens."""
+        rt = self.rt
+        stream = ResidualStream(self.embedding.forward(ctx.tokens))
+        for run in self.schedule:
+            layer = self.layers[run.layer]
+            store, table = None, None
+            if run.cache is not None:
+                need = cache.needs[run.cache]
+                if isinstance(need, KVNeed):
+                    store = cache.kv(run.cache)
+                    table = ctx.page_tables[store.group_index]
+                elif need is not None:
+                    store = cache.state(run.cache)
+            layer.forward(stream, ctx, store, table, rt.dtype)
+        if ctx.n_want == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=rt.device)
+        h = stream.normed(self.final_norm, rt.dtype, rows=ctx.want_rows)      # only the wanted rows
+        logits = self.head.forward(h)
+        if logits.shape != (ctx.n_want, self.spec.vocab_size):
+            raise ShapeError(f"logits are {list(logits.shape)}")
+        return logits
+
+
+def expected_tensors(spec: ModelSpec, for_writing: bool = False) -> dict[str, TensorSpec]:
+    return DecoderModel(spec).tensors(for_writing)
+
+
+def load_model(model_dir: str, dtype=torch.bfloat16, device="cuda:0") -> DecoderModel:
+    """The model of a folder: the class by config.json, the weights by name."""
+    arch, cfg = load_config(model_dir)
+    model = DecoderModel(arch.build_spec(cfg))
+    model.config = cfg
+    weights = load_checked(model_dir, model.tensors())
+    return model.bind(weights, Runtime(device, dtype))
+
+
+def random_model(config, seed: int, dtype=torch.bfloat16, device="cuda:0", store_dtype=torch.bfloat16) -> DecoderModel:
+    """A model with random weights made in memory, for sizes one would not write to disk."""
+    from ..config import config_from_dict
+    arch, cfg = config_from_dict(config if isinstance(config, dict) else config.to_dict())
+    model = DecoderModel(arch.build_spec(cfg))
+    model.config = cfg
+    rt = Runtime(device, dtype)
+    weights = random_tensors(model.tensors(for_writing=True), seed, store_dtype, device=rt.device)
+    return model.bind(weights, rt)

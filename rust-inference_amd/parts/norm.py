@@ -1,0 +1,26 @@
+"""RMSNorm, fused with the residual add that precedes it."""
+from __future__ import annotations
+
+from ..kernels import ops
+from ..weights.loader import GAIN, TensorSpec
+from .base import Norm
+from .registry import register_part
+
+
+@register_part("norm", "rmsnorm")
+class RMSNorm(Norm):
+    """``y = x * (1 / sqrt(mean(x^2) + eps)) * w`` over the last axis, statistics in
+    float32 (the reference: src/ops/norm.rs:7-32; fused with the add: :35-62)."""
+
+    def __init__(self, dim: int, eps: float, name: str):
+        self.dim, self.eps, self.name = dim, eps, name
+
+    def tensors(self):
+        return {self.name: TensorSpec((self.dim,), GAIN)}
+
+    def bind(self, weights, rt):
+        self.rt = rt
+        self.gain = rt.place_gain(weights[self.name])
+
+    def apply(self, residual, pending, out_dtype, rows=None):
+        return ops.add_rmsnorm(residual, pending, self.gain, self.eps, out_dtype, rows)

@@ -1,0 +1,52 @@
+"""Shared test set-up: the `gpu` marker, the two tiny configurations, model folders in temporary places."""
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.dirname(os.path.abspath(__file__))):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+# Two tiny configurations of the architecture that differ in every size and option.
+TINY_A = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "vocab_size": 256, "hidden_size": 64, "intermediate_size": 128, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16,
+    "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 128,
+}
+TINY_B = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "vocab_size": 320, "hidden_size": 96, "intermediate_size": 160, "num_hidden_layers": 3,
+    "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 32,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "max_position_embeddings": 256,
+}
+# A third one for long contexts and odd sizes: width and vocabulary that are no power of two,
+# three query heads per kv head, head_dim 48.
+TINY_C = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "vocab_size": 411, "hidden_size": 104, "intermediate_size": 232, "num_hidden_layers": 2,
+    "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 48,
+    "rope_theta": 50000.0, "rms_norm_eps": 3e-6, "tie_word_embeddings": False, "max_position_embeddings": 1024,
+}
+
+
+@pytest.fixture(scope="session")
+def model_dirs(tmp_path_factory):
+    """Model folders with random weights for the tiny configurations, made once per session.
+    A is stored in float32, B and C in bfloat16.  Weights are larger than the benchmark's
+    N(0, 0.02) so that logits are of order one and differences show."""
+    import torch
+    from rust_inference_amd.weights import write_random_model
+    base = tmp_path_factory.mktemp("models")
+    out = {}
+    for name, cfg, seed, dtype in (("A", TINY_A, 0, torch.float32), ("B", TINY_B, 1, torch.bfloat16),
+                                   ("C", TINY_C, 2, torch.bfloat16)):
+        out[name] = write_random_model(str(base / name), cfg, seed, dtype, matrix_std=0.12, gain_std=0.1)
+    return out

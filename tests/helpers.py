@@ -1,0 +1,40 @@
+"""Helpers shared by the tests: reading a model folder for the plain implementation, comparing logits."""
+import json
+import os
+
+import numpy as np
+
+
+def read_model_f64(model_dir):
+    """(config dict, {name: float64 array}) of a model folder, read with the safetensors package,
+    not with the library under test."""
+    from safetensors import safe_open
+    import torch
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    w = {}
+    with safe_open(os.path.join(model_dir, "model.safetensors"), framework="pt") as f:
+        for name in f.keys():
+            w[name] = f.get_tensor(name).to(torch.float64).numpy()
+    return cfg, w
+
+
+def rel_to_max(got, want):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, f"shape {got.shape} against {want.shape}"
+    scale = np.abs(want).max()
+    return np.abs(got - want).max() / (scale if scale > 0 else 1.0)
+
+
+# Bounds, stated once.  float32: the reference's own end-to-end bound is 2e-4 of the largest logit
+# (tests/model_parity.rs:23-28); this build's target is 1e-4.  bfloat16: activations are rounded to
+# 8 bits of mantissa after every product, the reference allows 1e-2 to 3e-2 of the largest value per
+# op (tests/cuda_parity.rs:43-127); whole-model logits get 3e-2.
+F32_BOUND = 1e-4
+BF16_BOUND = 3e-2
+
+
+def assert_logits_close(got, want, dtype_name, what=""):
+    bound = F32_BOUND if dtype_name == "float32" else BF16_BOUND
+    err = rel_to_max(got, want)
+    assert err <= bound, f"{what}: error {err:.3e} of the largest logit exceeds {bound:.0e} ({dtype_name})"

@@ -1,0 +1,150 @@
+"""The generation loop's decisions with a scripted step function (no GPU, no model)."""
+import pytest
+import torch
+
+from rust_inference_amd.cache import Cache, KVNeed
+from rust_inference_amd.engine import generate, plan_batches, plan_step, StepEntry, wanted_indices
+from rust_inference_amd.errors import CacheError, ShapeError
+from rust_inference_amd.sampling import SamplingParams
+
+VOCAB = 50
+
+
+class ScriptedEngine:
+    """Stands in for the engine: the next token of a sequence is a function of its last token and length,
+    so the expected output of every request is known whatever batch it is in."""
+
+    def __init__(self, slots=4, max_tokens=1024, max_seq_len=256):
+        self.cache = Cache([KVNeed(1, 16)], slots, max_tokens, max_seq_len, dtype=torch.float32, device="cpu",
+                           allocate=False)
+        self.steps = []                       # (slots, counts) of every step
+
+    @staticmethod
+    def rule(last_token, length):
+        return (3 * last_token + length) % VOCAB
+
+    def step(self, entries):
+        slots = [e.slot for e in entries]
+        counts = [len(e.tokens) for e in entries]
+        self.cache.reserve(slots, counts)
+        self.cache.commit(slots, counts)
+        self.steps.append((slots, counts))
+        logits = torch.zeros(len(entries), VOCAB)
+        for i, e in enumerate(entries):
+            assert e.want == "last"
+            logits[i, self.rule(e.tokens[-1], self.cache.length(e.slot))] = 5.0
+        return logits
+
+
+def expected(prompt, n, stop=()):
+    out, last, length = [], prompt[-1], len(prompt)
+    for _ in range(n):
+        nxt = ScriptedEngine.rule(last, length)
+        if nxt in stop:
+            return out, "stop"
+        out.append(nxt)
+        last, length = nxt, length + 1
+    return out, "length"
+
+
+def test_unequal_prompts_in_one_batch_match_each_alone():
+    eng = ScriptedEngine()
+    prompts = [[1, 2, 3, 4, 5], list(range(11)), [7], list(range(17))]
+    res = generate(eng, prompts, max_new_tokens=8)
+    for p, toks, why in zip(prompts, res.tokens, res.finish_reasons):
+        assert (toks, why) == expected(p, 8)
+    assert eng.steps[0] == ([0, 1, 2, 3], [5, 11, 1, 17])           # all prompts in one step
+    assert all(c == [1, 1, 1, 1] for _, c in eng.steps[1:]) and len(eng.steps) == 8   # the 8th token is not fed
+    assert res.stats.prompt_tokens == 34 and res.stats.decode_tokens == 4 * 7 and res.stats.decode_steps == 7
+    eng.cache.check_consistent()
+    assert eng.cache.slots.free_count == 4 and eng.cache.free_pages() == [32]
+
+
+def test_first_token_counts_and_one_token_needs_no_decode_step():
+    eng = ScriptedEngine()
+    res = generate(eng, [[4, 5, 6]], max_new_tokens=1)
+    assert res.tokens == [expected([4, 5, 6], 1)[0]] and res.finish_reasons == ["length"] and len(eng.steps) == 1
+    with pytest.raises(ShapeError):
+        generate(eng, [[1]], max_new_tokens=0)
+    with pytest.raises(ShapeError, match="empty prompt"):
+        generate(eng, [[1], []], max_new_tokens=2)
+
+
+def test_stop_token_ends_a_sequence_early_and_is_not_output():
+    prompts = [[1, 2, 3], [9, 9], [5]]
+    full = [expected(p, 10)[0] for p in prompts]
+    stop = {full[1][3]}                                            # the fourth token of request 1
+    eng = ScriptedEngine()
+    res = generate(eng, prompts, max_new_tokens=10, stop_token_ids=stop)
+    for p, toks, why in zip(prompts, res.tokens, res.finish_reasons):
+        assert (toks, why) == expected(p, 10, stop)
+    assert res.finish_reasons[1] == "stop" and len(res.tokens[1]) <= 3 and next(iter(stop)) not in res.tokens[1]
+    # after request 1 has ended, the steps carry the others only, and its slot went back at once
+    sizes = [len(s) for s, _ in eng.steps]
+    assert sizes[0] == 3 and sizes[-1] == 2 and sizes == sorted(sizes, reverse=True)
+    assert all(1 not in s for s, _ in eng.steps[len(res.tokens[1]) + 1:])
+    res2 = generate(ScriptedEngine(), prompts, max_new_tokens=10, stop_token_ids=stop, ignore_eos=True)
+    assert res2.tokens == full and res2.finish_reasons == ["length"] * 3
+
+
+def test_stop_token_as_the_very_first_token():
+    p = [3, 4]
+    first = expected(p, 1)[0][0]
+    res = generate(ScriptedEngine(), [p, [8]], max_new_tokens=5, stop_token_ids=[first])
+    assert res.tokens[0] == [] and res.finish_reasons[0] == "stop"
+    assert (res.tokens[1], res.finish_reasons[1]) == expected([8], 5, {first})
+
+
+def test_more_requests_than_slots_run_as_batches_one_after_another():
+    eng = ScriptedEngine(slots=2)
+    prompts = [[i + 1] * (i + 1) for i in range(5)]
+    res = generate(eng, prompts, max_new_tokens=4)
+    assert [t for t in res.tokens] == [expected(p, 4)[0] for p in prompts]
+    assert res.stats.batches == 3
+    assert eng.steps[0] == ([0, 1], [1, 2]) and eng.steps[4] == ([0, 1], [3, 4]) and eng.steps[8] == ([0], [5])
+    # slots are used again by the later batches
+    assert {s for sl, _ in eng.steps for s in sl} == {0, 1}
+    eng.cache.check_consistent()
+    assert eng.cache.slots.free_count == 2
+
+
+def test_batches_are_cut_to_fit_the_pages():
+    # pages of 32: each request of 40 + 30 - 1 = 69 tokens needs 3 pages; 7 pages hold two of them
+    assert plan_batches([40, 40, 40], 30, 32, 7, 8, 256) == [range(0, 2), range(2, 3)]
+    assert plan_batches([40, 40, 40], 30, 32, 9, 8, 256, max_batch=2) == [range(0, 2), range(2, 3)]
+    assert plan_batches([1], 1, 32, 1, 1, 32) == [range(0, 1)]
+    with pytest.raises(CacheError, match="needs 3 pages"):
+        plan_batches([40], 30, 32, 2, 8, 256)
+    with pytest.raises(CacheError, match="may hold"):
+        plan_batches([250], 30, 32, 64, 8, 256)
+    eng = ScriptedEngine(slots=8, max_tokens=7 * 32)
+    res = generate(eng, [[1] * 40, [2] * 40, [3] * 40], max_new_tokens=30)
+    assert res.stats.batches == 2 and all(len(t) == 30 for t in res.tokens)
+
+
+def test_temperature_sampling_is_per_sequence_and_seeded():
+    class Flat(ScriptedEngine):
+        def step(self, entries):
+            super().step(entries)
+            return torch.zeros(len(entries), VOCAB)            # uniform: the draw decides alone
+    prompts = [[1], [2], [3]]
+    p = SamplingParams(temperature=1.0, seed=11)
+    a = generate(Flat(), prompts, 6, p).tokens
+    b = generate(Flat(), prompts, 6, p).tokens
+    alone = generate(Flat(), prompts[:1], 6, p).tokens
+    other = generate(Flat(), prompts, 6, SamplingParams(temperature=1.0, seed=12)).tokens
+    assert a == b and a[0] == alone[0] and a != other and a[0] != a[1]
+
+
+def test_plan_step_layout():
+    entries = [StepEntry(3, [5, 6, 7], [0, 2]), StepEntry(0, [9], "last"), StepEntry(1, [1, 2], "none")]
+    tokens, seq, pos, cu, want = plan_step(entries, [10, 0, 4], VOCAB)
+    assert tokens == [5, 6, 7, 9, 1, 2] and seq == [0, 0, 0, 1, 2, 2] and pos == [10, 11, 12, 0, 4, 5]
+    assert cu == [0, 3, 4, 6] and want == [0, 2, 3]
+    assert wanted_indices(4, "all") == [0, 1, 2, 3]
+    with pytest.raises(ShapeError, match="outside the vocabulary"):
+        plan_step([StepEntry(0, [VOCAB])], [0], VOCAB)
+    with pytest.raises(ShapeError, match="outside the entry"):
+        plan_step([StepEntry(0, [1], [1])], [0], VOCAB)
+    with pytest.raises(ShapeError, match="no token"):
+        plan_step([StepEntry(0, [])], [0], VOCAB)

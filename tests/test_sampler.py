@@ -1,0 +1,72 @@
+"""The host sampler against the reference's vectors and against the plain sampler (no GPU)."""
+import numpy as np
+import pytest
+
+from plain.sampler_plain import PlainRng, PlainSampler, candidates
+from rust_inference_amd.sampling import HostSampler, SamplingParams, Xorshift64Star
+from rust_inference_amd.sampling.host import kept_candidates
+
+
+def test_generator_matches_the_plain_one_and_is_in_range():
+    for seed in (0, 1, 7, 0x5EED, 2 ** 63 + 5):
+        a, b = Xorshift64Star(seed), PlainRng(seed)
+        xs = [a.next_u64() for _ in range(50)]
+        assert xs == [b.next_u64() for _ in range(50)]
+    g = Xorshift64Star(3)
+    fs = [g.next_f32() for _ in range(2000)]
+    assert all(0.0 <= f < 1.0 for f in fs) and 0.45 < np.mean(fs) < 0.55
+    assert all(f == float(np.float32(f)) for f in fs)          # 24 bits: exact in float32
+
+
+def test_vectors_of_the_reference():
+    # src/sampling.rs:145-187
+    assert HostSampler(SamplingParams()).sample([0.1, 3.0, 2.0]) == 1
+    assert HostSampler(SamplingParams(repetition_penalty=2.0)).sample([0.1, 3.0, 2.0], [1]) == 2
+    s = HostSampler(SamplingParams(temperature=1.0, top_k=1))
+    assert all(s.sample([0.5, 0.4, 0.6, 0.1]) == 2 for _ in range(20))
+    params = SamplingParams(temperature=1.0, seed=7)
+    s = HostSampler(params)
+    picks = [s.sample([0.0, np.log(3.0)]) for _ in range(4000)]
+    assert abs(np.mean(picks) - 0.75) < 0.03
+    s2 = HostSampler(params)
+    assert picks == [s2.sample([0.0, np.log(3.0)]) for _ in range(4000)]
+    s = HostSampler(SamplingParams(temperature=1.0, top_p=0.5))
+    assert all(s.sample([3.0, 1.0, 0.5, 0.0]) == 0 for _ in range(50))
+
+
+def test_ties_go_to_the_lower_index():
+    assert HostSampler(SamplingParams()).sample([1.0, 3.0, 3.0]) == 1
+    order, _ = kept_candidates(np.array([1.0, 2.0, 2.0, 2.0], dtype=np.float32), SamplingParams(temperature=1.0, top_k=2))
+    assert list(order) == [1, 2]
+
+
+def test_penalty_divides_positive_and_multiplies_negative_logits_once():
+    from rust_inference_amd.sampling.host import apply_repetition_penalty
+    row = np.array([2.0, -2.0, 4.0, 0.0], dtype=np.float32)
+    out = apply_repetition_penalty(row, [0, 1, 1, 0, 99], 2.0)
+    assert list(out) == [1.0, -4.0, 4.0, 0.0] and list(row) == [2.0, -2.0, 4.0, 0.0]
+
+
+@pytest.mark.parametrize("params", [
+    dict(temperature=0.8, seed=1), dict(temperature=1.3, top_k=5, seed=2), dict(temperature=0.7, top_p=0.8, seed=3),
+    dict(temperature=1.0, top_k=12, top_p=0.6, repetition_penalty=1.3, seed=4), dict(repetition_penalty=1.7),
+])
+def test_same_tokens_as_the_plain_sampler(params):
+    rng = np.random.default_rng(5)
+    ours, plain = HostSampler(SamplingParams(**params)), PlainSampler(**params)
+    history = [3, 9, 9, 40]
+    for _ in range(60):
+        logits = (2.5 * rng.normal(size=97)).astype(np.float32)
+        logits[10] = logits[20]                                     # a tie in the row
+        a, b = ours.sample(logits, history), plain.sample(logits, history)
+        assert a == b
+        history.append(a)
+
+
+def test_kept_probabilities_match_the_plain_ones():
+    rng = np.random.default_rng(6)
+    logits = rng.normal(size=200).astype(np.float32) * 3
+    for k, p in ((0, 1.0), (10, 1.0), (0, 0.9), (50, 0.5)):
+        o1, p1 = kept_candidates(logits, SamplingParams(temperature=0.9, top_k=k, top_p=p))
+        o2, p2 = candidates(logits, 0.9, k, p)
+        assert list(o1) == list(o2) and np.allclose(p1, p2, rtol=1e-5, atol=1e-7)
