@@ -101,7 +101,7 @@ def test_more_requests_than_slots_run_as_batches_one_after_another():
     res = generate(eng, prompts, max_new_tokens=4)
     assert [t for t in res.tokens] == [expected(p, 4)[0] for p in prompts]
     assert res.stats.batches == 3
-    assert eng.steps[0] == ([0, 1], [1, 2]) and eng.steps[4] == ([0, 1], [3, 4]) and eng.steps[8] == ([0], [5])
+    assert [eng.steps[i][1] for i in (0, 4, 8)] == [[1, 2], [3, 4], [5]]     # a prompt step opens every batch
     # slots are used again by the later batches
     assert {s for sl, _ in eng.steps for s in sl} == {0, 1}
     eng.cache.check_consistent()
