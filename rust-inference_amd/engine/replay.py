@@ -21,44 +21,61 @@ from ..parts import load_model
 from .step import Engine, StepEntry
 
 
+class Replayer:
+    """Feeds trace steps to an engine, keeping the map from request ids to cache slots."""
+
+    def __init__(self, engine: Engine):
+        self.engine = engine
+        self.slot_of: dict[str, int] = {}
+
+    def feed(self, msg: dict):
+        """Run one step; returns the float32 logits ``[wanted, vocab]`` on the device, or None
+        when the step wants nothing."""
+        cache = self.engine.cache
+        entries = []
+        for e in msg.get("entries", []):
+            rid = str(e["id"])
+            if rid not in self.slot_of:
+                self.slot_of[rid] = cache.acquire()
+            entries.append(StepEntry(self.slot_of[rid], e["tokens"], list(e.get("want", []))))
+        logits = self.engine.step(entries) if entries else None
+        for rid in msg.get("end", []):
+            rid = str(rid)
+            if rid not in self.slot_of:
+                raise InferenceError(f"step {msg.get('step')} ends request {rid!r}, which never started")
+            cache.release(self.slot_of.pop(rid))
+        return logits if logits is not None and logits.shape[0] > 0 else None
+
+
+def engine_for_trace(model, max_tokens: int) -> Engine:
+    """An engine whose cache holds ``max_tokens`` tokens of live requests, each request's count
+    rounded up to a multiple of 64 by the caller (two pages of 32)."""
+    page = 32
+    max_tokens = max(max_tokens, page)
+    cache = model.new_cache(max_tokens=max_tokens, num_slots=max(1, -(-max_tokens // 64)),
+                            max_seq_len=min(max_tokens, model.spec.max_positions))
+    return Engine(model, cache)
+
+
 def run(model_dir: str, dtype: torch.dtype, out_dir: str, max_tokens: int, lines=None, device="cuda:0",
         reply=None) -> int:
     lines = sys.stdin if lines is None else lines
     reply = reply or (lambda s: print(s, flush=True))
     os.makedirs(out_dir, exist_ok=True)
-    model = load_model(model_dir, dtype, device)
-    page = 32
-    # a request's count is rounded up to 64 by the caller: pages of 32 tokens fit inside that
-    num_slots = max(1, -(-max_tokens // 64))
-    cache = model.new_cache(max_tokens=max(max_tokens, page), num_slots=num_slots,
-                            max_seq_len=min(max(max_tokens, page), model.spec.max_positions))
-    engine = Engine(model, cache)
-    slot_of: dict[str, int] = {}
+    player = Replayer(engine_for_trace(load_model(model_dir, dtype, device), max_tokens))
     for line in lines:
         line = line.strip()
         if not line:
             continue
         msg = json.loads(line)
         step = msg["step"]
-        entries = []
-        for e in msg.get("entries", []):
-            rid = str(e["id"])
-            if rid not in slot_of:
-                slot_of[rid] = cache.acquire()
-            entries.append(StepEntry(slot_of[rid], e["tokens"], list(e.get("want", []))))
-        if entries:
-            logits = engine.step(entries)
-            if logits.shape[0] > 0:
-                data = logits.detach().to("cpu", torch.float32).contiguous().numpy()
-                tmp = os.path.join(out_dir, f".{step}.f32.tmp")
-                data.astype("<f4").tofile(tmp)
-                os.replace(tmp, os.path.join(out_dir, f"{step}.f32"))
-            else:
-                torch.cuda.synchronize()
-        for rid in msg.get("end", []):
-            rid = str(rid)
-            if rid not in slot_of:
-                raise InferenceError(f"step {step} ends request {rid!r}, which never started")
-            cache.release(slot_of.pop(rid))
+        logits = player.feed(msg)
+        if logits is not None:
+            data = logits.detach().to("cpu", torch.float32).contiguous().numpy()
+            tmp = os.path.join(out_dir, f".{step}.f32.tmp")
+            data.astype("<f4").tofile(tmp)
+            os.replace(tmp, os.path.join(out_dir, f"{step}.f32"))
+        else:
+            torch.cuda.synchronize()
         reply(f"done {step}")
     return 0

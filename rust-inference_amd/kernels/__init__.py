@@ -1,4 +1,4 @@
 from . import ops
-from .build import build, load
+from .build import build as build_library, load as load_library
 
-__all__ = ["ops", "build", "load"]
+__all__ = ["ops", "build_library", "load_library"]

@@ -1,0 +1,217 @@
+"""The engine against the plain implementation on the GPU, in float32 and in bfloat16: each request
+alone and whole; with its last 32 tokens one by one; in batches of unequal lengths whose shorter
+requests end earlier, one batch after another so that slots and pages are used again; long decoding;
+the first tokens of a sequence; and the same through bin/trace_run."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import trace_plans as plans
+from helpers import assert_logits_close, read_model_f64, rel_to_max
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+_plain_cache = {}
+
+
+def plain_logits(model_dir, tokens):
+    key = (model_dir, tuple(tokens))
+    if key not in _plain_cache:
+        cfg, w = read_model_f64(model_dir)
+        _plain_cache[key] = P.forward(cfg, w, list(tokens))
+    return _plain_cache[key]
+
+
+def requests_for(name, cfg, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return {f"{name}{i}": [int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for i, n in enumerate(lengths)}
+
+
+@pytest.fixture(scope="module")
+def loaded(model_dirs):
+    from rust_inference_amd.parts import load_model
+    cache = {}
+
+    def get(name, dtype_name):
+        if (name, dtype_name) not in cache:
+            cache[(name, dtype_name)] = load_model(model_dirs[name], DTYPES[dtype_name])
+        return cache[(name, dtype_name)]
+    return get
+
+
+def replay_in_process(model, steps):
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    engine = engine_for_trace(model, plans.max_live_tokens(steps))
+    player = Replayer(engine)
+    outs = {}
+    for s in steps:
+        logits = player.feed(s)
+        if logits is not None:
+            outs[s["step"]] = logits.cpu().numpy()
+    engine.cache.check_consistent()
+    assert engine.cache.slots.free_count == engine.cache.num_slots, "a request's slot was not given back"
+    assert all(f == g.pool.num_pages for f, g in zip(engine.cache.free_pages(), engine.cache.groups))
+    return plans.collect(steps, lambda i: outs[i], model.spec.vocab_size)
+
+
+def check_against_plain(model_dir, got, requests, dtype_name, what):
+    for rid, toks in requests.items():
+        assert_logits_close(got[rid], plain_logits(model_dir, toks), dtype_name, f"{what}, request {rid}")
+
+
+CASES = [("A", [5, 11, 1, 17], 0), ("B", [33, 2, 40], 1), ("C", [70, 45, 3], 2)]
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, lengths, seed", CASES)
+def test_each_request_alone_and_whole(model_dirs, loaded, name, lengths, seed, dtype_name):
+    cfg, _ = read_model_f64(model_dirs[name])
+    reqs = requests_for(name, cfg, [n + 20 for n in lengths], seed)
+    got = replay_in_process(loaded(name, dtype_name), plans.whole(reqs))
+    check_against_plain(model_dirs[name], got, reqs, dtype_name, "whole")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, lengths, seed", CASES)
+def test_last_32_tokens_one_by_one(model_dirs, loaded, name, lengths, seed, dtype_name):
+    cfg, _ = read_model_f64(model_dirs[name])
+    reqs = requests_for(name, cfg, [n + 40 for n in lengths], seed + 10)      # prefixes 13.., crossing pages
+    model = loaded(name, dtype_name)
+    got = replay_in_process(model, plans.tail_one_by_one(reqs, 32))
+    check_against_plain(model_dirs[name], got, reqs, dtype_name, "last 32 one by one")
+    # decoding against whole prompts, engine against engine: a tighter bound than against the plain one
+    whole = replay_in_process(model, plans.whole(reqs))
+    bound = 2e-5 if dtype_name == "float32" else 2e-2
+    for rid in reqs:
+        err = rel_to_max(got[rid], whole[rid])
+        assert err <= bound, f"{rid}: one by one differs from whole by {err:.2e} of the largest logit"
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, lengths, seed", CASES)
+def test_unequal_batches_one_after_another(model_dirs, loaded, name, lengths, seed, dtype_name):
+    cfg, _ = read_model_f64(model_dirs[name])
+    rng = np.random.default_rng(seed + 20)
+    batches, reqs = [], {}
+    for b in range(3):                                       # three batches on one cache: slots come back
+        batch = {}
+        order = list(rng.permutation(len(lengths)))
+        for i in order:
+            p = lengths[i]
+            total = p + int(rng.integers(0, 14))             # unequal ends: some end at once, some late
+            rid = f"{name}{b}_{i}"
+            toks = [int(t) for t in rng.integers(0, cfg["vocab_size"], total)]
+            batch[rid] = (toks, p)
+            reqs[rid] = toks
+        batches.append(batch)
+    got = replay_in_process(loaded(name, dtype_name), plans.unequal_batches(batches))
+    check_against_plain(model_dirs[name], got, reqs, dtype_name, "unequal batches")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_batch_composition_and_padding_change_nothing(model_dirs, loaded, dtype_name):
+    """The same request alone, and as one of a batch of unequal others: equal beyond rounding."""
+    cfg, _ = read_model_f64(model_dirs["B"])
+    reqs = requests_for("B", cfg, [37, 5, 64, 1], 33)
+    model = loaded("B", dtype_name)
+    alone = replay_in_process(model, plans.whole(reqs))
+    together = replay_in_process(model, plans.unequal_batches([{rid: (t, len(t)) for rid, t in reqs.items()}]))
+    bound = 2e-5 if dtype_name == "float32" else 2e-2
+    for rid in reqs:
+        assert rel_to_max(together[rid], alone[rid]) <= bound
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_long_decoding(model_dirs, loaded, dtype_name):
+    """A short prompt and 300 tokens one by one: ten pages, three tiles of keys."""
+    cfg, _ = read_model_f64(model_dirs["C"])
+    reqs = requests_for("C", cfg, [310], 44)
+    got = replay_in_process(loaded("C", dtype_name), plans.tail_one_by_one(reqs, 300))
+    check_against_plain(model_dirs["C"], got, reqs, dtype_name, "long decoding")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(model_dirs, loaded, dtype_name):
+    """Every token from the first one on its own step: position 0 sees one key only."""
+    cfg, _ = read_model_f64(model_dirs["A"])
+    reqs = requests_for("A", cfg, [6, 3], 55)
+    got = replay_in_process(loaded("A", dtype_name), plans.tail_one_by_one(reqs, 32))
+    check_against_plain(model_dirs["A"], got, reqs, dtype_name, "first tokens")
+
+
+def test_a_prompt_in_pieces(model_dirs, loaded):
+    """Several tokens in a later step (a prompt cut in three): the same code as any other cut."""
+    cfg, _ = read_model_f64(model_dirs["B"])
+    toks = requests_for("B", cfg, [75], 66)["B0"]
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:30], "want": list(range(30))}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[30:34], "want": [0, 1, 2, 3]}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": toks[34:], "want": list(range(41))}], "end": ["x"]}]
+    got = replay_in_process(loaded("B", "float32"), steps)
+    assert_logits_close(got["x"], plain_logits(model_dirs["B"], toks), "float32", "prompt in pieces")
+
+
+def test_steps_that_want_nothing_still_fill_the_cache(model_dirs, loaded):
+    cfg, _ = read_model_f64(model_dirs["A"])
+    toks = requests_for("A", cfg, [20], 77)["A0"]
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:19], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[19:], "want": [0]}], "end": ["x"]}]
+    got = replay_in_process(loaded("A", "float32"), steps)
+    assert_logits_close(got["x"], plain_logits(model_dirs["A"], toks)[19:], "float32", "empty want")
+
+
+def test_errors_leave_the_cache_whole(model_dirs, loaded):
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.errors import CacheError, ShapeError
+    model = loaded("A", "float32")
+    engine = Engine(model, model.new_cache(max_tokens=64, num_slots=2, max_seq_len=64))
+    s = engine.cache.acquire()
+    with pytest.raises(ShapeError, match="outside the vocabulary"):
+        engine.step([StepEntry(s, [5, 256])])
+    with pytest.raises(CacheError, match="per sequence"):
+        engine.step([StepEntry(s, [1] * 65)])
+    with pytest.raises(CacheError, match="not held"):
+        engine.step([StepEntry(1, [1])])
+    assert engine.cache.length(s) == 0
+    assert engine.step([StepEntry(s, [1, 2, 3], "all")]).shape == (3, 256)
+
+
+# ---------------------------------------------------------------- through the program
+def run_trace_program(model_dir, dtype_name, steps, out_dir):
+    """Drives bin/trace_run as a user would: one line in, wait for `done <step>`, next line."""
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype_name,
+           "--out", out_dir, "--max-tokens", str(plans.max_live_tokens(steps))]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for s in steps:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {s['step']}", f"after step {s['step']} the program said {line!r}"
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_trace_run_program(model_dirs, tmp_path, dtype_name):
+    cfg, _ = read_model_f64(model_dirs["B"])
+    rng = np.random.default_rng(88)
+    reqs = requests_for("B", cfg, [33, 2, 40, 70], 88)
+    batches = [{rid: (t, max(1, len(t) - int(rng.integers(0, 9)))) for rid, t in list(reqs.items())[:3]},
+               {rid: (t, len(t) - 32) for rid, t in list(reqs.items())[3:]}]
+    steps = plans.unequal_batches(batches)
+    out_dir = str(tmp_path / "out")
+    run_trace_program(model_dirs["B"], dtype_name, steps, out_dir)
+    vocab = cfg["vocab_size"]
+    got = plans.collect(steps, lambda i: np.fromfile(os.path.join(out_dir, f"{i}.f32"), dtype="<f4"), vocab)
+    check_against_plain(model_dirs["B"], got, reqs, dtype_name, "bin/trace_run")
+    assert not os.path.exists(os.path.join(out_dir, f"{len(steps)}.f32"))

@@ -1,0 +1,269 @@
+"""Each HIP kernel alone against its plain reference, at other sizes than the tiny models use.
+Where random inputs would hide a fault, the inputs are made so that it shows."""
+import numpy as np
+import pytest
+import torch
+
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from rust_inference_amd.kernels import ops
+    return ops
+
+
+def t(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+
+
+def f64(x):
+    return x.detach().to("cpu", torch.float64).numpy()
+
+
+def close(got, want, rel, what=""):
+    want = np.asarray(want, dtype=np.float64)
+    err = np.abs(f64(got) - want).max() / max(np.abs(want).max(), 1e-30)
+    assert err <= rel, f"{what}: error {err:.3e} of the largest value exceeds {rel:.0e}"
+
+
+def test_the_extension_is_loaded_from_the_tree(ops):
+    from rust_inference_amd.kernels import load_library
+    lib = load_library()
+    assert lib.ri_abi_version() >= 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding(ops, dtype):
+    rng = np.random.default_rng(0)
+    table = t(rng.normal(size=(1000, 200)), dtype)               # a vocabulary and a width that are no power of two
+    ids = [999, 0, 2, 2, 517]
+    got = ops.embed_gather(table, t(ids, torch.int32))
+    assert got.dtype == torch.float32 and np.array_equal(f64(got), P.embedding(f64(table), ids))
+
+
+@pytest.mark.parametrize("dim", [104, 4096, 5000])
+@pytest.mark.parametrize("pending_dtype", [None, torch.float32, torch.bfloat16])
+def test_add_rmsnorm(ops, dim, pending_dtype):
+    rng = np.random.default_rng(dim)
+    res = t(rng.normal(size=(7, dim)) * 3)
+    pend = None if pending_dtype is None else t(rng.normal(size=(7, dim)), pending_dtype)
+    gain = t(1 + 0.1 * rng.normal(size=dim))
+    total = f64(res) + (0 if pend is None else f64(pend))
+    want = P.rms_norm(total, f64(gain), 1e-5)
+    before = res.clone()
+    out = ops.add_rmsnorm(res, pend, gain, 1e-5, torch.float32)
+    close(out, want, 2e-6, "norm")
+    close(res, total, 1e-7, "residual written back")
+    # rows: the same sums for a few rows, nothing written back
+    res2 = before.clone()
+    rows = t([5, 0, 5], torch.int32)
+    out2 = ops.add_rmsnorm(res2, pend, gain, 1e-5, torch.bfloat16, rows)
+    assert torch.equal(res2, before) and out2.dtype == torch.bfloat16
+    close(out2, P.bf16_round(want[[5, 0, 5]].astype(np.float32)), 5e-3, "gathered rows")
+    close(ops.add_rows(before.clone(), pend, rows), total[[5, 0, 5]], 1e-7, "add_rows")
+
+
+def test_add_rmsnorm_fused_equals_unfused_bit_for_bit(ops):
+    # src/ops/norm.rs:84-98
+    a, r = t([[0.5, -1.0, 2.0, 0.25]]), t([[1.0, 1.0, -1.0, 0.0]])
+    w = t([1.0, 0.5, 2.0, 1.0])
+    res = r.clone()
+    fused = ops.add_rmsnorm(res, a, w, 1e-6, torch.float32)
+    plain_sum = (a + r).contiguous()
+    assert torch.equal(res, plain_sum)
+    assert torch.equal(fused, ops.add_rmsnorm(plain_sum.clone(), None, w, 1e-6, torch.float32))
+
+
+def paged(rng, lens, hkv, dh, page_size=32, dtype=torch.float32, spare=3):
+    """Keys and values of several sequences laid into pages in a shuffled physical order."""
+    pages_per = [-(-n // page_size) for n in lens]
+    num_pages = sum(pages_per) + spare
+    order = list(rng.permutation(num_pages))
+    width = max(pages_per) + 1
+    table = np.full((len(lens), width), -1, dtype=np.int32)
+    k = [rng.normal(size=(n, hkv, dh)) for n in lens]
+    v = [rng.normal(size=(n, hkv, dh)) for n in lens]
+    kp = np.zeros((num_pages, hkv, page_size, dh))
+    vp = np.zeros((num_pages, hkv, page_size, dh))
+    for b, n in enumerate(lens):
+        for lp in range(pages_per[b]):
+            table[b, lp] = order.pop()
+        for pos in range(n):
+            kp[table[b, pos // page_size], :, pos % page_size] = k[b][pos]
+            vp[table[b, pos // page_size], :, pos % page_size] = v[b][pos]
+    return k, v, t(kp, dtype), t(vp, dtype), t(table, torch.int32)
+
+
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("heads, kv_heads, dh", [(6, 2, 48), (4, 4, 128), (9, 1, 16), (2, 1, 256)])
+def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh):
+    rng = np.random.default_rng(heads * dh)
+    lens_before, new = [37, 0, 63], [3, 2, 5]                    # writes cross page boundaries
+    lens = [a + b for a, b in zip(lens_before, new)]
+    _, _, kp, vp, table = paged(rng, lens, kv_heads, dh, dtype=dtype)
+    kp.zero_(); vp.zero_()
+    tokens = sum(new)
+    qkv = rng.normal(size=(tokens, (heads + 2 * kv_heads) * dh)) * 2
+    qkv_t = t(qkv, dtype)
+    qkv = f64(qkv_t)
+    tok_seq = [b for b, n in enumerate(new) for _ in range(n)]
+    tok_pos = [lens_before[b] + i for b, n in enumerate(new) for i in range(n)]
+    qg, kg = 1 + 0.2 * rng.normal(size=dh), 1 + 0.2 * rng.normal(size=dh)
+    theta, eps = 50000.0, 1e-5
+    inv_freq = t(P.rope_inv_freq(dh, theta))
+    ops.qk_norm_rope_kv_write(qkv_t, t(qg), t(kg), eps, inv_freq, t(tok_pos, torch.int32), t(tok_seq, torch.int32),
+                              table, kp, vp, heads, kv_heads, dh)
+    ang = P.rope_angles(tok_pos, dh, theta)
+    q = qkv[:, :heads * dh].reshape(tokens, heads, dh)
+    k = qkv[:, heads * dh:(heads + kv_heads) * dh].reshape(tokens, kv_heads, dh)
+    v = qkv[:, (heads + kv_heads) * dh:].reshape(tokens, kv_heads, dh)
+    q_want = P.apply_rope(P.rms_norm(q, f64(t(qg)), eps), ang)
+    k_want = P.apply_rope(P.rms_norm(k, f64(t(kg)), eps), ang)
+    close(qkv_t[:, :heads * dh].reshape(tokens, heads, dh), q_want, rel, "q in place")
+    tab = table.cpu().numpy()
+    for i in range(tokens):
+        page, off = tab[tok_seq[i], tok_pos[i] // 32], tok_pos[i] % 32
+        close(kp[page, :, off], k_want[i], rel, f"k of token {i}")
+        assert np.array_equal(f64(vp[page, :, off]), v[i]), "v is a copy"
+    # nothing else was written: as many rows are non-zero as tokens
+    assert int((kp.float().abs().sum(-1) > 0).sum()) == tokens * kv_heads
+    # without gains and rotation the kernel only moves k and v
+    qkv2 = t(qkv, dtype)
+    ops.qk_norm_rope_kv_write(qkv2, None, None, eps, None, t(tok_pos, torch.int32), t(tok_seq, torch.int32),
+                              table, kp, vp, heads, kv_heads, dh)
+    assert np.array_equal(f64(qkv2), qkv)
+
+
+def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None, boost=None):
+    k, v, kp, vp, table = paged(rng, lens, kv_heads, dh, dtype=dtype)
+    tokens = sum(new)
+    width = (heads + 2 * kv_heads) * dh
+    qkv = np.zeros((tokens, width))
+    qkv[:, :heads * dh] = rng.normal(size=(tokens, heads * dh))
+    tok_seq = [b for b, n in enumerate(new) for _ in range(n)]
+    tok_pos = [lens[b] - n + i for b, n in enumerate(new) for i in range(n)]
+    if boost is not None:
+        boost(qkv, k, kp, table)
+    qkv_t = t(qkv, dtype)
+    out = ops.attention(qkv_t, kp, vp, t(tok_pos, torch.int32), t(tok_seq, torch.int32), table, heads, kv_heads, dh,
+                        window, 1.0 / np.sqrt(dh))
+    q = f64(qkv_t)[:, :heads * dh].reshape(tokens, heads, dh)
+    want = np.zeros((tokens, heads, dh))
+    i = 0
+    for b, n in enumerate(new):
+        kb = np.stack([f64(kp[table[b, p // 32].item(), :, p % 32]) for p in range(lens[b])])
+        vb = np.stack([f64(vp[table[b, p // 32].item(), :, p % 32]) for p in range(lens[b])])
+        want[i:i + n] = P.attention(q[i:i + n], kb, vb, window=window)
+        i += n
+    return out.reshape(tokens, heads, dh), want
+
+
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("heads, kv_heads, dh", [(4, 2, 16), (6, 2, 48), (8, 1, 128), (3, 3, 64), (9, 1, 32)])
+def test_attention_prompts_pieces_and_single_tokens(ops, dtype, rel, heads, kv_heads, dh):
+    rng = np.random.default_rng(heads + dh)
+    # a whole prompt, a piece of five tokens at the end of 300, one token at 257 (a tile's first key), one at 1
+    out, want = attention_case(ops, rng, [70, 300, 257, 1], [70, 5, 1, 1], heads, kv_heads, dh, dtype)
+    close(out, want, rel, "attention")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
+    """One key far back gets a score that stands out: the output must be its value, wherever it lies."""
+    rng = np.random.default_rng(9)
+    heads, kv_heads, dh = 4, 2, 64
+    for far in (0, 31, 32, 255, 256, 511, 640):
+        def boost(qkv, k, kp, table, far=far):
+            # sequence 0's single query, head 1 (kv head 0): q = 8 * k_far / |k_far| * sqrt(dh)
+            kf = f64(kp[table[0, far // 32].item(), 0, far % 32])
+            qkv[0, dh:2 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        out, want = attention_case(ops, rng, [700], [1], heads, kv_heads, dh, dtype, boost=boost)
+        close(out, want, 3e-6 if dtype == torch.float32 else 1e-2, f"far key {far}")
+        # and the plain result really is that one value (the test is not vacuous)
+        assert np.abs(want[0, 1]).max() > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 32, 33, 100, 256, 300])
+def test_attention_window_edges(ops, dtype, window):
+    rng = np.random.default_rng(window)
+    out, want = attention_case(ops, rng, [290, 40], [34, 40], 4, 2, 32, dtype, window=window)
+    close(out, want, 3e-6 if dtype == torch.float32 else 1e-2, f"window {window}")
+
+
+@pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 9, 130])
+def test_gemm_f32(ops, w_dtype, m):
+    # sizes of the reference's own linear test (src/cpu/linear.rs:634-647): n = 37, k = 70
+    rng = np.random.default_rng(m)
+    x, w = t(rng.normal(size=(m, 70))), t(rng.normal(size=(37, 70)), w_dtype)
+    close(ops.gemm_f32(x, w), f64(x) @ f64(w).T, 2e-6, "gemm_f32")
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch(ops):
+    rng = np.random.default_rng(1)
+    x, w = t(rng.normal(size=(100, 333))), t(rng.normal(size=(129, 333)))
+    whole = ops.gemm_f32(x, w)
+    assert torch.equal(whole[17:18], ops.gemm_f32(x[17:18].contiguous(), w))
+    assert torch.equal(whole[60:], ops.gemm_f32(x[60:].contiguous(), w))
+
+
+def test_gemm_f32_is_true_32_bit(ops):
+    """Values that a reduced-precision matrix mode (tf32, bf16 inputs) would round away."""
+    x = t([[1.0, 2.0 ** -12, 0.0, 0.0]]).repeat(1, 16)
+    w = t([[1.0, 1.0, 0.0, 0.0]]).repeat(1, 16)
+    assert ops.gemm_f32(x, w).item() == 16.0 * (1.0 + 2.0 ** -12)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemv_bf16(ops, m, out_dtype):
+    rng = np.random.default_rng(m)
+    x, w = t(rng.normal(size=(m, 584)), torch.bfloat16), t(rng.normal(size=(37, 584)), torch.bfloat16)
+    want = f64(x) @ f64(w).T
+    close(ops.gemv_bf16(x, w, out_dtype), want, 2e-6 if out_dtype == torch.float32 else 5e-3, "gemv")
+    wgu = t(rng.normal(size=(2 * 45, 584)) * 0.1, torch.bfloat16)
+    y = f64(x) @ f64(wgu).T
+    close(ops.gemv_bf16(x, wgu, out_dtype, swiglu=True), P.silu(y[:, :45]) * y[:, 45:],
+          3e-6 if out_dtype == torch.float32 else 5e-3, "gemv with swiglu")
+    # a row's result does not depend on the other rows
+    if m > 1:
+        assert torch.equal(ops.gemv_bf16(x, w, out_dtype)[m - 1:], ops.gemv_bf16(x[m - 1:].contiguous(), w, out_dtype))
+
+
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 1e-6), (torch.bfloat16, 5e-3)])
+def test_swiglu(ops, dtype, rel):
+    assert f64(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])))[0, 0] == 0.0                 # src/ops/elementwise.rs:59-70
+    close(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])), [[0.0, 6.0 / (1.0 + np.exp(-2.0))]], 1e-6)
+    rng = np.random.default_rng(3)
+    y = t(rng.normal(size=(5, 2 * 333)) * 3, dtype)
+    close(ops.swiglu(y), P.silu(f64(y)[:, :333]) * f64(y)[:, 333:], rel, "swiglu")
+
+
+def test_argmax(ops):
+    assert ops.argmax(t([[1.0, 3.0, 3.0], [-1.0, 0.0, -5.0]])).tolist() == [1, 1]   # src/ops/reduce.rs:75-78
+    rng = np.random.default_rng(4)
+    x = rng.normal(size=(5, 151937)).astype(np.float32)
+    x[1, 70000] = x[1, 150000] = 9.0            # equal maxima far apart: the lower index wins
+    x[2, 151936] = 10.0                         # the last element
+    x[3, 0] = 10.0
+    x[4, :] = -np.inf
+    assert ops.argmax(t(x)).tolist() == [int(np.argmax(x[0])), 70000, 151936, 0, 0]
+
+
+def test_kernels_refuse_what_they_cannot_do(ops):
+    from rust_inference_amd.errors import KernelError, ShapeError
+    with pytest.raises(KernelError, match="GPU only"):
+        ops.swiglu(torch.zeros(2, 4))
+    with pytest.raises(KernelError, match="1 to 8"):
+        ops.gemv_bf16(torch.zeros(9, 16, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError, match="multiple of 16"):
+        ops.attention(torch.zeros(1, 3 * 24, device=DEV), torch.zeros(1, 1, 32, 24, device=DEV),
+                      torch.zeros(1, 1, 32, 24, device=DEV), t([0], torch.int32), t([0], torch.int32),
+                      t([[0]], torch.int32), 1, 1, 24, None, 1.0)
+    with pytest.raises(ShapeError, match="contiguous"):
+        ops.swiglu(torch.zeros(4, 8, device=DEV)[:, ::2])
