@@ -45,9 +45,12 @@ class StateNeed:
 class KVGroup:
     """Storage for all cache entries that share one key/value geometry.
 
-    ``k_pages[e]`` and ``v_pages[e]`` are ``[num_pages, kv_heads, page_size, head_dim]``
-    for entry ``e`` of the group (the reference's layout: src/kvcache.rs:42-50,
-    :145-147); one page number means the same page in every entry.
+    ``k_pages[e]`` is ``[num_pages, kv_heads, page_size, head_dim]`` for entry ``e`` of
+    the group (the reference's layout: src/kvcache.rs:42-50, :145-147).  ``v_pages[e]`` is
+    ``[num_pages, kv_heads, head_dim, page_size]``: values lie transposed inside a page,
+    the page's tokens contiguous for each channel, because that is the operand order
+    the matrix cores want for the product of weights and values.  One page number
+    means the same page in every entry.
     """
 
     def __init__(self, need: KVNeed, entries: list[int], num_pages: int, num_slots: int,
@@ -55,9 +58,10 @@ class KVGroup:
         self.need, self.entries, self.page_size = need, list(entries), page_size
         self.pool = PagePool(num_pages, page_size, num_slots, max_pages_per_slot, need.window)
         self.index_of = {e: i for i, e in enumerate(self.entries)}
-        shape = (len(self.entries), num_pages, need.kv_heads, page_size, need.head_dim)
-        self.k_pages = torch.zeros(shape, dtype=dtype, device=device) if allocate else None
-        self.v_pages = torch.zeros(shape, dtype=dtype, device=device) if allocate else None
+        k_shape = (len(self.entries), num_pages, need.kv_heads, page_size, need.head_dim)
+        v_shape = (len(self.entries), num_pages, need.kv_heads, need.head_dim, page_size)
+        self.k_pages = torch.zeros(k_shape, dtype=dtype, device=device) if allocate else None
+        self.v_pages = torch.zeros(v_shape, dtype=dtype, device=device) if allocate else None
 
     def table_rows(self, slots: Sequence[int], width: int) -> list[list[int]]:
         return [self.pool.tables[s][:width] for s in slots]

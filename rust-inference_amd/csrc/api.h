@@ -29,7 +29,8 @@ int ri_add_rows(float* out, const float* residual, const void* pending, int pend
 // Per-head RMSNorm of q and k (gains may be NULL: no norm), rotate-half position encoding of the first
 // rot_dim elements of each head (inv_freq NULL: none), in place for q, and write of k and v into the pages.
 // qkv: [tokens, (heads + 2 kv_heads) * head_dim] of act_dtype.  tok_pos/tok_seq: int32 [tokens].
-// page_table: int32 [seqs, table_width].  k_pages/v_pages: [pages, kv_heads, page_size, head_dim] of cache_dtype.
+// page_table: int32 [seqs, table_width].  k_pages: [pages, kv_heads, page_size, head_dim], v_pages (transposed
+// inside a page): [pages, kv_heads, head_dim, page_size], both of cache_dtype.
 int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
                              const float* inv_freq, int rot_dim, const int32_t* tok_pos, const int32_t* tok_seq,
                              const int32_t* page_table, int table_width, void* k_pages, void* v_pages,
@@ -43,6 +44,23 @@ int ri_attention(void* out, const void* q, int act_dtype, int q_stride, const vo
                  int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* page_table,
                  int table_width, int tokens, int heads, int kv_heads, int head_dim, int page_size, int window,
                  float scale, void* stream);
+
+// The same attention on the matrix cores, for bfloat16, pages of 32 tokens and head_dim 32, 64 or 128.
+// Prefill form: any number of new tokens per sequence (cu_seqlens: int32 [seqs + 1] over the flat tokens,
+// max_new: the most new tokens of any sequence); at most 64 query heads per kv head.
+int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const void* k_pages, const void* v_pages,
+                              const int32_t* cu_seqlens, const int32_t* tok_pos, const int32_t* page_table,
+                              int table_width, int seqs, int max_new, int heads, int kv_heads, int head_dim,
+                              int page_size, int window, float scale, void* stream);
+
+// Decode form: exactly one new token per sequence; keys in chunks of 256, joined by a second kernel.
+// workspace: float32 [seqs, heads, max_chunks, head_dim + 2]; max_chunks >= ri_attention_decode_chunks(longest
+// sequence after this step); at most 16 query heads per kv head.
+int ri_attention_decode_chunks(int max_len);
+int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride, const void* k_pages,
+                             const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
+                             const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
+                             int kv_heads, int head_dim, int page_size, int window, float scale, void* stream);
 
 // out[M, N] (float32) = x[M, K] (float32) . w[N, K]^T, w float32 or bfloat16; true 32-bit arithmetic.
 int ri_gemm_f32(float* out, const float* x, const void* w, int w_dtype, int m, int n, int k, void* stream);

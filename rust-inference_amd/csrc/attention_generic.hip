@@ -40,7 +40,7 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
                          int heads, int kv_heads, int head_dim, int page_size, int window, float scale) {
     extern __shared__ float qs[];                 // head_dim floats: the query
     __shared__ float ps[ATT_TILE];                // this tile's weights
-    __shared__ long rowoff[ATT_TILE];             // element offset of each key's row in the pools
+    __shared__ long rowoff[ATT_TILE];             // element offset of each key's column in the value pool
     __shared__ float scratch[16];
 
     const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
@@ -58,9 +58,9 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
         const bool valid = j >= lo && j <= qpos;
         float s = -INFINITY;
         if (valid) {
-            const long off = (((long)table[j / page_size] * kv_heads + kvh) * page_size + j % page_size) * head_dim;
-            rowoff[tid] = off;
-            const TC* kr = k_pages + off;
+            const long head_base = ((long)table[j / page_size] * kv_heads + kvh) * page_size * head_dim;
+            rowoff[tid] = head_base + j % page_size;       // the key's column in the transposed value page
+            const TC* kr = k_pages + head_base + (long)(j % page_size) * head_dim;
             float dot = 0.f;
             for (int d = 0; d < head_dim; d += Vec<TC>::N) {
                 float kv[Vec<TC>::N];
@@ -81,7 +81,8 @@ attention_generic_kernel(TA* __restrict__ out, const TA* __restrict__ q, int q_s
             acc *= corr;
             const int first = max(lo, tile * ATT_TILE) - tile * ATT_TILE;
             const int last = min(qpos, tile * ATT_TILE + ATT_TILE - 1) - tile * ATT_TILE;
-            for (int jj = first; jj <= last; ++jj) acc += ps[jj] * to_f32(v_pages[rowoff[jj] + tid]);
+            for (int jj = first; jj <= last; ++jj)
+                acc += ps[jj] * to_f32(v_pages[rowoff[jj] + (long)tid * page_size]);
         }
         __syncthreads();                                   // before the next tile overwrites ps and rowoff
     }

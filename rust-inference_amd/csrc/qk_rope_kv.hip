@@ -26,16 +26,18 @@ __global__ void qk_norm_rope_kv_write_kernel(
     TA* x = qkv + (size_t)t * all_heads * head_dim + (size_t)hh * head_dim;
 
     const int pos = tok_pos[t];
-    TC* dst = nullptr;          // where a k or v head goes
+    TC* dst = nullptr;          // where a k head goes
     if (hh >= heads) {
         const int kvh = (hh - heads) % kv_heads;
         const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
-        TC* pool = hh < heads + kv_heads ? k_pages : v_pages;
-        dst = pool + (((size_t)page * kv_heads + kvh) * page_size + pos % page_size) * head_dim;
-    }
-    if (hh >= heads + kv_heads) {                          // v: a copy, no norm and no rotation
-        for (int d = lane; d < head_dim; d += RI_WAVE) from_f32(dst + d, to_f32(x[d]));
-        return;
+        const size_t head_base = ((size_t)page * kv_heads + kvh) * page_size * head_dim;
+        if (hh >= heads + kv_heads) {
+            // v: a copy, no norm and no rotation, transposed inside the page: [head_dim][page_size]
+            TC* vt = v_pages + head_base + pos % page_size;
+            for (int d = lane; d < head_dim; d += RI_WAVE) from_f32(vt + (size_t)d * page_size, to_f32(x[d]));
+            return;
+        }
+        dst = k_pages + head_base + (size_t)(pos % page_size) * head_dim;
     }
 
     // lane owns pairs i = lane, lane + 64, ...: elements (i, i + half)

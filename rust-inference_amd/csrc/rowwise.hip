@@ -110,23 +110,25 @@ extern "C" int ri_add_rows(float* out, const float* residual, const void* pendin
 __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 
 template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ y, int inter) {
-    const int t = blockIdx.y;
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= inter) return;
-    const T* row = y + (size_t)t * 2 * inter;
-    from_f32(out + (size_t)t * inter + i, silu(to_f32(row[i])) * to_f32(row[inter + i]));
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ y, int inter, long total) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const long t = e / inter;
+    const int i = (int)(e - t * inter);
+    const T* row = y + t * 2 * inter;
+    from_f32(out + e, silu(to_f32(row[i])) * to_f32(row[inter + i]));
 }
 
 extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream) {
     RI_REQUIRE(tokens > 0 && inter > 0, "swiglu: tokens %d, inter %d", tokens, inter);
-    RI_REQUIRE(tokens <= 65535, "swiglu: %d tokens exceed one launch (65535)", tokens);
-    dim3 grid((inter + 255) / 256, tokens);
+    const long total = (long)tokens * inter;
+    RI_REQUIRE((total + 255) / 256 <= 2147483647L, "swiglu: %ld elements exceed one launch", total);
+    const unsigned grid = (unsigned)((total + 255) / 256);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == RI_F32)
-        swiglu_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)y, inter);
+        swiglu_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)y, inter, total);
     else if (dtype == RI_BF16)
-        swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, inter);
+        swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, inter, total);
     else
         RI_REQUIRE(false, "swiglu: dtype %d", dtype);
     RI_LAUNCH_CHECK("swiglu");

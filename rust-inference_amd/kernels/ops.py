@@ -27,6 +27,10 @@ _SIGNATURES = {
                                  c_void_p],
     "ri_attention": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -144,7 +148,7 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, 
     tokens = qkv.shape[0]
     width = (heads + 2 * kv_heads) * head_dim
     num_pages, hkv, page_size, dh = k_pages.shape
-    if (hkv, dh) != (kv_heads, head_dim) or v_pages.shape != k_pages.shape:
+    if (hkv, dh) != (kv_heads, head_dim) or tuple(v_pages.shape) != (num_pages, hkv, dh, page_size):
         raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv heads "
                          f"of {head_dim}")
     half = head_dim // 2
@@ -167,6 +171,47 @@ def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, k
           _dev(tok_seq, "tok_seq", torch.int32, (tokens,)), _dev(page_table, "page_table", torch.int32),
           page_table.shape[1], tokens, heads, kv_heads, head_dim, k_pages.shape[2], int(window or 0), float(scale),
           _stream())
+    return out
+
+
+MFMA_HEAD_DIMS = (32, 64, 128)
+DECODE_CHUNK = 256
+
+
+def mfma_attention_fits(dtype, head_dim: int, group: int, page_size: int, decode: bool) -> bool:
+    """Whether the matrix-core attention kernels take this case (else the generic kernel does)."""
+    return (dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page_size == 32
+            and group <= (16 if decode else (64 if head_dim <= 64 else 32)))
+
+
+def attention_prefill_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_new: int,
+                           heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float) -> torch.Tensor:
+    """Matrix-core attention for any number of new tokens per sequence (bfloat16, pages of 32)."""
+    tokens, stride = qkv.shape
+    out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    _call("ri_attention_prefill_bf16", _dev(out, "out"), _dev(qkv, "qkv", torch.bfloat16), stride,
+          _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, max_new, heads, kv_heads, head_dim,
+          k_pages.shape[2], int(window or 0), float(scale), _stream())
+    return out
+
+
+def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_len: int,
+                          heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float) -> torch.Tensor:
+    """Matrix-core attention for one new token per sequence; ``max_len`` bounds every sequence's length
+    after this step (it sizes the grid and the workspace, not the result)."""
+    tokens, stride = qkv.shape
+    if tokens != seqs:
+        raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
+    chunks = -(-max_len // DECODE_CHUNK)
+    out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
+    _call("ri_attention_decode_bf16", _dev(out, "out"), _dev(ws, "workspace"), _dev(qkv, "qkv", torch.bfloat16), stride,
+          _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
+          _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
+          k_pages.shape[2], int(window or 0), float(scale), _stream())
     return out
 
 

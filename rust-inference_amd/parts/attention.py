@@ -75,6 +75,17 @@ class GroupedQueryAttention(Mixer):
         ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
                                   ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
                                   self.heads, self.kv_heads, self.head_dim)
-        o = ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table,
-                          self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
-        return rt.linear(o, self.w_o)
+        return rt.linear(self.attend(qkv, ctx, store, page_table), self.w_o)
+
+    def attend(self, qkv, ctx, store, page_table):
+        """The attention kernel that fits the step: matrix cores for bfloat16 (one new token per
+        sequence, or any number), the generic kernel for everything else."""
+        args = (self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
+        group = self.heads // self.kv_heads
+        if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
+            if ctx.is_decode:
+                return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
+                                                 page_table, ctx.B, ctx.max_len, *args)
+            return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
+                                              page_table, ctx.B, ctx.max_new, *args)
+        return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args)

@@ -81,6 +81,7 @@ def test_groups_with_different_needs_have_storage_of_their_own():
     assert len(c.groups) == 3
     assert [g.entries for g in c.groups] == [[0, 3], [1], [2]]
     assert c.kv(3).k_pages.shape == (8, 2, 32, 16) and c.kv(2).k_pages.shape == (8, 1, 32, 32)
+    assert c.kv(3).v_pages.shape == (8, 2, 16, 32)
     assert c.kv(0).k_pages.data_ptr() != c.kv(3).k_pages.data_ptr()
     assert c.state(4).shape == (4, 5) and c.has_state(4) and not c.has_state(0)
     s = c.acquire()

@@ -88,13 +88,13 @@ def paged(rng, lens, hkv, dh, page_size=32, dtype=torch.float32, spare=3):
     k = [rng.normal(size=(n, hkv, dh)) for n in lens]
     v = [rng.normal(size=(n, hkv, dh)) for n in lens]
     kp = np.zeros((num_pages, hkv, page_size, dh))
-    vp = np.zeros((num_pages, hkv, page_size, dh))
+    vp = np.zeros((num_pages, hkv, dh, page_size))                 # values lie transposed inside a page
     for b, n in enumerate(lens):
         for lp in range(pages_per[b]):
             table[b, lp] = order.pop()
         for pos in range(n):
             kp[table[b, pos // page_size], :, pos % page_size] = k[b][pos]
-            vp[table[b, pos // page_size], :, pos % page_size] = v[b][pos]
+            vp[table[b, pos // page_size], :, :, pos % page_size] = v[b][pos]
     return k, v, t(kp, dtype), t(vp, dtype), t(table, torch.int32)
 
 
@@ -128,7 +128,7 @@ def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh):
     for i in range(tokens):
         page, off = tab[tok_seq[i], tok_pos[i] // 32], tok_pos[i] % 32
         close(kp[page, :, off], k_want[i], rel, f"k of token {i}")
-        assert np.array_equal(f64(vp[page, :, off]), v[i]), "v is a copy"
+        assert np.array_equal(f64(vp[page, :, :, off]), v[i]), "v is a copy"
     # nothing else was written: as many rows are non-zero as tokens
     assert int((kp.float().abs().sum(-1) > 0).sum()) == tokens * kv_heads
     # without gains and rotation the kernel only moves k and v
@@ -138,8 +138,8 @@ def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh):
     assert np.array_equal(f64(qkv2), qkv)
 
 
-def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None, boost=None):
-    k, v, kp, vp, table = paged(rng, lens, kv_heads, dh, dtype=dtype)
+def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None, boost=None, kernel="generic"):
+    k, v, kp, vp, table = paged(rng, lens, kv_heads, dh, dtype=dtype, spare=12)
     tokens = sum(new)
     width = (heads + 2 * kv_heads) * dh
     qkv = np.zeros((tokens, width))
@@ -149,14 +149,25 @@ def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None,
     if boost is not None:
         boost(qkv, k, kp, table)
     qkv_t = t(qkv, dtype)
-    out = ops.attention(qkv_t, kp, vp, t(tok_pos, torch.int32), t(tok_seq, torch.int32), table, heads, kv_heads, dh,
-                        window, 1.0 / np.sqrt(dh))
+    pos_t, seq_t = t(tok_pos, torch.int32), t(tok_seq, torch.int32)
+    cu = t(np.concatenate([[0], np.cumsum(new)]), torch.int32)
+    scale = 1.0 / np.sqrt(dh)
+    if kernel == "generic":
+        out = ops.attention(qkv_t, kp, vp, pos_t, seq_t, table, heads, kv_heads, dh, window, scale)
+    elif kernel == "prefill":
+        out = ops.attention_prefill_bf16(qkv_t, kp, vp, cu, pos_t, table, len(lens), max(new), heads, kv_heads, dh,
+                                         window, scale)
+    else:
+        assert all(n == 1 for n in new)
+        # a bound on the length well above the real one: it sizes grid and workspace, never the result
+        out = ops.attention_decode_bf16(qkv_t, kp, vp, cu, pos_t, table, len(lens), max(lens) + 300, heads,
+                                        kv_heads, dh, window, scale)
     q = f64(qkv_t)[:, :heads * dh].reshape(tokens, heads, dh)
     want = np.zeros((tokens, heads, dh))
     i = 0
     for b, n in enumerate(new):
         kb = np.stack([f64(kp[table[b, p // 32].item(), :, p % 32]) for p in range(lens[b])])
-        vb = np.stack([f64(vp[table[b, p // 32].item(), :, p % 32]) for p in range(lens[b])])
+        vb = np.stack([f64(vp[table[b, p // 32].item(), :, :, p % 32]) for p in range(lens[b])])
         want[i:i + n] = P.attention(q[i:i + n], kb, vb, window=window)
         i += n
     return out.reshape(tokens, heads, dh), want
@@ -193,6 +204,62 @@ def test_attention_window_edges(ops, dtype, window):
     rng = np.random.default_rng(window)
     out, want = attention_case(ops, rng, [290, 40], [34, 40], 4, 2, 32, dtype, window=window)
     close(out, want, 3e-6 if dtype == torch.float32 else 1e-2, f"window {window}")
+
+
+MFMA_SHAPES = [(4, 1, 32), (8, 2, 32), (6, 2, 64), (3, 3, 64), (32, 8, 128), (16, 1, 128), (5, 5, 128)]
+
+
+@pytest.mark.parametrize("heads, kv_heads, dh", MFMA_SHAPES)
+def test_mfma_prefill_attention(ops, heads, kv_heads, dh):
+    rng = np.random.default_rng(heads * 7 + dh)
+    # whole prompts of unequal lengths (one shorter than a tile, one of one token), and pieces that
+    # continue sequences already in the cache, all in one call
+    out, want = attention_case(ops, rng, [70, 300, 257, 1, 45, 131], [70, 5, 1, 1, 45, 99], heads, kv_heads, dh,
+                               torch.bfloat16, kernel="prefill")
+    close(out, want, 1e-2, "prefill attention on the matrix cores")
+
+
+@pytest.mark.parametrize("heads, kv_heads, dh", MFMA_SHAPES)
+def test_mfma_decode_attention(ops, heads, kv_heads, dh):
+    rng = np.random.default_rng(heads * 11 + dh)
+    # lengths at and around page and chunk edges: 1, 32, 33, 256, 257, 512, 700
+    lens = [1, 32, 33, 256, 257, 512, 700, 5]
+    out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, kernel="decode")
+    close(out, want, 1e-2, "decode attention on the matrix cores")
+
+
+@pytest.mark.parametrize("kernel", ["prefill", "decode"])
+def test_mfma_attention_finds_one_far_key(ops, kernel):
+    rng = np.random.default_rng(19)
+    heads, kv_heads, dh = 8, 2, 128
+    for far in (0, 3, 4, 31, 32, 255, 256, 511, 640, 699):
+        def boost(qkv, k, kp, table, far=far):
+            kf = f64(kp[table[0, far // 32].item(), 1, far % 32])          # kv head 1: query heads 4..7
+            qkv[0, 6 * dh:7 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        out, want = attention_case(ops, rng, [700], [1], heads, kv_heads, dh, torch.bfloat16, boost=boost,
+                                   kernel=kernel)
+        close(out, want, 1e-2, f"far key {far}")
+        vfar = f64(out[0, 6])
+        assert np.abs(vfar - want[0, 6]).max() < 0.05
+
+
+@pytest.mark.parametrize("kernel", ["prefill", "decode"])
+@pytest.mark.parametrize("window", [1, 32, 33, 100, 256, 300])
+def test_mfma_attention_window_edges(ops, kernel, window):
+    rng = np.random.default_rng(window + 5)
+    new = [1, 1] if kernel == "decode" else [34, 40]
+    out, want = attention_case(ops, rng, [290, 40], new, 4, 2, 64, torch.bfloat16, window=window, kernel=kernel)
+    close(out, want, 1e-2, f"window {window}")
+
+
+def test_mfma_and_generic_attention_agree(ops):
+    """The same call through all three kernels: decode against prefill against generic."""
+    outs = []
+    for kernel in ("generic", "prefill", "decode"):
+        rng = np.random.default_rng(23)
+        out, want = attention_case(ops, rng, [400, 77, 1], [1, 1, 1], 8, 2, 128, torch.bfloat16, kernel=kernel)
+        outs.append(f64(out))
+    assert np.abs(outs[0] - outs[1]).max() < 2e-2 and np.abs(outs[1] - outs[2]).max() < 2e-2
 
 
 @pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
@@ -263,7 +330,7 @@ def test_kernels_refuse_what_they_cannot_do(ops):
         ops.gemv_bf16(torch.zeros(9, 16, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(KernelError, match="multiple of 16"):
         ops.attention(torch.zeros(1, 3 * 24, device=DEV), torch.zeros(1, 1, 32, 24, device=DEV),
-                      torch.zeros(1, 1, 32, 24, device=DEV), t([0], torch.int32), t([0], torch.int32),
+                      torch.zeros(1, 1, 24, 32, device=DEV), t([0], torch.int32), t([0], torch.int32),
                       t([[0]], torch.int32), 1, 1, 24, None, 1.0)
     with pytest.raises(ShapeError, match="contiguous"):
         ops.swiglu(torch.zeros(4, 8, device=DEV)[:, ::2])
