@@ -56,6 +56,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prompt", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this library is single-GPU, --gpus {args.gpus} is not run")
@@ -81,7 +82,8 @@ def main() -> int:
 
     def fresh_engine(batch):
         per_seq = -(-args.context // 32) * 32
-        return Engine(model, model.new_cache(max_tokens=per_seq * batch, num_slots=batch, max_seq_len=args.context))
+        return Engine(model, model.new_cache(max_tokens=per_seq * batch, num_slots=batch, max_seq_len=args.context),
+                      use_graphs=not args.no_graphs)
 
     def sync():
         torch.cuda.synchronize()

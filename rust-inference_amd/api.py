@@ -30,14 +30,15 @@ def as_dtype(dtype) -> torch.dtype:
 class Model:
     """A loaded model with a cache sized for ``max_batch`` sequences of ``max_seq_len`` tokens."""
 
-    def __init__(self, decoder, max_batch: int = 8, max_seq_len: int = 4096, max_tokens: int | None = None):
+    def __init__(self, decoder, max_batch: int = 8, max_seq_len: int = 4096, max_tokens: int | None = None,
+                 use_graphs: bool = True):
         self.decoder = decoder
         self.config = getattr(decoder, "config", None)
         max_seq_len = min(max_seq_len, decoder.spec.max_positions)
         page = 32
         per_seq = -(-max_seq_len // page) * page
         self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
-        self.engine = Engine(decoder, self.cache)
+        self.engine = Engine(decoder, self.cache, use_graphs=use_graphs)
 
     @classmethod
     def load(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **cache_options) -> "Model":

@@ -70,6 +70,11 @@ int ri_gemm_f32(float* out, const float* x, const void* w, int w_dtype, int m, i
 int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
                  void* stream);
 
+// The same product on the matrix cores for M <= 16: eight wavefronts split K, weights stream straight
+// into the MFMA operand.  Same swiglu convention.
+int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
+                        void* stream);
+
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);
 

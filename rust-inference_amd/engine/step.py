@@ -90,13 +90,32 @@ class _Staging:
         return self.dev
 
 
-class Engine:
-    """A model, its cache, and the step function over them."""
+class _DecodeGraph:
+    """One captured decode step for a fixed number of sequences: the kernels of the whole model as
+    one HIP graph, replayed with fresh tokens, positions and page tables in the same buffers."""
 
-    def __init__(self, model, cache):
+    def __init__(self, batch: int, device):
+        self.batch = batch
+        self.staging = None          # its own buffers: their addresses are part of the graph
+        self.graph = None
+        self.ctx = None
+        self.logits = None
+
+
+class Engine:
+    """A model, its cache, and the step function over them.
+
+    With ``use_graphs`` a step in which every sequence brings one token and wants its logits runs
+    as a HIP graph captured once per batch size: the launches of a decode step cost more than its
+    kernels otherwise.  Page tables then have the cache's full width and the attention grid is
+    sized for the longest sequence the cache allows; the results are the same."""
+
+    def __init__(self, model, cache, use_graphs: bool = False):
         self.model, self.cache = model, cache
         self.device = model.rt.device
+        self.use_graphs = use_graphs
         self._staging = None
+        self._graphs: dict[int, _DecodeGraph] = {}
 
     def _stage(self, n: int) -> _Staging:
         if self._staging is None or self._staging.capacity < n:
@@ -104,7 +123,8 @@ class Engine:
             self._staging = _Staging(cap, self.device)
         return self._staging
 
-    def build_context(self, entries: Sequence[StepEntry], table_width: int | None = None) -> StepContext:
+    def build_context(self, entries: Sequence[StepEntry], staging: _Staging | None = None,
+                      full_width: bool = False) -> StepContext:
         cache = self.cache
         slots = [e.slot for e in entries]
         starts = [cache.length(s) for s in slots]
@@ -113,7 +133,7 @@ class Engine:
         cache.reserve(slots, counts)
         len_after = [s + n for s, n in zip(starts, counts)]
         max_len = max(len_after)
-        width = table_width or -(-max_len // cache.page_size)
+        width = cache.max_pages_per_slot if full_width else -(-max_len // cache.page_size)
         pieces = [tokens, tok_seq, tok_pos, cu, slots, len_after, want_rows]
         for g in cache.groups:
             rows = g.table_rows(slots, width)
@@ -123,7 +143,7 @@ class Engine:
             offsets.append(len(flat))
             flat.extend(p)
             flat.extend([0] * (-len(flat) % 4))           # keep every piece 16-byte aligned
-        dev = self._stage(len(flat)).upload(flat)
+        dev = (staging or self._stage(len(flat))).upload(flat)
 
         def piece(i, n):
             return dev[offsets[i]:offsets[i] + n]
@@ -132,15 +152,43 @@ class Engine:
         ctx = StepContext(T=T, B=B, new_counts=counts, slot_list=slots, starts=starts,
                           tokens=piece(0, T), tok_seq=piece(1, T), tok_pos=piece(2, T), cu_seqlens=piece(3, B + 1),
                           slots=piece(4, B), len_after=piece(5, B), want_rows=piece(6, len(want_rows)),
-                          n_want=len(want_rows), max_new=max(counts), max_len=max_len)
+                          n_want=len(want_rows), max_new=max(counts),
+                          max_len=cache.max_seq_len if full_width else max_len)
         ctx.page_tables = [piece(7 + gi, B * width).view(B, width) for gi in range(len(cache.groups))]
         return ctx
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run one step; float32 logits ``[n_want, vocab]`` on the device, in the order of
-        the entries and of each entry's wanted places."""
+        the entries and of each entry's wanted places.  (With graphs the logits of a decode step
+        live in the graph's own buffer and are overwritten by the next decode step of that size.)"""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        if self.use_graphs and all(len(e.tokens) == 1 and wanted_indices(1, e.want) == [0] for e in entries):
+            return self._graph_step(entries)
         ctx = self.build_context(entries)
         logits = self.model.forward(ctx, self.cache)
         self.cache.commit(ctx.slot_list, ctx.new_counts)
         return logits
+
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        batch = len(entries)
+        dg = self._graphs.get(batch)
+        if dg is None:
+            dg = self._graphs[batch] = _DecodeGraph(batch, self.device)
+            width = self.cache.max_pages_per_slot
+            need = 7 * (batch + 4) + len(self.cache.groups) * (batch * width + 4)
+            dg.staging = _Staging(need, self.device)
+        # the layout of a decode step depends on the batch size alone, so the buffers a captured
+        # graph reads are refilled in place
+        ctx = self.build_context(entries, staging=dg.staging, full_width=True)
+        if dg.graph is None:
+            # once eagerly (libraries set themselves up outside the capture), then capture; writing
+            # the same keys and values to the same places twice changes nothing
+            self.model.forward(ctx, self.cache)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                dg.logits = self.model.forward(ctx, self.cache)
+            dg.graph, dg.ctx = graph, ctx
+        dg.graph.replay()
+        self.cache.commit(ctx.slot_list, ctx.new_counts)
+        return dg.logits

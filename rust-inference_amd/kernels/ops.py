@@ -33,6 +33,7 @@ _SIGNATURES = {
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemm_skinny_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -233,5 +234,16 @@ def gemv_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu
     n = w.shape[0] // 2 if swiglu else w.shape[0]
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _call("ri_gemv_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
+          _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
+    return out
+
+
+def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu: bool = False) -> torch.Tensor:
+    """``x @ w.T`` for up to 16 bfloat16 rows on the matrix cores, the weights read once; ``swiglu`` as
+    in ``gemv_bf16``."""
+    m, k = x.shape
+    n = w.shape[0] // 2 if swiglu else w.shape[0]
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _call("ri_gemm_skinny_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
           _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
     return out

@@ -7,7 +7,14 @@ import torch
 from ..errors import KernelError, ShapeError
 from ..kernels import ops
 
-GEMV_MAX_ROWS = 8     # up to this many rows a product is a weight-streaming kernel of this library
+# Which product kernel runs, by the number of rows of x (measured on MI355X at Qwen3-8B sizes with the
+# weights streamed from HBM): the one-wavefront-per-row kernel is fastest for one or two rows
+# (5.1 to 5.5 TB/s on the large matrices); from three rows on it is bound by its vector
+# arithmetic and the vendor library's product is faster (4.2 to 4.9 TB/s); the matrix-core kernel of
+# this library wins only on matrices up to 4096 x 4096.
+GEMV_MAX_ROWS = 2
+SKINNY_MAX_ROWS = 16
+SKINNY_MAX_SIDE = 4096
 
 
 class Runtime:
@@ -47,8 +54,11 @@ class Runtime:
             raise ShapeError(f"linear: x has {x.shape[1]} columns, the weight {w.shape[1]}")
         if self.dtype == torch.float32:
             return ops.gemm_f32(x, w)
-        if x.shape[0] <= GEMV_MAX_ROWS and x.shape[1] % 8 == 0:
+        m, k = x.shape
+        if m <= GEMV_MAX_ROWS and k % 8 == 0:
             return ops.gemv_bf16(x, w, out_dtype)
+        if m <= SKINNY_MAX_ROWS and k % 8 == 0 and k <= SKINNY_MAX_SIDE and w.shape[0] <= SKINNY_MAX_SIDE:
+            return ops.gemm_skinny_bf16(x, w, out_dtype)
         return self._library_mm(x, w, out_dtype)
 
     def _library_mm(self, x, w, out_dtype):

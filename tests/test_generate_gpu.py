@@ -1,0 +1,108 @@
+"""Generation through the Python entry point and the command line on the GPU, against the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import read_model_f64
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_greedy_with_margins(model_dir, prompts, steps, stop=()):
+    cfg, w = read_model_f64(model_dir)
+    out = []
+    for p in prompts:
+        toks, rows = P.greedy(cfg, w, p, steps, stop)
+        margins = [float(np.sort(r)[-1] - np.sort(r)[-2]) for r in rows]
+        out.append((toks, margins))
+    return out
+
+
+def assert_same_tokens(got, want, dtype_name):
+    """Token for token; in bfloat16 a sequence may part from the plain one only at a place where the
+    plain implementation's two best logits are closer than bfloat16 rounding of the logits."""
+    for i, (g, (toks, margins)) in enumerate(zip(got, want)):
+        for j, (a, b) in enumerate(zip(g, toks)):
+            if a != b:
+                assert dtype_name == "bfloat16" and margins[j] < 0.08, \
+                    f"request {i}, token {j}: {a} against {b} (margin {margins[j]:.3f}, {dtype_name})"
+                break
+        else:
+            assert len(g) == len(toks), f"request {i}: {len(g)} tokens against {len(toks)}"
+
+
+def prompts_for(cfg, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in lengths]
+
+
+@pytest.mark.parametrize("use_graphs", [False, True])
+@pytest.mark.parametrize("name, lengths, steps, dtype_name", [
+    ("A", [5, 11, 1, 17], 8, "float32"), ("A", [5, 11, 1, 17], 8, "bfloat16"),
+    ("B", [33, 2, 40], 16, "float32"), ("B", [33, 2, 40], 16, "bfloat16"),
+])
+def test_greedy_generation_through_the_entry_point(model_dirs, name, lengths, steps, dtype_name, use_graphs):
+    from rust_inference_amd import Model
+    cfg, _ = read_model_f64(model_dirs[name])
+    prompts = prompts_for(cfg, lengths, 3)
+    model = Model.load(model_dirs[name], dtype=dtype_name, max_batch=4, max_seq_len=96, use_graphs=use_graphs)
+    res = model.generate(prompts, max_new_tokens=steps)
+    assert_same_tokens(res.tokens, plain_greedy_with_margins(model_dirs[name], prompts, steps), dtype_name)
+    assert res.finish_reasons == ["length"] * len(prompts)
+    assert res.stats.prompt_tokens == sum(lengths) and res.stats.decode_tokens == len(prompts) * (steps - 1)
+    model.cache.check_consistent()
+    assert model.cache.slots.free_count == 4
+
+
+def test_stop_tokens_and_batches_one_after_another(model_dirs):
+    """Five requests on two slots: three batches, slots used again; a stop token ends sequences early."""
+    from rust_inference_amd import Model
+    cfg, _ = read_model_f64(model_dirs["A"])
+    prompts = prompts_for(cfg, [4, 9, 2, 7, 12], 4)
+    free = plain_greedy_with_margins(model_dirs["A"], prompts, 10)
+    stop = [free[1][0][3], free[3][0][0]]                       # ends request 1 after 3 tokens, request 3 at once
+    want = plain_greedy_with_margins(model_dirs["A"], prompts, 10, stop)
+    model = Model.load(model_dirs["A"], dtype="float32", max_batch=2, max_seq_len=64)
+    res = model.generate(prompts, max_new_tokens=10, stop_token_ids=stop)
+    assert_same_tokens(res.tokens, want, "float32")
+    assert res.stats.batches == 3 and res.finish_reasons[3] == "stop" and res.tokens[3] == []
+    assert all(s not in toks for toks in res.tokens for s in stop)
+
+
+def test_graph_and_eager_decoding_give_the_same_logits(model_dirs):
+    import torch
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.parts import load_model
+    model = load_model(model_dirs["B"], torch.bfloat16)
+    cfg, _ = read_model_f64(model_dirs["B"])
+    prompts = prompts_for(cfg, [33, 2, 40], 5)
+    outs = []
+    for graphs in (False, True):
+        eng = Engine(model, model.new_cache(max_tokens=3 * 96, num_slots=3, max_seq_len=96), use_graphs=graphs)
+        slots = [eng.cache.acquire() for _ in prompts]
+        eng.step([StepEntry(s, p, "last") for s, p in zip(slots, prompts)])
+        rows = []
+        for step in range(20):
+            live = slots if step < 12 else slots[:2]            # a sequence leaves: another batch size, another graph
+            rows.append(eng.step([StepEntry(s, [(7 * step + s) % 300], "last") for s in live]).clone())
+        outs.append(rows)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b), "a captured step must compute what the launched one computes"
+
+
+def test_temperature_sampling_is_seeded(model_dirs):
+    from rust_inference_amd import Model
+    cfg, _ = read_model_f64(model_dirs["A"])
+    prompts = prompts_for(cfg, [6, 3], 6)
+    model = Model.load(model_dirs["A"], dtype="float32", max_batch=2, max_seq_len=64)
+    a = model.generate(prompts, max_new_tokens=12, temperature=0.8, seed=1).tokens
+    b = model.generate(prompts, max_new_tokens=12, temperature=0.8, seed=1).tokens
+    c = model.generate(prompts, max_new_tokens=12, temperature=0.8, seed=2).tokens
+    alone = model.generate(prompts[:1], max_new_tokens=12, temperature=0.8, seed=1).tokens
+    assert a == b and a != c and alone[0] == a[0]

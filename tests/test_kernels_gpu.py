@@ -302,6 +302,22 @@ def test_gemv_bf16(ops, m, out_dtype):
         assert torch.equal(ops.gemv_bf16(x, w, out_dtype)[m - 1:], ops.gemv_bf16(x[m - 1:].contiguous(), w, out_dtype))
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 13, 16])
+@pytest.mark.parametrize("n, k", [(37, 584), (100, 96), (4096, 4096), (50, 12288)])
+def test_gemm_skinny_bf16(ops, m, n, k):
+    rng = np.random.default_rng(m + n)
+    x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
+    want = f64(x) @ f64(w).T
+    close(ops.gemm_skinny_bf16(x, w, torch.float32), want, 3e-6, "skinny product")
+    close(ops.gemm_skinny_bf16(x, w, torch.bfloat16), want, 5e-3, "skinny product, bfloat16 out")
+    wgu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
+    y = f64(x) @ f64(wgu).T
+    close(ops.gemm_skinny_bf16(x, wgu, torch.float32, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 5e-6, "with swiglu")
+    if m > 1:      # a row's result does not depend on the other rows: bit for bit
+        assert torch.equal(ops.gemm_skinny_bf16(x, w, torch.float32)[m - 1:],
+                           ops.gemm_skinny_bf16(x[m - 1:].contiguous(), w, torch.float32))
+
+
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 1e-6), (torch.bfloat16, 5e-3)])
 def test_swiglu(ops, dtype, rel):
     assert f64(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])))[0, 0] == 0.0                 # src/ops/elementwise.rs:59-70
