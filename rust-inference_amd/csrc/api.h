@@ -78,8 +78,9 @@ int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, 
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);
 
-// ids[r] = first index of the maximum of logits[r, :] (float32).
-int ri_argmax(int32_t* ids, const float* logits, int rows, int vocab, void* stream);
+// ids[r] = first index of the maximum of logits[r, :] (float32).  workspace: ri_argmax_workspace_bytes(rows).
+int ri_argmax_workspace_bytes(int rows);
+int ri_argmax(int32_t* ids, const float* logits, void* workspace, int rows, int vocab, void* stream);
 
 #ifdef __cplusplus
 }

@@ -22,7 +22,7 @@
 //
 // Prefill: one wavefront per tile of tokens, walking the sequence's pages in order.  Decode (one new
 // token per sequence): the keys are cut into chunks of 256 at fixed places, one workgroup per chunk
-// (its four wavefronts take two pages each), partial results go to a workspace and a second kernel
+// (its eight wavefronts take one page each), partial results go to a workspace and a second kernel
 // joins them in chunk order.  Neither order depends on the batch or on how tokens were cut.
 #include "api.h"
 #include "common.h"
@@ -38,7 +38,7 @@ union Frag {
 
 #define PAGE 32
 #define DECODE_CHUNK 256          // keys per workgroup of the decode kernel: 8 pages
-#define DECODE_WAVES 4
+#define DECODE_WAVES 8            // wavefronts of a decode workgroup: one page each
 
 template <int DH>
 struct PageFrags {
@@ -208,19 +208,23 @@ template <int DH>
 __global__ void __launch_bounds__(DECODE_WAVES * 64)
 attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride,
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-                        const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ tok_pos,
-                        const int32_t* __restrict__ page_table, int table_width, int heads, int kv_heads,
-                        int window, float scale_log2, int max_chunks) {
+                        const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                        int heads, int kv_heads, int window, float scale_log2, int max_chunks) {
     __shared__ float o_lds[DECODE_WAVES][DH * 17];           // [d * 17 + col]: no bank conflicts either way
     __shared__ float ml_lds[DECODE_WAVES][2][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int chunk = blockIdx.x, b = blockIdx.y, kvh = blockIdx.z;
     const int group = heads / kv_heads;
-    const int tok = cu_seqlens[b];                           // the sequence's one new token
+    const int tok = b;                                       // one new token per sequence: token b is sequence b's
     const int qpos = tok_pos[tok];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
+
+    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;   // this wavefront's page
+    const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
+    PageFrags<DH> f;
+    if (has) load_page<DH>(f, k_pages, v_pages, page_table[(long)b * table_width + page], kv_heads, kvh, lane);
 
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
@@ -232,16 +236,7 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
     }
-    const int32_t* table = page_table + (long)b * table_width;
-    const int pages_per_chunk = DECODE_CHUNK / PAGE;
-    const int pa = chunk * pages_per_chunk + wave, pb = pa + DECODE_WAVES;     // this wavefront's two pages
-    const bool has_a = pa * PAGE <= qpos && pa * PAGE + PAGE - 1 >= lo;
-    const bool has_b = pb * PAGE <= qpos && pb * PAGE + PAGE - 1 >= lo;
-    PageFrags<DH> fa, fb;
-    if (has_a) load_page<DH>(fa, k_pages, v_pages, table[pa], kv_heads, kvh, lane);
-    if (has_b) load_page<DH>(fb, k_pages, v_pages, table[pb], kv_heads, kvh, lane);
-    if (has_a) process_page<DH, 1>(c, fa, pa, lane, scale_log2);
-    if (has_b) process_page<DH, 1>(c, fb, pb, lane, scale_log2);
+    if (has) process_page<DH, 1>(c, f, page, lane, scale_log2);
 
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt)
@@ -261,9 +256,9 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 #pragma unroll
         for (int w = 0; w < DECODE_WAVES; ++w) {
             const float mw = ml_lds[w][0][g];
-            const float f = mw == -INFINITY ? 0.f : exp2f(mw - m);
-            acc += o_lds[w][d * 17 + g] * f;
-            l += ml_lds[w][1][g] * f;
+            const float f2 = mw == -INFINITY ? 0.f : exp2f(mw - m);
+            acc += o_lds[w][d * 17 + g] * f2;
+            l += ml_lds[w][1][g] * f2;
         }
         float* dst = ws + (((long)b * heads + kvh * group + g) * max_chunks + chunk) * (DH + 2);
         dst[d] = acc;
@@ -276,10 +271,10 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 
 template <int DH>
 __global__ void __launch_bounds__(DH)
-attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ cu_seqlens,
+attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws,
                         const int32_t* __restrict__ tok_pos, int heads, int window, int max_chunks) {
     const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
-    const int tok = cu_seqlens[b];
+    const int tok = b;
     const int qpos = tok_pos[tok];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     const int c_lo = lo / DECODE_CHUNK, c_hi = qpos / DECODE_CHUNK;
@@ -361,10 +356,10 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
 #define RI_DECODE_CASE(DH)                                                                                        \
     case DH:                                                                                                      \
         attn_decode_mfma_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                           \
-            workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, cu_seqlens, \
+            workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
             tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks);                   \
-        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, cu_seqlens,        \
-                                                                      tok_pos, heads, window, max_chunks);        \
+        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos, heads,    \
+                                                                      window, max_chunks);                        \
         break;
     switch (head_dim) {
         RI_DECODE_CASE(32)

@@ -56,13 +56,88 @@ __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ res
     }
 }
 
+// The same for rows of up to 8192 elements (a multiple of 4): every thread loads its elements in
+// 16-byte pieces up front and keeps them in registers, so the loads of a row are in flight together
+// and the row is read once.  The sum of squares is taken per thread over its own elements, then over
+// the workgroup in a fixed order.
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xFFFF0000u), __uint_as_float(w.y << 16),
+                       __uint_as_float(w.y & 0xFFFF0000u));
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, float4 v) {
+    uint2 w;
+    w.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+    w.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = w;
+}
+
+template <typename TP, typename TO, int VPT>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const TP* __restrict__ pending,
+                       const float* __restrict__ gain, float eps, const int32_t* __restrict__ rows, int dim) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const size_t src = (size_t)(rows ? rows[row] : row) * dim;
+    const bool write_back = rows == nullptr && pending != nullptr;
+    float4 v[VPT], g[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int d = (i * 256 + threadIdx.x) * 4;
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (d < dim) {
+            v[i] = load4(residual + src + d);
+            g[i] = load4(gain + d);
+            if (pending) {
+                const float4 p = load4(pending + src + d);
+                v[i].x += p.x; v[i].y += p.y; v[i].z += p.z; v[i].w += p.w;
+            }
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int d = (i * 256 + threadIdx.x) * 4;
+        if (d < dim) {
+            if (write_back) store4(residual + src + d, v[i]);
+            ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)dim + eps);
+    TO* o = out + (size_t)row * dim;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int d = (i * 256 + threadIdx.x) * 4;
+        if (d < dim)
+            store4(o + d, make_float4(v[i].x * inv * g[i].x, v[i].y * inv * g[i].y, v[i].z * inv * g[i].z,
+                                      v[i].w * inv * g[i].w));
+    }
+}
+
+template <typename TP, typename TO>
+static void launch_add_rmsnorm_typed(TO* out, float* residual, const TP* pending, const float* gain, float eps,
+                                     const int32_t* rows, int n_rows, int dim, hipStream_t s) {
+    if (dim % 4 == 0 && dim <= 1024)
+        add_rmsnorm_vec_kernel<TP, TO, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+    else if (dim % 4 == 0 && dim <= 2048)
+        add_rmsnorm_vec_kernel<TP, TO, 2><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+    else if (dim % 4 == 0 && dim <= 4096)
+        add_rmsnorm_vec_kernel<TP, TO, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+    else if (dim % 4 == 0 && dim <= 8192)
+        add_rmsnorm_vec_kernel<TP, TO, 8><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+    else
+        add_rmsnorm_kernel<TP, TO><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+}
+
 template <typename TP>
 static void launch_add_rmsnorm(void* out, int out_dtype, float* residual, const TP* pending, const float* gain,
                                float eps, const int32_t* rows, int n_rows, int dim, hipStream_t s) {
     if (out_dtype == RI_F32)
-        add_rmsnorm_kernel<TP, float><<<n_rows, 256, 0, s>>>((float*)out, residual, pending, gain, eps, rows, dim);
+        launch_add_rmsnorm_typed<TP, float>((float*)out, residual, pending, gain, eps, rows, n_rows, dim, s);
     else
-        add_rmsnorm_kernel<TP, bf16_t><<<n_rows, 256, 0, s>>>((bf16_t*)out, residual, pending, gain, eps, rows, dim);
+        launch_add_rmsnorm_typed<TP, bf16_t>((bf16_t*)out, residual, pending, gain, eps, rows, n_rows, dim, s);
 }
 
 extern "C" int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype,
@@ -142,13 +217,12 @@ __device__ __forceinline__ void better(float& v, int& i, float ov, int oi) {
     if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
 }
 
-__global__ void argmax_kernel(int32_t* __restrict__ ids, const float* __restrict__ logits, int vocab) {
-    __shared__ float sv[16];
-    __shared__ int si[16];
-    const float* row = logits + (size_t)blockIdx.x * vocab;
-    float v = -INFINITY;
-    int idx = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) better(v, idx, row[i], i);
+// Stage one: every workgroup takes a slice of the row and writes its best (value, index);
+// stage two: one workgroup per row picks the best of the slices.  Slices are in index order and
+// equal values keep the lower index, so the result is the first maximum of the row.
+#define ARGMAX_SLICES 64
+
+__device__ __forceinline__ void block_best(float& v, int& idx, float* sv, int* si) {
     for (int m = RI_WAVE / 2; m > 0; m >>= 1) {
         float ov = __shfl_xor(v, m, RI_WAVE);
         int oi = __shfl_xor(idx, m, RI_WAVE);
@@ -157,15 +231,48 @@ __global__ void argmax_kernel(int32_t* __restrict__ ids, const float* __restrict
     const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
     if (lane == 0) { sv[wave] = v; si[wave] = idx; }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0)
         for (int w = 1; w < (int)(blockDim.x / RI_WAVE); ++w) better(v, idx, sv[w], si[w]);
-        ids[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
+}
+
+__global__ void argmax_slices_kernel(float* __restrict__ part_v, int32_t* __restrict__ part_i,
+                                     const float* __restrict__ logits, int vocab, int per_slice) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const float* row = logits + (size_t)blockIdx.y * vocab;
+    const int begin = blockIdx.x * per_slice, end = min(vocab, begin + per_slice);
+    float v = -INFINITY;
+    int idx = 0x7FFFFFFF;
+    for (int i = begin + threadIdx.x; i < end; i += blockDim.x) better(v, idx, row[i], i);
+    block_best(v, idx, sv, si);
+    if (threadIdx.x == 0) {
+        part_v[blockIdx.y * ARGMAX_SLICES + blockIdx.x] = v;
+        part_i[blockIdx.y * ARGMAX_SLICES + blockIdx.x] = idx;
     }
 }
 
-extern "C" int ri_argmax(int32_t* ids, const float* logits, int rows, int vocab, void* stream) {
-    RI_REQUIRE(rows > 0 && vocab > 0, "argmax: rows %d, vocab %d", rows, vocab);
-    argmax_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(ids, logits, vocab);
+__global__ void argmax_pick_kernel(int32_t* __restrict__ ids, const float* __restrict__ part_v,
+                                   const int32_t* __restrict__ part_i) {
+    float v = part_v[blockIdx.x * ARGMAX_SLICES + threadIdx.x];
+    int idx = part_i[blockIdx.x * ARGMAX_SLICES + threadIdx.x];
+    for (int m = RI_WAVE / 2; m > 0; m >>= 1) {
+        float ov = __shfl_xor(v, m, RI_WAVE);
+        int oi = __shfl_xor(idx, m, RI_WAVE);
+        better(v, idx, ov, oi);
+    }
+    if (threadIdx.x == 0) ids[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
+}
+
+extern "C" int ri_argmax_workspace_bytes(int rows) { return rows * ARGMAX_SLICES * 8; }
+
+extern "C" int ri_argmax(int32_t* ids, const float* logits, void* workspace, int rows, int vocab, void* stream) {
+    RI_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "argmax: rows %d, vocab %d", rows, vocab);
+    float* part_v = (float*)workspace;
+    int32_t* part_i = (int32_t*)(part_v + (size_t)rows * ARGMAX_SLICES);
+    const int per_slice = (vocab + ARGMAX_SLICES - 1) / ARGMAX_SLICES;
+    hipStream_t s = (hipStream_t)stream;
+    argmax_slices_kernel<<<dim3(ARGMAX_SLICES, rows), 256, 0, s>>>(part_v, part_i, logits, vocab, per_slice);
+    argmax_pick_kernel<<<rows, ARGMAX_SLICES, 0, s>>>(ids, part_v, part_i);
     RI_LAUNCH_CHECK("argmax");
     return 0;
 }

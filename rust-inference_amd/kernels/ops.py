@@ -35,7 +35,7 @@ _SIGNATURES = {
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_skinny_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-    "ri_argmax": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
 _fn = {}
@@ -138,7 +138,9 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     """int32 index of the first maximum of every row of float32 ``logits``."""
     rows, vocab = logits.shape
     ids = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    _call("ri_argmax", _dev(ids, "ids"), _dev(logits, "logits", torch.float32), rows, vocab, _stream())
+    ws = torch.empty((rows * 64 * 2,), dtype=torch.int32, device=logits.device)      # 64 (value, index) pairs a row
+    _call("ri_argmax", _dev(ids, "ids"), _dev(logits, "logits", torch.float32), _dev(ws, "workspace"), rows, vocab,
+          _stream())
     return ids
 
 
