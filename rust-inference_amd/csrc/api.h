@@ -82,6 +82,16 @@ int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* 
 int ri_argmax_workspace_bytes(int rows);
 int ri_argmax(int32_t* ids, const float* logits, void* workspace, int rows, int vocab, void* stream);
 
+// Next-token selection, one row of float32 logits per sequence: repetition penalty over the token ids
+// marked in seen (a byte per vocabulary entry; row seen_rows[r] of it, or row r when seen_rows is NULL;
+// seen may be NULL), greedy when temperature <= 0, else temperature, top-k (0: off), top-p (1: off) and
+// one draw with uniform[r] in [0, 1).
+int ri_sample(int32_t* out, const float* logits, const uint8_t* seen, const int32_t* seen_rows, const float* uniform,
+              int rows, int vocab, float temperature, int top_k, float top_p, float penalty, void* stream);
+
+// seen[rows[i], tokens[i]] = 1 for i < n.
+int ri_mark_seen(uint8_t* seen, const int32_t* rows, const int32_t* tokens, int n, int vocab, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

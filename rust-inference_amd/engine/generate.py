@@ -18,7 +18,7 @@ from dataclasses import dataclass, field
 from typing import Sequence
 
 from ..errors import CacheError, ShapeError
-from ..sampling import SamplingParams, SequenceSampler, sample_batch
+from ..sampling import DeviceHistory, SamplingParams, SequenceSampler, sample_batch
 from .step import StepEntry
 
 
@@ -106,7 +106,10 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
     try:
         t0 = time.perf_counter()
         logits = engine.step([StepEntry(s.slot, s.prompt, "last") for s in live])
-        picks = sample_batch(logits, [s.sampler for s in live])
+        history = None
+        if sampling.repetition_penalty != 1.0 and logits.is_cuda:
+            history = DeviceHistory([s.sampler for s in live], logits.shape[1], logits.device)
+        picks = sample_batch(logits, [s.sampler for s in live], history)
         stats.prompt_tokens += sum(len(s.prompt) for s in live)
         stats.prefill_seconds += time.perf_counter() - t0      # includes the first sample, as in the reference
         for s, tok in zip(live, picks):
@@ -135,7 +138,9 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
             logits = engine.step([StepEntry(s.slot, [s.next_token], "last") for s in live])
             for s in live:
                 s.sampler.history.append(s.next_token)
-            picks = sample_batch(logits, [s.sampler for s in live])
+            if history is not None:
+                history.mark([s.sampler.seen_row for s in live], [s.next_token for s in live])
+            picks = sample_batch(logits, [s.sampler for s in live], history)
             for s, tok in zip(live, picks):
                 s.next_token = int(tok)
                 s.generated += 1

@@ -34,6 +34,9 @@ _SIGNATURES = {
     "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_skinny_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_float,
+                  c_void_p],
+    "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -142,6 +145,27 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _call("ri_argmax", _dev(ids, "ids"), _dev(logits, "logits", torch.float32), _dev(ws, "workspace"), rows, vocab,
           _stream())
     return ids
+
+
+def sample(logits: torch.Tensor, uniform, temperature: float, top_k: int = 0, top_p: float = 1.0,
+           penalty: float = 1.0, seen: torch.Tensor | None = None, seen_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """int32 token per row of float32 ``logits``: repetition penalty over the ids marked in ``seen``
+    (uint8 ``[*, vocab]``), greedy when the temperature is not positive, else temperature, top-k, top-p
+    and one draw with ``uniform[r]`` in [0, 1)."""
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _call("ri_sample", _dev(out, "out"), _dev(logits, "logits", torch.float32),
+          _opt(seen, "seen", torch.uint8), _opt(seen_rows, "seen_rows", torch.int32, (rows,)),
+          _opt(uniform, "uniform", torch.float32, (rows,)), rows, vocab, float(temperature), int(top_k), float(top_p),
+          float(penalty), _stream())
+    return out
+
+
+def mark_seen(seen: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor) -> None:
+    """``seen[rows[i], tokens[i]] = 1``."""
+    n = rows.shape[0]
+    _call("ri_mark_seen", _dev(seen, "seen", torch.uint8), _dev(rows, "rows", torch.int32, (n,)),
+          _dev(tokens, "tokens", torch.int32, (n,)), n, seen.shape[1], _stream())
 
 
 # ---------------------------------------------------------------- attention

@@ -1,5 +1,6 @@
-"""Sampling for a batch: one generator and one history per sequence, so that a
-sequence's tokens do not depend on what else is in its batch."""
+"""Sampling for a batch: one generator and one history per sequence, so that a sequence's tokens do
+not depend on what else is in its batch.  On the GPU the selection itself is the device kernel
+(one workgroup per sequence); the uniform draws come from each sequence's host generator."""
 from __future__ import annotations
 
 import torch
@@ -10,21 +11,55 @@ from .params import SamplingParams
 
 
 class SequenceSampler:
-    """The sampling state of one sequence.  Sequence ``index`` of a call draws from the
-    generator seeded ``seed + index``; sequence 0 has the reference's stream."""
+    """The sampling state of one sequence.  Sequence ``index`` of a call draws from the generator
+    seeded ``seed + index``; sequence 0 has the reference's stream."""
 
     def __init__(self, params: SamplingParams, index: int, prompt):
         self.params = params
         self.host = HostSampler(params, seed=(params.seed + index) & ((1 << 64) - 1))
         self.history = list(prompt)          # prompt plus generated, for the repetition penalty
+        self.seen_row = None                 # this sequence's row of the device history, when there is one
 
 
-def sample_batch(logits: torch.Tensor, samplers: list[SequenceSampler]) -> list[int]:
+class DeviceHistory:
+    """The repetition penalty's history on the device: a byte per vocabulary entry and sequence."""
+
+    def __init__(self, samplers: list[SequenceSampler], vocab: int, device):
+        self.seen = torch.zeros((len(samplers), vocab), dtype=torch.uint8, device=device)
+        rows, toks = [], []
+        for r, s in enumerate(samplers):
+            s.seen_row = r
+            rows.extend([r] * len(s.history))
+            toks.extend(s.history)
+        self.mark(rows, toks)
+
+    def mark(self, rows, tokens) -> None:
+        if rows:
+            dev = self.seen.device
+            ops.mark_seen(self.seen, torch.tensor(rows, dtype=torch.int32, device=dev),
+                          torch.tensor(tokens, dtype=torch.int32, device=dev))
+
+
+def sample_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> list[int]:
     """One token per row of float32 ``logits [B, vocab]``; appends nothing to the histories."""
     if logits.shape[0] != len(samplers):
         raise ValueError(f"{logits.shape[0]} rows of logits for {len(samplers)} sequences")
-    plain_greedy = all(s.params.greedy and s.params.repetition_penalty == 1.0 for s in samplers)
-    if plain_greedy and logits.is_cuda:
+    if not logits.is_cuda:          # logits that never were on a GPU (tests of the loop): the host sampler
+        rows = logits.detach().to(torch.float32).numpy()
+        return [s.host.sample(rows[i], s.history) for i, s in enumerate(samplers)]
+    p = samplers[0].params
+    if any(s.params != p for s in samplers):
+        raise ValueError("the sequences of one batch share their sampling parameters")
+    if p.greedy and p.repetition_penalty == 1.0:
         return ops.argmax(logits).tolist()
-    rows = logits.detach().to("cpu", torch.float32).numpy()
-    return [s.host.sample(rows[i], s.history) for i, s in enumerate(samplers)]
+    dev = logits.device
+    uniform = None
+    if not p.greedy:
+        uniform = torch.tensor([s.host.rng.next_f32() for s in samplers], dtype=torch.float32, device=dev)
+    seen = seen_rows = None
+    if p.repetition_penalty != 1.0:
+        if history is None:
+            raise ValueError("a repetition penalty needs the device history of the batch")
+        seen = history.seen
+        seen_rows = torch.tensor([s.seen_row for s in samplers], dtype=torch.int32, device=dev)
+    return ops.sample(logits, uniform, p.temperature, p.top_k, p.top_p, p.repetition_penalty, seen, seen_rows).tolist()
