@@ -1,0 +1,130 @@
+"""The command line, in the manner of the reference's runner (src/bin/runner.rs:24-123): the same
+option names and meanings where it has them.
+
+    runner <MODEL_DIR> [-p PROMPT] [-n N] [--temperature T] [--top-k K] [--top-p P]
+           [--repetition-penalty R] [--seed S] [--ignore-eos] [--max-pages N] [--pages-per-seq N]
+           [--dtype bfloat16|float32] [--profile]
+
+The prompt is text when the model folder has a tokenizer.json (read with the `tokenizers` package),
+else a list of token ids (`-p "5 17 3"` or `--prompt-ids 5,17,3`); it is read from standard input when
+omitted.  Several prompts (repeat `-p`, or one per input line with `--batch`) are served as a batch.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+from ..sampling import DEFAULT_SEED
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="runner", description="Text generation with a Qwen3 checkpoint on one MI355X")
+    ap.add_argument("model_dir", help="HuggingFace checkpoint directory (config.json, *.safetensors, tokenizer.json)")
+    ap.add_argument("-p", "--prompt", action="append", help="prompt text or token ids; read from stdin when omitted")
+    ap.add_argument("--prompt-ids", action="append", help="a prompt as comma-separated token ids")
+    ap.add_argument("--batch", action="store_true", help="read one prompt per line of standard input")
+    ap.add_argument("-n", "--max-new-tokens", type=int, default=600, help="number of tokens to generate")
+    ap.add_argument("--ignore-eos", action="store_true", help="keep generating past end-of-sequence tokens")
+    ap.add_argument("--tokenizer", help="directory holding tokenizer.json, if not the model directory")
+    ap.add_argument("--max-pages", type=int, default=256, help="KV cache pages per layer (32 tokens each)")
+    ap.add_argument("--pages-per-seq", type=int, default=128, help="maximum KV pages per sequence")
+    ap.add_argument("--profile", action="store_true", help="print a per-step timing summary at the end")
+    ap.add_argument("--temperature", type=float, default=0.0, help="sampling temperature; 0 = greedy")
+    ap.add_argument("--top-k", type=int, default=0, help="keep only the k most likely tokens (0 = off)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="nucleus sampling threshold (1.0 = off)")
+    ap.add_argument("--repetition-penalty", type=float, default=1.0, help="penalty for tokens already in the context")
+    ap.add_argument("--seed", type=lambda s: int(s, 0), default=DEFAULT_SEED, help="sampling seed")
+    ap.add_argument("--device", default="cuda", choices=["cuda"], help="this build runs on the GPU only")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="compute precision")
+    ap.add_argument("--stop-token-ids", default=None, help="comma-separated ids that end a sequence "
+                    "(default: eos_token_id of generation_config.json or config.json, if present)")
+    ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    return ap
+
+
+def load_tokenizer(folder: str):
+    path = os.path.join(folder, "tokenizer.json")
+    if not os.path.exists(path):
+        return None
+    try:
+        from tokenizers import Tokenizer
+    except ImportError:
+        return None
+    return Tokenizer.from_file(path)
+
+
+def default_stop_ids(model_dir: str) -> list[int]:
+    for name in ("generation_config.json", "config.json"):
+        path = os.path.join(model_dir, name)
+        if os.path.exists(path):
+            with open(path) as f:
+                eos = json.load(f).get("eos_token_id")
+            if eos is not None:
+                return [int(e) for e in (eos if isinstance(eos, list) else [eos])]
+    return []
+
+
+def parse_ids(text: str) -> list[int]:
+    return [int(t) for t in text.replace(",", " ").split()]
+
+
+def main(argv=None) -> int:
+    args = build_parser().parse_args(argv)
+    tokenizer = load_tokenizer(args.tokenizer or args.model_dir)
+    raw = list(args.prompt or [])
+    id_prompts = [parse_ids(p) for p in (args.prompt_ids or [])]
+    if not raw and not id_prompts:
+        lines = [ln.rstrip("\n") for ln in sys.stdin]
+        raw = [ln for ln in lines if ln.strip()] if args.batch else ["\n".join(lines).strip()]
+    prompts = list(id_prompts)
+    for p in raw:
+        prompts.append(tokenizer.encode(p).ids if tokenizer is not None else parse_ids(p))
+    if not prompts or any(len(p) == 0 for p in prompts):
+        print("error: empty prompt", file=sys.stderr)                  # src/bin/runner.rs:235-237
+        return 1
+
+    from ..api import Model
+    from ..errors import InferenceError
+    t0 = time.perf_counter()
+    try:
+        per_seq = args.pages_per_seq * 32
+        model = Model.load(args.model_dir, dtype=args.dtype, max_batch=min(len(prompts), 64), max_seq_len=per_seq,
+                           max_tokens=args.max_pages * 32, use_graphs=not args.no_graphs)
+    except InferenceError as e:
+        print(f"error: {e}", file=sys.stderr)
+        return 1
+    print(f"loaded {args.model_dir} in {time.perf_counter() - t0:.2f} s", file=sys.stderr)
+    stop = parse_ids(args.stop_token_ids) if args.stop_token_ids is not None else default_stop_ids(args.model_dir)
+
+    single = len(prompts) == 1
+
+    def on_token(request, token):
+        if single:                                                     # streamed, as the reference prints
+            sys.stdout.write(tokenizer.decode([token]) if tokenizer is not None else f"{token} ")
+            sys.stdout.flush()
+
+    try:
+        res = model.generate(prompts, max_new_tokens=args.max_new_tokens, temperature=args.temperature,
+                             top_k=args.top_k, top_p=args.top_p, repetition_penalty=args.repetition_penalty,
+                             seed=args.seed, stop_token_ids=stop, ignore_eos=args.ignore_eos, on_token=on_token)
+    except InferenceError as e:
+        print(f"error: {e}", file=sys.stderr)
+        return 1
+    if single:
+        print()
+    else:
+        for toks in res.tokens:
+            print(tokenizer.decode(toks) if tokenizer is not None else " ".join(str(t) for t in toks))
+    st = res.stats
+    print(f"prefill: {st.prompt_tokens} tokens in {st.prefill_seconds:.3f} s ({st.prefill_tokens_per_second:.1f} tok/s)",
+          file=sys.stderr)                                             # src/bin/runner.rs:243-251
+    print(f"decode: {st.decode_tokens} tokens in {st.decode_seconds:.3f} s ({st.decode_tokens_per_second:.1f} tok/s)",
+          file=sys.stderr)
+    if args.profile:
+        per_step = 1e3 * st.decode_seconds / st.decode_steps if st.decode_steps else 0.0
+        print(f"profile: {st.batches} batches, {st.decode_steps} decode steps, {per_step:.3f} ms per step",
+              file=sys.stderr)
+    return 0

@@ -1,0 +1,290 @@
+"""Each part alone against its plain counterpart, and the parts' generality: a toy architecture,
+registered here and nowhere in the package, with a windowed attention layer that runs twice (its
+weights shared, a cache entry per run), a toy mixer that keeps a state of its own per sequence, and
+no position encoding in one layer; built and stepped through the unchanged engine."""
+import json
+import os
+from dataclasses import dataclass
+from typing import ClassVar
+
+import numpy as np
+import pytest
+import torch
+
+import trace_plans as plans
+from helpers import assert_logits_close, rel_to_max
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def t(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+
+
+def f64(x):
+    return x.detach().to("cpu", torch.float64).numpy()
+
+
+class _StubModel:
+    """Just enough of a model for the engine to lay out a step for a part on its own."""
+    def __init__(self, rt, vocab=1000):
+        self.rt = rt
+        self.spec = type("S", (), {"vocab_size": vocab})()
+
+
+def context_for(rt, needs, counts, starts=None):
+    from rust_inference_amd.cache import Cache
+    from rust_inference_amd.engine import Engine, StepEntry
+    cache = Cache(needs, num_slots=len(counts), max_tokens=4096, max_seq_len=1024, dtype=rt.dtype, device=rt.device)
+    eng = Engine(_StubModel(rt), cache)
+    slots = [cache.acquire() for _ in counts]
+    if starts:                                   # pretend earlier steps: only the lengths matter to a test that
+        for s, n in zip(slots, starts):          # writes the earlier keys itself
+            if n:
+                cache.reserve([s], [n]); cache.commit([s], [n])
+    ctx = eng.build_context([StepEntry(s, [1] * n, "all") for s, n in zip(slots, counts)])
+    return cache, ctx
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(dtype):
+    from rust_inference_amd.parts import PartSpec, Runtime, build_part
+    rng = np.random.default_rng(0)
+    rt = Runtime(DEV, dtype)
+    norm = build_part("norm", PartSpec("rmsnorm", {"dim": 104, "eps": 3e-6, "name": "n.weight"}))
+    assert list(norm.tensors()) == ["n.weight"] and norm.tensors()["n.weight"].shape == (104,)
+    gain = torch.tensor(1 + 0.1 * rng.normal(size=104)).to(torch.bfloat16)
+    norm.bind({"n.weight": gain}, rt)
+    res, pend = t(rng.normal(size=(5, 104))), t(rng.normal(size=(5, 104)), dtype)
+    want = P.rms_norm(f64(res) + f64(pend), f64(gain), float(np.float32(3e-6)))
+    out = norm.apply(res, pend, dtype)
+    assert rel_to_max(f64(out), want) < (2e-6 if dtype == torch.float32 else 5e-3)
+
+
+def test_rotate_half_part_table():
+    from rust_inference_amd.parts import PartSpec, Runtime, build_part
+    for dh, theta in ((16, 10000.0), (48, 50000.0), (128, 1e6)):
+        pos = build_part("position", PartSpec("rotate_half", {"head_dim": dh, "theta": theta}))
+        pos.bind({}, Runtime(DEV, torch.float32))
+        got, want = pos.rotation_table().cpu().numpy(), P.rope_inv_freq(dh, theta)
+        assert got.dtype == np.float32 and np.allclose(got, want, rtol=2e-7, atol=0)
+
+
+@pytest.mark.parametrize("dtype, bound", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("heads, kv_heads, dh, window", [(6, 2, 48, None), (8, 2, 32, None), (4, 4, 64, 20), (4, 1, 128, None)])
+def test_attention_part(dtype, bound, heads, kv_heads, dh, window):
+    from rust_inference_amd.parts import PartSpec, Runtime, build_part
+    rng = np.random.default_rng(heads + dh)
+    rt, hidden, eps, theta = Runtime(DEV, dtype), 72, 1e-5, 30000.0
+    mixer = build_part("mixer", PartSpec("attention", {
+        "hidden": hidden, "heads": heads, "kv_heads": kv_heads, "head_dim": dh, "prefix": "a.", "qk_norm": True,
+        "eps": eps, "window": window, "position": PartSpec("rotate_half", {"head_dim": dh, "theta": theta})}))
+    w = {}
+    for name, spec in mixer.tensors().items():
+        std = 0.1 if spec.kind == "matrix" else 0.0
+        base = 1.0 if spec.kind == "gain" else 0.0
+        w[name] = torch.tensor(base + (std or 0.1) * rng.normal(size=spec.shape)).to(torch.bfloat16)
+    mixer.bind(w, rt)
+    counts = [37, 3, 70]                         # three sequences from their first token, unequal lengths
+    cache, ctx = context_for(rt, [mixer.cache_need()], counts)
+    x = t(rng.normal(size=(sum(counts), hidden)), dtype)
+    out = mixer.forward(x, ctx, cache.kv(0), ctx.page_tables[0])
+    w64 = {k: v.to(torch.float64).numpy() for k, v in w.items()}
+    cfg = {"num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": dh, "rms_norm_eps": eps,
+           "rope_theta": theta}
+    i = 0
+    for n in counts:
+        want = P.attention_block(f64(x[i:i + n]), w64, "a.", cfg, np.arange(n), window=window)
+        assert rel_to_max(f64(out[i:i + n]), want) < bound
+        i += n
+
+
+@pytest.mark.parametrize("dtype, bound", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("rows", [1, 7, 40])
+def test_swiglu_part(dtype, bound, rows):
+    from rust_inference_amd.parts import PartSpec, Runtime, build_part
+    rng = np.random.default_rng(rows)
+    ff = build_part("feed_forward", PartSpec("swiglu", {"hidden": 104, "inter": 232, "prefix": "m."}))
+    w = {n: torch.tensor(0.1 * rng.normal(size=s.shape)).to(torch.bfloat16) for n, s in ff.tensors().items()}
+    ff.bind(w, Runtime(DEV, dtype))
+    x = t(rng.normal(size=(rows, 104)), dtype)
+    w64 = {k: v.to(torch.float64).numpy() for k, v in w.items()}
+    want = P.swiglu_mlp(f64(x), w64["m.gate_proj.weight"], w64["m.up_proj.weight"], w64["m.down_proj.weight"])
+    assert rel_to_max(f64(ff.forward(x, None)), want) < bound
+
+
+# ------------------------------------------------------------------------------------------------ the toy architecture
+TOY = {"architectures": ["ToyMixForCausalLM"], "vocab_size": 130, "hidden_size": 48, "inter": 80, "heads": 4,
+       "kv_heads": 2, "head_dim": 16, "window": 24, "eps": 1e-5, "theta": 10000.0}
+
+
+def register_toy():
+    from rust_inference_amd.cache import StateNeed
+    from rust_inference_amd.config import ModelConfig, register_architecture
+    from rust_inference_amd.parts import LayerSpec, Mixer, ModelSpec, PartSpec, Run, register_part
+    from rust_inference_amd.weights import MATRIX, TensorSpec
+
+    @register_part("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """y_t = W . mean(x_0 .. x_t): the state is the running sum and the count, per sequence."""
+        def __init__(self, hidden, name):
+            self.hidden, self.name = hidden, name
+
+        def tensors(self):
+            return {self.name: TensorSpec((self.hidden, self.hidden), MATRIX)}
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.w = weights[self.name].to(rt.device, torch.float32)
+
+        def cache_need(self):
+            return StateNeed((self.hidden + 1,), torch.float32)
+
+        def forward(self, x, ctx, store, page_table):
+            out = torch.empty_like(x)
+            begin = 0
+            for slot, n in zip(ctx.slot_list, ctx.new_counts):        # a sequence's tokens are contiguous, in order
+                xs = x[begin:begin + n].float()
+                total = store[slot, :-1] + torch.cumsum(xs, 0)
+                count = store[slot, -1] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+                out[begin:begin + n] = ((total / count[:, None]) @ self.w.T).to(x.dtype)
+                store[slot, :-1], store[slot, -1] = total[-1], count[-1]
+                begin += n
+            return out
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        inter: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        window: int = 0
+        eps: float = 1e-5
+        theta: float = 1e4
+        ARCHITECTURE: ClassVar[str] = "ToyMixForCausalLM"
+        MODEL_TYPE: ClassVar[str] = "toy_mix"
+
+        @classmethod
+        def from_dict(cls, raw):
+            import dataclasses
+            return cls(**{f.name: raw[f.name] for f in dataclasses.fields(cls)})
+
+    def spec(c):
+        d = c.hidden_size
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"dim": d, "eps": c.eps, "name": name})
+
+        def ff(p):
+            return PartSpec("swiglu", {"hidden": d, "inter": c.inter, "prefix": p})
+        windowed = LayerSpec(
+            mixer_norm=norm("l0.n1"), feed_forward_norm=norm("l0.n2"), feed_forward=ff("l0.ff."),
+            mixer=PartSpec("attention", {"hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                         "prefix": "l0.attn.", "qk_norm": False, "eps": c.eps, "window": c.window,
+                                         "position": PartSpec("rotate_half", {"head_dim": c.head_dim, "theta": c.theta})}))
+        stateful = LayerSpec(mixer_norm=norm("l1.n1"), feed_forward_norm=norm("l1.n2"), feed_forward=ff("l1.ff."),
+                             mixer=PartSpec("toy_running_mean", {"hidden": d, "name": "l1.mean.weight"}))
+        unrotated = LayerSpec(
+            mixer_norm=norm("l2.n1"), feed_forward_norm=norm("l2.n2"), feed_forward=ff("l2.ff."),
+            mixer=PartSpec("attention", {"hidden": d, "heads": 2, "kv_heads": 1, "head_dim": 32, "prefix": "l2.attn.",
+                                         "qk_norm": True, "eps": c.eps, "window": None, "position": PartSpec("none")}))
+        return ModelSpec(
+            architecture="ToyMixForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
+            embedding=PartSpec("table", {"vocab": c.vocab_size, "dim": d, "name": "embed.weight"}),
+            layers=(windowed, stateful, unrotated),
+            # layer 0 runs twice with the same weights; each run has a cache entry of its own
+            schedule=(Run(0, 0), Run(1, 1), Run(0, 2), Run(2, 3)),
+            final_norm=norm("final.weight"),
+            head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": False}),
+            max_positions=512)
+
+    register_architecture("ToyMixForCausalLM", ToyConfig, spec, model_types=("toy_mix",))
+
+
+def toy_plain(w, ids):
+    """The toy model, whole sequence, no cache, from the plain parts."""
+    c = TOY
+    d = c["hidden_size"]
+    h = P.embedding(w["embed.weight"], ids)
+    pos = np.arange(len(ids))
+
+    def block(h, p, mixer):
+        r = h + mixer(P.rms_norm(h, w[p + ".n1"], c["eps"]))
+        return r + P.swiglu_mlp(P.rms_norm(r, w[p + ".n2"], c["eps"]), w[p + ".ff.gate_proj.weight"],
+                                w[p + ".ff.up_proj.weight"], w[p + ".ff.down_proj.weight"])
+
+    def windowed(x):
+        s = x.shape[0]
+        q = (x @ w["l0.attn.q_proj.weight"].T).reshape(s, c["heads"], c["head_dim"])
+        k = (x @ w["l0.attn.k_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        v = (x @ w["l0.attn.v_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        ang = P.rope_angles(pos, c["head_dim"], c["theta"])
+        o = P.attention(P.apply_rope(q, ang), P.apply_rope(k, ang), v, window=c["window"])
+        return o.reshape(s, -1) @ w["l0.attn.o_proj.weight"].T
+
+    def running_mean(x):
+        return (np.cumsum(x, 0) / np.arange(1, x.shape[0] + 1)[:, None]) @ w["l1.mean.weight"].T
+
+    def unrotated(x):
+        s = x.shape[0]
+        q = P.rms_norm((x @ w["l2.attn.q_proj.weight"].T).reshape(s, 2, 32), w["l2.attn.q_norm.weight"], c["eps"])
+        k = P.rms_norm((x @ w["l2.attn.k_proj.weight"].T).reshape(s, 1, 32), w["l2.attn.k_norm.weight"], c["eps"])
+        v = (x @ w["l2.attn.v_proj.weight"].T).reshape(s, 1, 32)
+        return P.attention(q, k, v).reshape(s, -1) @ w["l2.attn.o_proj.weight"].T
+
+    h = block(h, "l0", windowed)
+    h = block(h, "l1", running_mean)
+    h = block(h, "l0", windowed)
+    h = block(h, "l2", unrotated)
+    return P.rms_norm(h, w["final.weight"], c["eps"]) @ w["head.weight"].T
+
+
+@pytest.fixture(scope="module")
+def toy_dir(tmp_path_factory):
+    register_toy()
+    from rust_inference_amd.weights import write_random_model
+    return write_random_model(str(tmp_path_factory.mktemp("toy") / "m"), TOY, seed=7, dtype=torch.float32,
+                              matrix_std=0.15)
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_toy_architecture_builds_and_steps_through_the_unchanged_engine(toy_dir, dtype_name):
+    from rust_inference_amd.cache import KVNeed, StateNeed
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from safetensors import safe_open
+    model = load_model(toy_dir, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
+    needs = model.cache_needs()
+    assert needs[0] == needs[2] == KVNeed(2, 16, 24) and isinstance(needs[1], StateNeed) and needs[3] == KVNeed(1, 32, None)
+    with safe_open(os.path.join(toy_dir, "model.safetensors"), framework="pt") as f:
+        w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
+    rng = np.random.default_rng(8)
+    reqs = {f"r{i}": [int(x) for x in rng.integers(0, TOY["vocab_size"], n)] for i, n in enumerate([70, 9, 41, 100])}
+    results = {}
+    for plan_name, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 32)),
+                             ("batches", plans.unequal_batches([
+                                 {k: (v, max(1, len(v) - 20)) for k, v in list(reqs.items())[:2]},
+                                 {k: (v, max(1, len(v) - 33)) for k, v in list(reqs.items())[2:]}]))):
+        engine = engine_for_trace(model, plans.max_live_tokens(steps))
+        assert len(engine.cache.groups) == 2                     # the windowed entries and the full one: own storage
+        player, outs = Replayer(engine), {}
+        for s in steps:
+            logits = player.feed(s)
+            if logits is not None:
+                outs[s["step"]] = logits.cpu().numpy()
+        engine.cache.check_consistent()
+        results[plan_name] = plans.collect(steps, lambda i: outs[i], TOY["vocab_size"])
+        for rid, toks in reqs.items():
+            assert_logits_close(results[plan_name][rid], toy_plain(w, toks), dtype_name, f"toy, {plan_name}, {rid}")
+    # a window's pages go back while a sequence is still running: fewer pages held than a full group would
+    engine = engine_for_trace(model, 128)
+    slot = engine.cache.acquire()
+    from rust_inference_amd.engine import StepEntry
+    engine.step([StepEntry(slot, reqs["r3"], "last")])
+    windowed = next(g for g in engine.cache.groups if g.need.window)
+    full = next(g for g in engine.cache.groups if not g.need.window)
+    assert len(windowed.pool.pages_of(slot)) == 2 and len(full.pool.pages_of(slot)) == 4
