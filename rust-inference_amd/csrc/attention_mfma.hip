@@ -20,7 +20,8 @@
 // second product rounded to bfloat16 and the running sum is taken of the rounded weights, so they
 // still sum to one.
 //
-// Prefill: one wavefront per tile of tokens, walking the sequence's pages in order.  Decode (one new
+// Prefill: one wavefront per tile of tokens, walking the sequence's pages in order; the four
+// wavefronts of a workgroup share the pages through LDS.  Decode (one new
 // token per sequence): the keys are cut into chunks of 256 at fixed places, one workgroup per chunk
 // (its eight wavefronts take one page each), partial results go to a workspace and a second kernel
 // joins them in chunk order.  Neither order depends on the batch or on how tokens were cut.
@@ -74,9 +75,15 @@ struct Columns {
     int qpos[NT], lo[NT];         // the column's query position (-1: no such column) and first visible key
 };
 
+// One page for NT tiles of columns, in two halves so that the key fragments and the value fragments
+// need not be in registers at the same time.  `open` says that every key of the page is visible to
+// every column of this wavefront (the usual case away from the diagonal and the window's edge): no
+// mask then.  The running sum l stays per lane (the lane's own eight keys of every page) and is added
+// up over the four lane groups once at the end; the running maximum is shared by a column's lanes at
+// every page.
 template <int DH, int NT>
-__device__ __forceinline__ void process_page(Columns<DH, NT>& c, const PageFrags<DH>& f, int page, int lane,
-                                             float scale_log2) {
+__device__ __forceinline__ void scores_and_weights(Columns<DH, NT>& c, const Frag (&kf)[2][DH / 32], Frag (&p)[NT],
+                                                   int page, int lane, float scale_log2, bool open) {
     const int jg = lane >> 4;
     const int key0 = page * PAGE + jg * 8;
 #pragma unroll
@@ -84,40 +91,65 @@ __device__ __forceinline__ void process_page(Columns<DH, NT>& c, const PageFrags
         floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks) {
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[0][ks].v, c.q[j][ks].v, s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[1][ks].v, c.q[j][ks].v, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][ks].v, c.q[j][ks].v, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][ks].v, c.q[j][ks].v, s1, 0, 0, 0);
         }
         float s[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-        float mx = -INFINITY;
+        if (!open) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int key = key0 + e;
-            s[e] = (key <= c.qpos[j] && key >= c.lo[j]) ? s[e] * scale_log2 : -INFINITY;
-            mx = fmaxf(mx, s[e]);
+            for (int e = 0; e < 8; ++e) {
+                const int key = key0 + e;
+                if (key > c.qpos[j] || key < c.lo[j]) s[e] = -INFINITY;
+            }
         }
+        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
         mx = fmaxf(mx, __shfl_xor(mx, 16, RI_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, RI_WAVE));
-        const float m_new = fmaxf(c.m[j], mx);
+        const float m_new = fmaxf(c.m[j], mx * scale_log2);        // the scale is positive: max commutes with it
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;     // a column that has seen no key yet
-        const float corr = exp2f(c.m[j] - m_safe);                  // 0 while m is -inf
-        Frag p;
         float ps = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const bf16_t a = f32_to_bf16(exp2f(s[2 * e] - m_safe));
-            const bf16_t b = f32_to_bf16(exp2f(s[2 * e + 1] - m_safe));
-            p.w[e] = (uint32_t)a | ((uint32_t)b << 16);
-            ps += bf16_to_f32(a) + bf16_to_f32(b);
+            const float a = __builtin_amdgcn_exp2f(fmaf(s[2 * e], scale_log2, -m_safe));
+            const float b = __builtin_amdgcn_exp2f(fmaf(s[2 * e + 1], scale_log2, -m_safe));
+            p[j].w[e] = pack_bf16x2(a, b);
+            ps += a + b;
         }
-        ps += __shfl_xor(ps, 16, RI_WAVE);
-        ps += __shfl_xor(ps, 32, RI_WAVE);
-        c.l[j] = c.l[j] * corr + ps;
-        c.m[j] = m_new;
+        if (__any(m_new != c.m[j])) {                               // a new maximum somewhere in the wavefront
+            const float corr = __builtin_amdgcn_exp2f(c.m[j] - m_safe);      // 0 while m is -inf
+            c.l[j] *= corr;
 #pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) {
-            c.o[j][dt] *= corr;
-            c.o[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt].v, p.v, c.o[j][dt], 0, 0, 0);
+            for (int dt = 0; dt < DH / 16; ++dt) c.o[j][dt] *= corr;
+            c.m[j] = m_new;
         }
+        c.l[j] += ps;
+    }
+}
+
+template <int DH, int NT>
+__device__ __forceinline__ void weighted_values(Columns<DH, NT>& c, const Frag (&vf)[DH / 16], const Frag (&p)[NT]) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt)
+            c.o[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, p[j].v, c.o[j][dt], 0, 0, 0);
+}
+
+template <int DH, int NT>
+__device__ __forceinline__ void process_page(Columns<DH, NT>& c, const PageFrags<DH>& f, int page, int lane,
+                                             float scale_log2, bool open) {
+    Frag p[NT];
+    scores_and_weights<DH, NT>(c, f.k, p, page, lane, scale_log2, open);
+    weighted_values<DH, NT>(c, f.v, p);
+}
+
+// The columns' sums over all their lanes: call once after the last page.
+template <int DH, int NT>
+__device__ __forceinline__ void finish_columns(Columns<DH, NT>& c) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        c.l[j] += __shfl_xor(c.l[j], 16, RI_WAVE);
+        c.l[j] += __shfl_xor(c.l[j], 32, RI_WAVE);
     }
 }
 
@@ -137,22 +169,68 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
 }
 
 // ------------------------------------------------------------------ prefill
+// A workgroup of four wavefronts takes 4 * (16 NT / group) consecutive tokens of one sequence and one kv
+// head.  The pages of keys and values go through LDS, fetched once for all four wavefronts and
+// double-buffered: while a page is in work the next one is on its way from global memory.  In LDS a key
+// row is padded to head_dim + 8 elements and a value row (one channel, 32 tokens) to 40, which spreads
+// the 16-byte fragment reads over all banks; the key rows of a page are stored in the order the two
+// MFMA tiles take them (rows {0-3, 8-11, 16-19, 24-27}, then the rest).
+template <int DH>
+struct LdsPage {
+    static constexpr int KS = DH + 8;                        // key row stride, elements
+    static constexpr int VS = PAGE + 8;                      // value row stride, elements
+    static constexpr int CHUNKS = 4 * DH;                    // 16-byte pieces of a key page (and of a value page)
+    static constexpr int PER_THREAD = (CHUNKS + 255) / 256;
+};
+
+template <int DH>
+__device__ __forceinline__ void stage_store_one(bf16_t* k_lds, bf16_t* v_lds, int c, const uint4& k, const uint4& v) {
+    const int krow = c / (DH / 8), kcol = c % (DH / 8);                  // key row 0..31, 16-byte column
+    const int w = krow & 7;
+    const int lrow = (w >= 4 ? 16 : 0) + (krow >> 3) * 4 + (w & 3);
+    *reinterpret_cast<uint4*>(k_lds + lrow * LdsPage<DH>::KS + kcol * 8) = k;
+    const int vrow = c / 4, vcol = c % 4;                                // channel 0..DH-1, 16-byte column
+    *reinterpret_cast<uint4*>(v_lds + vrow * LdsPage<DH>::VS + vcol * 8) = v;
+}
+
+template <int DH>
+__device__ __forceinline__ void key_frags_from_lds(Frag (&kf)[2][DH / 32], const bf16_t* k_lds, int lane) {
+    const int i = lane & 15, jg = lane >> 4;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks)
+            kf[kt][ks].u = *reinterpret_cast<const uint4*>(k_lds + (kt * 16 + i) * LdsPage<DH>::KS + ks * 32 + jg * 8);
+}
+
+template <int DH>
+__device__ __forceinline__ void value_frags_from_lds(Frag (&vf)[DH / 16], const bf16_t* v_lds, int lane) {
+    const int i = lane & 15, jg = lane >> 4;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt)
+        vf[dt].u = *reinterpret_cast<const uint4*>(v_lds + (dt * 16 + i) * LdsPage<DH>::VS + jg * 8);
+}
+
 template <int DH, int NT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv, int q_stride,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                          const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ tok_pos,
                          const int32_t* __restrict__ page_table, int table_width, int heads, int kv_heads,
                          int window, float scale_log2) {
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][PAGE * LdsPage<DH>::KS];
+    __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][DH * LdsPage<DH>::VS];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.y, kvh = blockIdx.z;
     const int group = heads / kv_heads;
     const int tile_tokens = (16 * NT) / group;               // tokens per wavefront
     const int t_end = cu_seqlens[b + 1];
-    const int t0 = cu_seqlens[b] + (blockIdx.x * 4 + wave) * tile_tokens;
-    if (t0 >= t_end) return;                                 // the whole wavefront leaves; no barrier below
-    const int nt = min(tile_tokens, t_end - t0);
+    // the last tokens of a sequence see the most keys: their workgroups are launched first
+    const int t_wg = cu_seqlens[b] + (int)(gridDim.x - 1 - blockIdx.x) * 4 * tile_tokens;
+    if (t_wg >= t_end) return;                               // the whole workgroup leaves
+    const int t0 = t_wg + wave * tile_tokens;
+    const int nt = max(0, min(tile_tokens, t_end - t0));     // a wavefront without tokens still helps to fetch
 
     Columns<DH, NT> c;
     init_columns<DH, NT>(c);
@@ -170,20 +248,69 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
             for (int ks = 0; ks < DH / 32; ++ks) c.q[j][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
         }
     }
-    const int first_pos = tok_pos[t0], last_pos = tok_pos[t0 + nt - 1];
-    const int p_lo = window > 0 ? max(0, first_pos - window + 1) / PAGE : 0;
-    const int p_hi = last_pos / PAGE;
+    // pages the workgroup walks, and the part of them this wavefront's tokens can see
+    const int wg_first = tok_pos[t_wg], wg_last = tok_pos[min(t_end, t_wg + 4 * tile_tokens) - 1];
+    const int p_lo = window > 0 ? max(0, wg_first - window + 1) / PAGE : 0;
+    const int p_hi = wg_last / PAGE;
+    const int my_hi = nt > 0 ? tok_pos[t0 + nt - 1] / PAGE : -1;
+    const int my_lo = (nt > 0 && window > 0) ? max(0, tok_pos[t0] - window + 1) / PAGE : 0;
+    // a page is open to the whole wavefront when its last key is at or before the first token's position
+    // and its first key inside the last token's window; wavefronts with unused columns mask always
+    const bool full = nt * group == 16 * NT;
+    const int min_qpos = (nt > 0 && full) ? tok_pos[t0] : -1;
+    const int max_lo = (nt > 0 && window > 0) ? max(0, tok_pos[t0 + nt - 1] - window + 1) : 0;
     const int32_t* table = page_table + (long)b * table_width;
 
-    PageFrags<DH> fa, fb;                                    // the page in work and the one being fetched
-    load_page<DH>(fa, k_pages, v_pages, table[p_lo], kv_heads, kvh, lane);
-    for (int p = p_lo; p <= p_hi; p += 2) {
-        if (p + 1 <= p_hi) load_page<DH>(fb, k_pages, v_pages, table[p + 1], kv_heads, kvh, lane);
-        process_page<DH, NT>(c, fa, p, lane, scale_log2);
-        if (p + 1 > p_hi) break;
-        if (p + 2 <= p_hi) load_page<DH>(fa, k_pages, v_pages, table[p + 2], kv_heads, kvh, lane);
-        process_page<DH, NT>(c, fb, p + 1, lane, scale_log2);
+    // What this thread carries of a page on its way from global memory to LDS: up to two 16-byte pieces
+    // of the key page and of the value page, in plain registers.
+    static_assert(LdsPage<DH>::PER_THREAD <= 2, "a page is at most two pieces per thread");
+    constexpr bool TWO = LdsPage<DH>::PER_THREAD > 1;
+    const int c0 = threadIdx.x;
+    const bool has0 = c0 < LdsPage<DH>::CHUNKS;
+    uint4 sk0 = make_uint4(0, 0, 0, 0), sk1 = sk0, sv0 = sk0, sv1 = sk0;
+#define RI_STAGE_LOAD(PHYS)                                                                          \
+    {                                                                                                \
+        const long base_ = ((long)(PHYS) * kv_heads + kvh) * (long)(PAGE * DH);                      \
+        if (has0) {                                                                                  \
+            sk0 = *reinterpret_cast<const uint4*>(k_pages + base_ + c0 * 8);                         \
+            sv0 = *reinterpret_cast<const uint4*>(v_pages + base_ + c0 * 8);                         \
+        }                                                                                            \
+        if (TWO) {                                                                                   \
+            sk1 = *reinterpret_cast<const uint4*>(k_pages + base_ + (c0 + 256) * 8);                 \
+            sv1 = *reinterpret_cast<const uint4*>(v_pages + base_ + (c0 + 256) * 8);                 \
+        }                                                                                            \
     }
+#define RI_STAGE_STORE(BUF)                                                                          \
+    {                                                                                                \
+        if (has0) stage_store_one<DH>(k_lds[BUF], v_lds[BUF], c0, sk0, sv0);                         \
+        if (TWO) stage_store_one<DH>(k_lds[BUF], v_lds[BUF], c0 + 256, sk1, sv1);                    \
+    }
+    RI_STAGE_LOAD(table[p_lo]);
+    RI_STAGE_STORE(0);
+    __syncthreads();
+    for (int p = p_lo; p <= p_hi; ++p) {
+        const int buf = (p - p_lo) & 1;
+        if (p < p_hi) RI_STAGE_LOAD(table[p + 1]);
+        if (p >= my_lo && p <= my_hi) {
+            const bool open = p * PAGE + PAGE - 1 <= min_qpos && p * PAGE >= max_lo;
+            Frag w[NT];
+            {
+                Frag kf[2][DH / 32];
+                key_frags_from_lds<DH>(kf, k_lds[buf], lane);
+                scores_and_weights<DH, NT>(c, kf, w, p, lane, scale_log2, open);
+            }
+            {
+                Frag vf[DH / 16];
+                value_frags_from_lds<DH>(vf, v_lds[buf], lane);
+                weighted_values<DH, NT>(c, vf, w);
+            }
+        }
+        if (p < p_hi) RI_STAGE_STORE(buf ^ 1);
+        __syncthreads();                                     // the next page is in place; this one may be overwritten
+    }
+#undef RI_STAGE_LOAD
+#undef RI_STAGE_STORE
+    finish_columns<DH, NT>(c);
 
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -236,7 +363,8 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
     }
-    if (has) process_page<DH, 1>(c, f, page, lane, scale_log2);
+    if (has) process_page<DH, 1>(c, f, page, lane, scale_log2, false);
+    finish_columns<DH, 1>(c);
 
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt)

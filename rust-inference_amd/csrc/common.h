@@ -15,11 +15,17 @@ typedef uint16_t bf16_t;   // bfloat16 carried as its bits
 __device__ __forceinline__ float bf16_to_f32(bf16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
 // Round to nearest, ties to even; a NaN stays a quiet NaN (the reference: src/dtype.rs:82-89).
+// gfx950 converts in hardware (v_cvt_pk_bf16_f32) with exactly this rounding.
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+    const __bf16 h = (__bf16)f;
+    return *reinterpret_cast<const bf16_t*>(&h);
+}
+
+// Two floats to two bfloat16 in one 32-bit word, the first in the low half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+    const bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+    return *reinterpret_cast<const uint32_t*>(&v);
 }
 
 __device__ __forceinline__ float to_f32(float v) { return v; }
