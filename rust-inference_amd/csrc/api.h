@@ -75,6 +75,12 @@ int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, 
 int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
                         void* stream);
 
+// The same with the weights packed ahead of time into MFMA tiles: [ceil(n/16)][ceil(k/32)][64 lanes][8],
+// lane l of a tile holding row l % 16, k 8 * (l / 16)..+8, zero beyond n and k; with swiglu the up matrix's
+// ceil(n/16) row tiles follow the gate's.
+int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
+                               int swiglu, void* stream);
+
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);
 

@@ -75,6 +75,94 @@ gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
     }
 }
 
+// The same product with the weights packed for the matrix cores ahead of time: the matrix is cut into
+// tiles of 16 rows by 32 k, each tile stored as the 1 KB that one MFMA A operand is (lane l's 16 bytes:
+// row l % 16, k 8 * (l / 16) ..+8), tiles of one row block consecutive in k.  A wavefront's loads are
+// then whole contiguous kilobytes, which is what the memory system streams fastest.
+// packed: [row_tiles][k_tiles][64 lanes][8]; for SwiGLU the up matrix's tiles follow the gate's.
+template <bool SWIGLU, typename TO>
+__global__ void __launch_bounds__(SK_WAVES * 64)
+gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked,
+                          int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset) {
+    __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, jg = lane >> 4;
+    const int nt = blockIdx.x;
+    const bool x_ok = i < M;
+    const int kt_begin = wave * tiles_per_wave, kt_end = min(k_tiles, kt_begin + tiles_per_wave);
+    const bf16_t* wp = wpacked + ((size_t)nt * k_tiles * 64 + lane) * 8;
+    const bf16_t* up = SWIGLU ? wpacked + ((size_t)(up_tile_offset + nt) * k_tiles * 64 + lane) * 8 : nullptr;
+    const bf16_t* xp = x + (size_t)(x_ok ? i : 0) * K + jg * 8;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
+    for (int kt = kt_begin; kt < kt_end; kt += SK_CHUNK) {
+        Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];
+#pragma unroll
+        for (int c = 0; c < SK_CHUNK; ++c) {
+            const bool ok = kt + c < kt_end;
+            wf[c].u = ok ? *reinterpret_cast<const uint4*>(wp + (size_t)(kt + c) * 512) : zero;
+            if (SWIGLU) uf[c].u = ok ? *reinterpret_cast<const uint4*>(up + (size_t)(kt + c) * 512) : zero;
+            // the packed matrix is zero beyond K; x is not padded
+            xf[c].u = (ok && x_ok && (kt + c) * 32 + jg * 8 < K) ? *reinterpret_cast<const uint4*>(xp + (kt + c) * 32)
+                                                                 : zero;
+        }
+#pragma unroll
+        for (int c = 0; c < SK_CHUNK; ++c) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
+            if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        red[0][wave][r][lane] = acc[r];
+        if (SWIGLU) red[1][wave][r][lane] = accu[r];
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < 256) {
+        const int ln = t & 63, r = t >> 6;
+        float g = 0.f, u = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < SK_WAVES; ++wv) {
+            g += red[0][wv][r][ln];
+            if (SWIGLU) u += red[1][wv][r][ln];
+        }
+        const int n = nt * 16 + 4 * (ln >> 4) + r, m = ln & 15;
+        if (m < M && n < N) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_sk(g) * u : g);
+    }
+}
+
+extern "C" int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
+                                          int k, int swiglu, void* stream) {
+    RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_packed_bf16: %d rows of x, this kernel takes 1 to 16", m);
+    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_packed_bf16: out dtype %d", out_dtype);
+    const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
+    const int tiles_per_wave = (k_tiles + SK_WAVES - 1) / SK_WAVES;
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)wpacked;
+    if (swiglu) {
+        if (out_dtype == RI_F32)
+            gemm_skinny_packed_kernel<true, float><<<row_tiles, SK_WAVES * 64, 0, s>>>(
+                (float*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+        else
+            gemm_skinny_packed_kernel<true, bf16_t><<<row_tiles, SK_WAVES * 64, 0, s>>>(
+                (bf16_t*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+    } else {
+        if (out_dtype == RI_F32)
+            gemm_skinny_packed_kernel<false, float><<<row_tiles, SK_WAVES * 64, 0, s>>>(
+                (float*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, 0);
+        else
+            gemm_skinny_packed_kernel<false, bf16_t><<<row_tiles, SK_WAVES * 64, 0, s>>>(
+                (bf16_t*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, 0);
+    }
+    RI_LAUNCH_CHECK("gemm_skinny_packed_bf16");
+    return 0;
+}
+
 extern "C" int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
                                    int swiglu, void* stream) {
     RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_bf16: %d rows of x, this kernel takes 1 to 16", m);

@@ -194,6 +194,25 @@ __global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ y, int 
     from_f32(out + e, silu(to_f32(row[i])) * to_f32(row[inter + i]));
 }
 
+// Eight bfloat16 elements per thread with 16-byte loads and stores, for inter a multiple of 8.
+__global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y, int inter8, long total8) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total8) return;
+    const long t = e / inter8;
+    const int i = (int)(e - t * inter8);
+    const uint4 g = *reinterpret_cast<const uint4*>(y + (t * 2 * inter8 + i) * 8);
+    const uint4 u = *reinterpret_cast<const uint4*>(y + (t * 2 * inter8 + inter8 + i) * 8);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float a = silu(__uint_as_float(gw[k] << 16)) * __uint_as_float(uw[k] << 16);
+        const float b = silu(__uint_as_float(gw[k] & 0xFFFF0000u)) * __uint_as_float(uw[k] & 0xFFFF0000u);
+        o[k] = pack_bf16x2(a, b);
+    }
+    *reinterpret_cast<uint4*>(out + e * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream) {
     RI_REQUIRE(tokens > 0 && inter > 0, "swiglu: tokens %d, inter %d", tokens, inter);
     const long total = (long)tokens * inter;
@@ -202,6 +221,9 @@ extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int in
     hipStream_t s = (hipStream_t)stream;
     if (dtype == RI_F32)
         swiglu_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)y, inter, total);
+    else if (dtype == RI_BF16 && inter % 8 == 0)
+        swiglu_bf16x8_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y,
+                                                                                  inter / 8, total / 8);
     else if (dtype == RI_BF16)
         swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, inter, total);
     else

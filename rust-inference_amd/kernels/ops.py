@@ -37,6 +37,7 @@ _SIGNATURES = {
     "ri_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_float,
                   c_void_p],
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -272,4 +273,36 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16,
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _call("ri_gemm_skinny_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
           _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
+    return out
+
+
+def pack_for_mfma(w: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
+    """A bfloat16 weight ``[N, K]`` cut into MFMA A-operand tiles: ``[ceil(N/16), ceil(K/32), 64, 8]``, lane
+    ``l`` of a tile holding row ``l % 16`` and ``k = 8 * (l // 16) ..+8``, zero beyond N and K.  With
+    ``swiglu`` the gate half and the up half of ``[2 N, K]`` are packed one after the other."""
+    if swiglu:
+        half = w.shape[0] // 2
+        return torch.cat([pack_for_mfma(w[:half]), pack_for_mfma(w[half:])], 0)
+    n, k = w.shape
+    n16, k32 = -(-n // 16) * 16, -(-k // 32) * 32
+    if (n16, k32) != (n, k):
+        padded = torch.zeros((n16, k32), dtype=w.dtype, device=w.device)
+        padded[:n, :k] = w
+        w = padded
+    tiles = w.view(n16 // 16, 16, k32 // 32, 4, 8).permute(0, 2, 3, 1, 4)      # [row tile, k tile, k group, row, 8]
+    return tiles.reshape(n16 // 16, k32 // 32, 64, 8).contiguous()
+
+
+def gemm_skinny_packed_bf16(x: torch.Tensor, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16,
+                            swiglu: bool = False) -> torch.Tensor:
+    """``x @ w.T`` for up to 16 bfloat16 rows with ``w`` packed by ``pack_for_mfma``; ``n`` is the number of
+    output columns (rows of w; of its gate half with ``swiglu``)."""
+    m, k = x.shape
+    row_tiles = -(-n // 16)
+    want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
+    if tuple(wpacked.shape) != want:
+        raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _call("ri_gemm_skinny_packed_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
+          _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), _stream())
     return out

@@ -60,7 +60,7 @@ class GroupedQueryAttention(Mixer):
         p = self.prefix
         qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
         self.w_qkv = rt.place_matrix(qkv)
-        self.w_o = rt.place_matrix(weights[p + "o_proj.weight"])
+        self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]))
         self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
         self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
         self.position.bind(weights, rt)
@@ -75,7 +75,7 @@ class GroupedQueryAttention(Mixer):
         ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
                                   ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
                                   self.heads, self.kv_heads, self.head_dim)
-        return rt.linear(self.attend(qkv, ctx, store, page_table), self.w_o)
+        return rt.linear_packed(self.attend(qkv, ctx, store, page_table), self.w_o)
 
     def attend(self, qkv, ctx, store, page_table):
         """The attention kernel that fits the step: matrix cores for bfloat16 (one new token per

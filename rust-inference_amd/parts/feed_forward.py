@@ -7,7 +7,6 @@ from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part
-from .runtime import GEMV_MAX_ROWS
 
 
 @register_part("feed_forward", "swiglu")
@@ -30,13 +29,11 @@ class SwiGLU(FeedForward):
     def bind(self, weights, rt):
         self.rt = rt
         p = self.prefix
-        self.w_gate_up = rt.place_matrix(torch.cat([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], 0))
+        gate_up = rt.place_matrix(torch.cat([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], 0))
+        self.w_gate_up = rt.pack(gate_up, swiglu=True)
         self.w_down = rt.place_matrix(weights[p + "down_proj.weight"])
 
     def forward(self, x, ctx):
         rt = self.rt
-        if rt.dtype == torch.bfloat16 and x.shape[0] <= GEMV_MAX_ROWS and self.hidden % 8 == 0:
-            a = ops.gemv_bf16(x, self.w_gate_up, torch.bfloat16, swiglu=True)      # activation in the epilogue
-        else:
-            a = ops.swiglu(rt.linear(x, self.w_gate_up))
+        a = rt.linear_packed(x, self.w_gate_up)        # the activation is in the epilogue of the decode-size kernels
         return rt.linear(a, self.w_down)

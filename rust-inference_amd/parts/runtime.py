@@ -8,13 +8,27 @@ from ..errors import KernelError, ShapeError
 from ..kernels import ops
 
 # Which product kernel runs, by the number of rows of x (measured on MI355X at Qwen3-8B sizes with the
-# weights streamed from HBM): the one-wavefront-per-row kernel is fastest for one or two rows
-# (5.1 to 5.5 TB/s on the large matrices); from three rows on it is bound by its vector
-# arithmetic and the vendor library's product is faster (4.2 to 4.9 TB/s); the matrix-core kernel of
-# this library wins only on matrices up to 4096 x 4096.
+# weights streamed from HBM, every variant replayed as a graph):
+#   1-2 rows   one wavefront per weight row (gemv_bf16): 5.1 to 5.5 TB/s on the large matrices;
+#              from three rows on it is bound by its vector arithmetic.
+#   3-16 rows  the matrix-core kernel on weights packed into MFMA tiles ahead of time, where a part
+#              asked for the packed copy (the attention output matrix and the fused gate|up matrix:
+#              4.5 TB/s with the activation in the epilogue against 4.2 TB/s for the library's product
+#              plus an activation kernel; 3.0 against 2.2 TB/s on the 4096 x 4096 matrix).  Elsewhere
+#              the vendor library's product is as fast or faster (4.5 to 4.9 TB/s) and is used.
+#   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
 GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
-SKINNY_MAX_SIDE = 4096
+
+
+class PackedWeight:
+    """A bfloat16 weight as the library product wants it (row-major) and, for decode-size products,
+    packed into MFMA tiles."""
+
+    def __init__(self, w: torch.Tensor, packed: torch.Tensor | None, swiglu: bool):
+        self.w, self.packed, self.swiglu = w, packed, swiglu
+        self.n = w.shape[0] // 2 if swiglu else w.shape[0]
+        self.k = w.shape[1]
 
 
 class Runtime:
@@ -57,9 +71,26 @@ class Runtime:
         m, k = x.shape
         if m <= GEMV_MAX_ROWS and k % 8 == 0:
             return ops.gemv_bf16(x, w, out_dtype)
-        if m <= SKINNY_MAX_ROWS and k % 8 == 0 and k <= SKINNY_MAX_SIDE and w.shape[0] <= SKINNY_MAX_SIDE:
-            return ops.gemm_skinny_bf16(x, w, out_dtype)
         return self._library_mm(x, w, out_dtype)
+
+    def pack(self, w: torch.Tensor, swiglu: bool = False) -> PackedWeight:
+        """A placed weight with its packed copy for decode-size products (bfloat16 compute only)."""
+        if self.dtype != torch.bfloat16 or w.shape[1] % 8:
+            return PackedWeight(w, None, swiglu)
+        return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
+
+    def linear_packed(self, x: torch.Tensor, pw: PackedWeight, out_dtype=None) -> torch.Tensor:
+        """``x @ w.T`` (or ``silu(x @ gate.T) * (x @ up.T)`` for a fused gate|up weight) with the kernel
+        that fits the number of rows."""
+        out_dtype = out_dtype or self.dtype
+        m = x.shape[0]
+        if self.dtype == torch.bfloat16 and pw.k % 8 == 0:
+            if m <= GEMV_MAX_ROWS:
+                return ops.gemv_bf16(x, pw.w, out_dtype, swiglu=pw.swiglu)
+            if m <= SKINNY_MAX_ROWS and pw.packed is not None:
+                return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
+        y = self.linear(x, pw.w, None if pw.swiglu else out_dtype)
+        return ops.swiglu(y) if pw.swiglu else y
 
     def _library_mm(self, x, w, out_dtype):
         # The reference hands every product to a vendor library (src/cuda/mod.rs:186-232);

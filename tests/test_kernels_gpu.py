@@ -318,13 +318,30 @@ def test_gemm_skinny_bf16(ops, m, n, k):
                            ops.gemm_skinny_bf16(x[m - 1:].contiguous(), w, torch.float32))
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("n, k", [(37, 584), (100, 96), (4096, 4096), (50, 12288), (320, 104)])
+def test_gemm_skinny_packed_bf16(ops, m, n, k):
+    rng = np.random.default_rng(m + n)
+    x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
+    want = f64(x) @ f64(w).T
+    packed = ops.pack_for_mfma(w)
+    close(ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32), want, 3e-6, "packed skinny product")
+    # the same sums in the same order as the unpacked kernel: bit for bit
+    assert torch.equal(ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32), ops.gemm_skinny_bf16(x, w, torch.float32))
+    wgu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
+    y = f64(x) @ f64(wgu).T
+    close(ops.gemm_skinny_packed_bf16(x, ops.pack_for_mfma(wgu, swiglu=True), n, torch.bfloat16, swiglu=True),
+          P.silu(y[:, :n]) * y[:, n:], 5e-3, "packed, with swiglu")
+
+
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 1e-6), (torch.bfloat16, 5e-3)])
 def test_swiglu(ops, dtype, rel):
     assert f64(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])))[0, 0] == 0.0                 # src/ops/elementwise.rs:59-70
     close(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])), [[0.0, 6.0 / (1.0 + np.exp(-2.0))]], 1e-6)
     rng = np.random.default_rng(3)
-    y = t(rng.normal(size=(5, 2 * 333)) * 3, dtype)
-    close(ops.swiglu(y), P.silu(f64(y)[:, :333]) * f64(y)[:, 333:], rel, "swiglu")
+    for inter in (333, 232, 1000):                 # odd, and multiples of 8 (the 16-byte form)
+        y = t(rng.normal(size=(5, 2 * inter)) * 3, dtype)
+        close(ops.swiglu(y), P.silu(f64(y)[:, :inter]) * f64(y)[:, inter:], rel, f"swiglu, {inter}")
 
 
 def test_argmax(ops):
