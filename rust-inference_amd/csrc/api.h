@@ -62,6 +62,15 @@ int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q
                              const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
                              int kv_heads, int head_dim, int page_size, int window, float scale, void* stream);
 
+// The decode attention of a layer from the raw fused projection (which is not changed): per-head norm (gains
+// may be NULL) and rotation (inv_freq may be NULL) of the new token's q and k, its k and v into their pages
+// and attention in chunks of 256 keys in one kernel, the join in a second.
+int ri_attention_decode_fused_bf16(void* out, float* workspace, const void* qkv, int q_stride, const float* q_gain,
+                                   const float* k_gain, float eps, const float* inv_freq, void* k_pages,
+                                   void* v_pages, const int32_t* tok_pos, const int32_t* page_table, int table_width,
+                                   int seqs, int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
+                                   int window, float scale, void* stream);
+
 // out[M, N] (float32) = x[M, K] (float32) . w[N, K]^T, w float32 or bfloat16; true 32-bit arithmetic.
 int ri_gemm_f32(float* out, const float* x, const void* w, int w_dtype, int m, int n, int k, void* stream);
 

@@ -419,6 +419,161 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws,
     out[((long)tok * heads + h) * DH + d] = f32_to_bf16(acc / l);
 }
 
+// ------------------------------------------------------------------ decode, everything in one kernel
+// The decode step's attention from the raw projection: per-head RMSNorm and rotation of the new token's q
+// and k, the write of its k and v into their page, and the attention over chunks of 256 keys, in one
+// kernel; the join of the chunks follows as a second one.  Every workgroup norms and rotates the group's
+// queries for itself (a few hundred elements); the workgroup whose chunk holds the new token's position
+// also makes the new key and value, stores them for later steps and patches them into the fragments it
+// has just read from the page (the page in memory does not have them yet).  (Joining inside the same
+// kernel, by the workgroup that finishes last, was tried: the device-wide fences it needs write the
+// whole L2 back and cost many times what the second launch costs.)
+template <int DH>
+__device__ __forceinline__ void norm_rotate_head(bf16_t* dst_lds, const bf16_t* __restrict__ x,
+                                                 const float* __restrict__ gain, float eps,
+                                                 const float* __restrict__ inv_freq, int pos, int lane) {
+    constexpr int HALF = DH / 2;
+    float x1 = 0.f, x2 = 0.f, ss = 0.f;                      // DH <= 128: one pair per lane
+    if (lane < HALF) {
+        x1 = bf16_to_f32(x[lane]);
+        x2 = bf16_to_f32(x[lane + HALF]);
+        ss = x1 * x1 + x2 * x2;
+    }
+    if (gain) {
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)DH + eps);
+        if (lane < HALF) { x1 = x1 * inv * gain[lane]; x2 = x2 * inv * gain[lane + HALF]; }
+    }
+    if (lane < HALF) {
+        if (inv_freq) {
+            float sn, cs;
+            sincosf((float)pos * inv_freq[lane], &sn, &cs);
+            const float a = x1 * cs - x2 * sn, b = x2 * cs + x1 * sn;
+            x1 = a; x2 = b;
+        }
+        dst_lds[lane] = f32_to_bf16(x1);
+        dst_lds[lane + HALF] = f32_to_bf16(x2);
+    }
+}
+
+template <int DH>
+__global__ void __launch_bounds__(DECODE_WAVES * 64)
+attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ q_gain,
+                         const float* __restrict__ k_gain, float eps, const float* __restrict__ inv_freq,
+                         bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages,
+                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                         int heads, int kv_heads, int window, float scale_log2, int max_chunks) {
+    static_assert(DH <= 128, "one (d, d + DH/2) pair per lane");
+    __shared__ float o_lds[DECODE_WAVES][DH * 17];
+    __shared__ float ml_lds[DECODE_WAVES][2][16];
+    __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][DH];
+    __shared__ __attribute__((aligned(16))) bf16_t knew[DH];
+    __shared__ __attribute__((aligned(16))) bf16_t vnew[DH];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int chunk = blockIdx.x, b = blockIdx.y, kvh = blockIdx.z;
+    const int group = heads / kv_heads;
+    const int qpos = tok_pos[b];                             // token b is sequence b's one new token
+    const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
+    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
+    const bool owner = chunk == qpos / DECODE_CHUNK;         // this chunk holds the new token's position
+
+    // 1. this wavefront's page is on its way while the queries are made
+    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;
+    const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
+    const long phys_new = page_table[(long)b * table_width + qpos / PAGE];
+    PageFrags<DH> f;
+    if (has) load_page<DH>(f, k_pages, v_pages, page_table[(long)b * table_width + page], kv_heads, kvh, lane);
+
+    // 2. queries of the group; in the owner also the new key and value
+    const bf16_t* row = qkv + (long)b * q_stride;
+    for (int g = wave; g < group; g += DECODE_WAVES)
+        norm_rotate_head<DH>(q_lds[g], row + (kvh * group + g) * DH, q_gain, eps, inv_freq, qpos, lane);
+    if (owner) {
+        const int slot = qpos % PAGE;
+        const long head_base = (phys_new * kv_heads + kvh) * (long)(PAGE * DH);
+        if (wave == DECODE_WAVES - 1) {                      // the key: norm, rotation, into LDS and into its page
+            norm_rotate_head<DH>(knew, row + (heads + kvh) * DH, k_gain, eps, inv_freq, qpos, lane);
+            __builtin_amdgcn_wave_barrier();
+            for (int d = lane; d < DH; d += 64) k_pages[head_base + (long)slot * DH + d] = knew[d];
+        } else if (wave == DECODE_WAVES - 2) {               // the value: a copy, transposed inside the page
+            for (int d = lane; d < DH; d += 64) {
+                const bf16_t v = row[(heads + kv_heads + kvh) * DH + d];
+                vnew[d] = v;
+                v_pages[head_base + (long)d * PAGE + slot] = v;
+            }
+        }
+    }
+    __syncthreads();
+
+    // 3. this wavefront's page against the group's queries
+    Columns<DH, 1> c;
+    init_columns<DH, 1>(c);
+    const int jg = lane >> 4, col = lane & 15;
+    if (col < group) {
+        c.qpos[0] = qpos;
+        c.lo[0] = lo;
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks)
+            c.q[0][ks].u = *reinterpret_cast<const uint4*>(&q_lds[col][ks * 32 + jg * 8]);
+    }
+    if (has && page == qpos / PAGE) {                        // the new token's key and value are not in memory yet
+        const int r = qpos % PAGE;
+        const int i_new = (r >> 3) * 4 + (r & 3);            // the fragment row that holds key r
+        if (col == i_new) {
+#pragma unroll
+            for (int ks = 0; ks < DH / 32; ++ks) {
+                const uint4 kv = *reinterpret_cast<const uint4*>(&knew[ks * 32 + jg * 8]);
+                if ((r & 7) >= 4) f.k[1][ks].u = kv; else f.k[0][ks].u = kv;
+            }
+        }
+        if (jg == (r >> 3)) {                                // lanes whose eight keys include key r
+            const int e = r & 7;
+#pragma unroll
+            for (int dt = 0; dt < DH / 16; ++dt) {
+                const uint32_t v = vnew[dt * 16 + col];
+                uint32_t w[4] = {f.v[dt].u.x, f.v[dt].u.y, f.v[dt].u.z, f.v[dt].u.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (k == (e >> 1)) w[k] = (e & 1) ? ((w[k] & 0x0000FFFFu) | (v << 16)) : ((w[k] & 0xFFFF0000u) | v);
+                f.v[dt].u = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    }
+    if (has) process_page<DH, 1>(c, f, page, lane, scale_log2, false);
+    finish_columns<DH, 1>(c);
+
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_lds[wave][(dt * 16 + jg * 4 + r) * 17 + col] = c.o[0][dt][r];
+    if (jg == 0) {
+        ml_lds[wave][0][col] = c.m[0];
+        ml_lds[wave][1][col] = c.l[0];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < group * DH; idx += DECODE_WAVES * 64) {
+        const int g = idx / DH, d = idx - g * DH;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, ml_lds[w][0][g]);
+        float acc = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < DECODE_WAVES; ++w) {
+            const float mw = ml_lds[w][0][g];
+            const float f2 = mw == -INFINITY ? 0.f : exp2f(mw - m);
+            acc += o_lds[w][d * 17 + g] * f2;
+            l += ml_lds[w][1][g] * f2;
+        }
+        float* dst = ws + (((long)b * heads + kvh * group + g) * max_chunks + chunk) * (DH + 2);
+        dst[d] = acc;
+        if (d == 0) {
+            dst[DH] = m;
+            dst[DH + 1] = l;
+        }
+    }
+
+}
+
 // ------------------------------------------------------------------ host side
 static int check_common(const char* name, int heads, int kv_heads, int head_dim, int page_size, int q_stride,
                         int table_width) {
@@ -496,5 +651,42 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
     }
 #undef RI_DECODE_CASE
     RI_LAUNCH_CHECK("attention_decode_bf16");
+    return 0;
+}
+
+// The decode attention of a layer from the raw fused projection (which is not changed): q/k norm, rotation,
+// the new token's k and v into their pages and attention in chunks in one kernel, then the join.
+extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const void* qkv, int q_stride,
+                                              const float* q_gain, const float* k_gain, float eps,
+                                              const float* inv_freq, void* k_pages, void* v_pages,
+                                              const int32_t* tok_pos, const int32_t* page_table, int table_width,
+                                              int seqs, int max_chunks, int heads, int kv_heads, int head_dim,
+                                              int page_size, int window, float scale, void* stream) {
+    if (check_common("attention_decode_fused_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width))
+        return 1;
+    const int group = heads / kv_heads;
+    RI_REQUIRE(group <= 16, "attention_decode_fused_bf16: %d query heads per kv head (at most 16)", group);
+    RI_REQUIRE(seqs > 0 && seqs <= 65535 && max_chunks > 0 && heads <= 65535,
+               "attention_decode_fused_bf16: seqs %d, chunks %d, heads %d", seqs, max_chunks, heads);
+    RI_REQUIRE(q_stride >= (heads + 2 * kv_heads) * head_dim, "attention_decode_fused_bf16: qkv row stride %d",
+               q_stride);
+    dim3 grid(max_chunks, seqs, kv_heads);
+    const float scale_log2 = scale * 1.4426950408889634f;
+    hipStream_t s = (hipStream_t)stream;
+#define RI_FUSED_CASE(DH)                                                                                         \
+    case DH:                                                                                                      \
+        attn_decode_fused_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                          \
+            workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq, (bf16_t*)k_pages,             \
+            (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks); \
+        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos, heads,    \
+                                                                      window, max_chunks);                        \
+        break;
+    switch (head_dim) {
+        RI_FUSED_CASE(32)
+        RI_FUSED_CASE(64)
+        RI_FUSED_CASE(128)
+    }
+#undef RI_FUSED_CASE
+    RI_LAUNCH_CHECK("attention_decode_fused_bf16");
     return 0;
 }

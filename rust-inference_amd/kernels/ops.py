@@ -31,6 +31,9 @@ _SIGNATURES = {
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "ri_attention_decode_fused_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float,
+                                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_skinny_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -240,6 +243,32 @@ def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
           k_pages.shape[2], int(window or 0), float(scale), _stream())
+    return out
+
+
+def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_pages, tok_pos, page_table, seqs: int,
+                                max_len: int, heads: int, kv_heads: int, head_dim: int, window: int | None,
+                                scale: float) -> torch.Tensor:
+    """A layer's decode attention from the raw ``qkv: [seqs, (H + 2 Hkv) dh]``: q/k norm, rotation, the new
+    token's k and v into their pages and attention in one kernel, then the join."""
+    tokens, stride = qkv.shape
+    if tokens != seqs:
+        raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
+    num_pages, hkv, page_size, dh = k_pages.shape
+    if (hkv, dh) != (kv_heads, head_dim) or tuple(v_pages.shape) != (num_pages, hkv, dh, page_size):
+        raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv heads "
+                         f"of {head_dim}")
+    chunks = -(-max_len // DECODE_CHUNK)
+    out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
+    half = head_dim // 2
+    _call("ri_attention_decode_fused_bf16", _dev(out, "out"), _dev(ws, "workspace"),
+          _dev(qkv, "qkv", torch.bfloat16), stride, _opt(q_gain, "q_gain", torch.float32, (head_dim,)),
+          _opt(k_gain, "k_gain", torch.float32, (head_dim,)), float(eps),
+          _opt(inv_freq, "inv_freq", torch.float32, (half,)), _dev(k_pages, "k_pages", torch.bfloat16),
+          _dev(v_pages, "v_pages", torch.bfloat16), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
+          _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
+          page_size, int(window or 0), float(scale), _stream())
     return out
 
 

@@ -72,6 +72,14 @@ class GroupedQueryAttention(Mixer):
         rt = self.rt
         qkv = rt.linear(x, self.w_qkv)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
+        group = self.heads // self.kv_heads
+        if ctx.is_decode and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, True):
+            # one token per sequence: norm, rotation, cache write and attention are one kernel
+            o = ops.attention_decode_fused_bf16(qkv, self.q_gain, self.k_gain, self.eps,
+                                                self.position.rotation_table(), store.k_pages, store.v_pages,
+                                                ctx.tok_pos, page_table, ctx.B, ctx.max_len, self.heads,
+                                                self.kv_heads, self.head_dim, self.window, self.scale)
+            return rt.linear_packed(o, self.w_o)
         ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
                                   ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
                                   self.heads, self.kv_heads, self.head_dim)

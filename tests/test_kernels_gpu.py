@@ -252,6 +252,45 @@ def test_mfma_attention_window_edges(ops, kernel, window):
     close(out, want, 1e-2, f"window {window}")
 
 
+@pytest.mark.parametrize("heads, kv_heads, dh", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [None, 40])
+def test_fused_decode_attention(ops, heads, kv_heads, dh, window):
+    """Norm, rotation, cache write and attention from the raw projection, against the plain parts; twice in
+    a row on the same buffers, then one token further."""
+    rng = np.random.default_rng(heads * 13 + dh)
+    lens = [1, 32, 33, 256, 257, 512, 700, 5]                # lengths after this step
+    B = len(lens)
+    k, v, kp, vp, table = paged(rng, [n + 1 for n in lens], kv_heads, dh, dtype=torch.bfloat16, spare=12)
+    width = (heads + 2 * kv_heads) * dh
+    qg, kg = t(1 + 0.2 * rng.normal(size=dh)), t(1 + 0.2 * rng.normal(size=dh))
+    theta, eps = 50000.0, 1e-5
+    inv_freq = t(P.rope_inv_freq(dh, theta))
+    for step in range(2):
+        cur = [n + step for n in lens]
+        pos = [n - 1 for n in cur]
+        raw = t(rng.normal(size=(B, width)) * 2, torch.bfloat16)
+        raw64 = f64(raw)
+        for repeat in range(2):
+            out = ops.attention_decode_fused_bf16(raw, qg, kg, eps, inv_freq, kp, vp, t(pos, torch.int32), table, B,
+                                                  max(cur) + 300, heads, kv_heads, dh, window, 1.0 / np.sqrt(dh))
+            assert torch.equal(raw, t(raw64, torch.bfloat16)), "the projection is read, not changed"
+            q = raw64[:, :heads * dh].reshape(B, heads, dh)
+            kn = raw64[:, heads * dh:(heads + kv_heads) * dh].reshape(B, kv_heads, dh)
+            vn = raw64[:, (heads + kv_heads) * dh:].reshape(B, kv_heads, dh)
+            ang = P.rope_angles(pos, dh, theta)
+            q = P.bf16_round(P.apply_rope(P.rms_norm(q, f64(qg), eps), ang).astype(np.float32)).astype(np.float64)
+            kn = P.apply_rope(P.rms_norm(kn, f64(kg), eps), ang)
+            tab = table.cpu().numpy()
+            for b in range(B):
+                page, off = tab[b, pos[b] // 32], pos[b] % 32
+                close(kp[page, :, off], kn[b], 1e-2, "the new key in its page")
+                assert np.array_equal(f64(vp[page, :, :, off]), vn[b]), "the new value in its page"
+                kb = np.stack([f64(kp[tab[b, p // 32], :, p % 32]) for p in range(cur[b])])
+                vb = np.stack([f64(vp[tab[b, p // 32], :, :, p % 32]) for p in range(cur[b])])
+                want = P.attention(q[b:b + 1], kb, vb, window=window)
+                close(out[b].reshape(1, heads, dh), want, 1e-2, f"sequence {b}, step {step}, repeat {repeat}")
+
+
 def test_mfma_and_generic_attention_agree(ops):
     """The same call through all three kernels: decode against prefill against generic."""
     outs = []
