@@ -31,8 +31,11 @@ int ri_add_rows(float* out, const float* residual, const void* pending, int pend
 // qkv: [tokens, (heads + 2 kv_heads) * head_dim] of act_dtype.  tok_pos/tok_seq: int32 [tokens].
 // page_table: int32 [seqs, table_width].  k_pages: [pages, kv_heads, page_size, head_dim], v_pages (transposed
 // inside a page): [pages, kv_heads, head_dim, page_size], both of cache_dtype.
+// cu_seqlens (int32 [seqs + 1], may be NULL), seqs and max_new (most new tokens of a sequence) let values be
+// written a page at a time; without them every element is written on its own.
 int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
                              const float* inv_freq, int rot_dim, const int32_t* tok_pos, const int32_t* tok_seq,
+                             const int32_t* cu_seqlens, int seqs, int max_new,
                              const int32_t* page_table, int table_width, void* k_pages, void* v_pages,
                              int cache_dtype, int tokens, int heads, int kv_heads, int head_dim, int page_size,
                              int num_pages, void* stream);

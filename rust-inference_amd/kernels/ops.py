@@ -23,8 +23,8 @@ _SIGNATURES = {
     "ri_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p],
     "ri_add_rows": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_qk_norm_rope_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p,
-                                 c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                 c_void_p],
+                                 c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                 c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention": [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
@@ -174,8 +174,9 @@ def mark_seen(seen: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor) -> N
 
 # ---------------------------------------------------------------- attention
 def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, k_pages, v_pages,
-                          heads: int, kv_heads: int, head_dim: int) -> None:
-    """In place on ``qkv: [T, (H + 2 Hkv) dh]``: per-head norm and rotation of q and k; k and v go to their pages."""
+                          heads: int, kv_heads: int, head_dim: int, cu_seqlens=None, max_new: int = 0) -> None:
+    """In place on ``qkv: [T, (H + 2 Hkv) dh]``: per-head norm and rotation of q and k; k and v go to their
+    pages.  With ``cu_seqlens`` (int32 ``[seqs + 1]``) and ``max_new`` values are written a page at a time."""
     tokens = qkv.shape[0]
     width = (heads + 2 * kv_heads) * head_dim
     num_pages, hkv, page_size, dh = k_pages.shape
@@ -187,7 +188,8 @@ def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, 
           _opt(q_gain, "q_gain", torch.float32, (head_dim,)), _opt(k_gain, "k_gain", torch.float32, (head_dim,)),
           float(eps), _opt(inv_freq, "inv_freq", torch.float32, (half,)), head_dim,
           _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
-          _dev(page_table, "page_table", torch.int32), page_table.shape[1],
+          _opt(cu_seqlens, "cu_seqlens", torch.int32), 0 if cu_seqlens is None else cu_seqlens.shape[0] - 1,
+          int(max_new), _dev(page_table, "page_table", torch.int32), page_table.shape[1],
           _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), code(k_pages.dtype), tokens, heads, kv_heads, head_dim,
           page_size, num_pages, _stream())
 

@@ -89,7 +89,7 @@ class GroupedQueryAttention(Mixer):
             return rt.linear_packed(o, self.w_o)
         ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
                                   ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
-                                  self.heads, self.kv_heads, self.head_dim)
+                                  self.heads, self.kv_heads, self.head_dim, ctx.cu_seqlens, ctx.max_new)
         return rt.linear_packed(self.attend(qkv, ctx, store, page_table), self.w_o)
 
     def attend(self, qkv, ctx, store, page_table):

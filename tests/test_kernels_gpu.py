@@ -98,11 +98,12 @@ def paged(rng, lens, hkv, dh, page_size=32, dtype=torch.float32, spare=3):
     return k, v, t(kp, dtype), t(vp, dtype), t(table, torch.int32)
 
 
+@pytest.mark.parametrize("paged_values", [False, True])
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
-@pytest.mark.parametrize("heads, kv_heads, dh", [(6, 2, 48), (4, 4, 128), (9, 1, 16), (2, 1, 256)])
-def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh):
+@pytest.mark.parametrize("heads, kv_heads, dh", [(6, 2, 48), (4, 4, 128), (9, 1, 16), (2, 1, 256), (5, 5, 64), (8, 2, 32)])
+def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh, paged_values):
     rng = np.random.default_rng(heads * dh)
-    lens_before, new = [37, 0, 63], [3, 2, 5]                    # writes cross page boundaries
+    lens_before, new = [37, 0, 63, 30], [3, 2, 5, 70]            # writes cross page boundaries; one spans four pages
     lens = [a + b for a, b in zip(lens_before, new)]
     _, _, kp, vp, table = paged(rng, lens, kv_heads, dh, dtype=dtype)
     kp.zero_(); vp.zero_()
@@ -115,8 +116,10 @@ def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh):
     qg, kg = 1 + 0.2 * rng.normal(size=dh), 1 + 0.2 * rng.normal(size=dh)
     theta, eps = 50000.0, 1e-5
     inv_freq = t(P.rope_inv_freq(dh, theta))
+    # with the sequences' bounds the 16-byte kernels and the page-wise value writer run (where the head size fits)
+    extra = dict(cu_seqlens=t(np.concatenate([[0], np.cumsum(new)]), torch.int32), max_new=max(new)) if paged_values else {}
     ops.qk_norm_rope_kv_write(qkv_t, t(qg), t(kg), eps, inv_freq, t(tok_pos, torch.int32), t(tok_seq, torch.int32),
-                              table, kp, vp, heads, kv_heads, dh)
+                              table, kp, vp, heads, kv_heads, dh, **extra)
     ang = P.rope_angles(tok_pos, dh, theta)
     q = qkv[:, :heads * dh].reshape(tokens, heads, dh)
     k = qkv[:, heads * dh:(heads + kv_heads) * dh].reshape(tokens, kv_heads, dh)
@@ -131,10 +134,11 @@ def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh):
         assert np.array_equal(f64(vp[page, :, :, off]), v[i]), "v is a copy"
     # nothing else was written: as many rows are non-zero as tokens
     assert int((kp.float().abs().sum(-1) > 0).sum()) == tokens * kv_heads
+    assert int((vp.float().abs().sum(-2) > 0).sum()) == tokens * kv_heads
     # without gains and rotation the kernel only moves k and v
     qkv2 = t(qkv, dtype)
     ops.qk_norm_rope_kv_write(qkv2, None, None, eps, None, t(tok_pos, torch.int32), t(tok_seq, torch.int32),
-                              table, kp, vp, heads, kv_heads, dh)
+                              table, kp, vp, heads, kv_heads, dh, **extra)
     assert np.array_equal(f64(qkv2), qkv)
 
 
