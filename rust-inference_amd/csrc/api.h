@@ -19,8 +19,10 @@ int ri_embed_gather(float* out, const void* table, int table_dtype, const int32_
 // r = residual[src] (+ pending[src]); if rows == NULL: src = row and residual[row] = r is written back;
 // else src = rows[row] and nothing is written back.  out[row] = r * rsqrt(mean(r^2) + eps) * gain.
 // residual float32, pending of pending_dtype (may be NULL), gain float32, out of out_dtype.
-int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype,
-                   const float* gain, float eps, const int32_t* rows, int n_rows, int dim, void* stream);
+// pending may be `parts` tensors [parts][total_rows][dim] that are added one after the other.
+int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype, int parts,
+                   int total_rows, const float* gain, float eps, const int32_t* rows, int n_rows, int dim,
+                   void* stream);
 
 // Plain residual add on gathered rows, no norm: out[row] = residual[src] + pending[src], float32.
 int ri_add_rows(float* out, const float* residual, const void* pending, int pending_dtype,
@@ -90,8 +92,10 @@ int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, 
 // The same with the weights packed ahead of time into MFMA tiles: [ceil(n/16)][ceil(k/32)][64 lanes][8],
 // lane l of a tile holding row l % 16, k 8 * (l / 16)..+8, zero beyond n and k; with swiglu the up matrix's
 // ceil(n/16) row tiles follow the gate's.
+// parts > 1 cuts K into that many pieces whose float32 sums go to out[part][m][n] (the consumer adds them in
+// order); it needs out_dtype float32 and no swiglu.
 int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
-                               int swiglu, void* stream);
+                               int swiglu, int parts, void* stream);
 
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);

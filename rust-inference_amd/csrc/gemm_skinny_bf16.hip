@@ -1,6 +1,6 @@
 // Decode-size products on the matrix cores: out[M, N] = x[M, K] . w[N, K]^T for bfloat16 with up to
 // 16 rows of x per tile of MFMA 16x16x32 columns.  The weights are the traffic and are read once:
-// a workgroup of eight wavefronts owns 16 rows of w, each wavefront one eighth of K; the weight
+// a workgroup of four or eight wavefronts owns 16 rows of w, each wavefront its share of K; the weight
 // fragments go from global memory straight into the A operand (lane l: row l % 16, eight
 // consecutive k at 8 * (l / 16)), the rows of x into the B operand the same way (they come from
 // the L2 cache), and the eight partial sums are added through LDS in wavefront order.  Rows of x
@@ -17,12 +17,11 @@ union Frag {
     uint4 u;
 };
 
-#define SK_WAVES 8
 #define SK_CHUNK 8            // MFMA steps (of 32 k) whose loads are in flight together
 
 __device__ __forceinline__ float silu_sk(float z) { return z / (1.0f + expf(-z)); }
 
-template <bool SWIGLU, typename TO>
+template <int SK_WAVES, bool SWIGLU, typename TO>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N,
                         int K, int kslice) {
@@ -80,7 +79,7 @@ gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
 // row l % 16, k 8 * (l / 16) ..+8), tiles of one row block consecutive in k.  A wavefront's loads are
 // then whole contiguous kilobytes, which is what the memory system streams fastest.
 // packed: [row_tiles][k_tiles][64 lanes][8]; for SwiGLU the up matrix's tiles follow the gate's.
-template <bool SWIGLU, typename TO>
+template <int SK_WAVES, bool SWIGLU, typename TO>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked,
                           int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset) {
@@ -90,7 +89,11 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     const int i = lane & 15, jg = lane >> 4;
     const int nt = blockIdx.x;
     const bool x_ok = i < M;
-    const int kt_begin = wave * tiles_per_wave, kt_end = min(k_tiles, kt_begin + tiles_per_wave);
+    // blockIdx.y cuts K into gridDim.y parts whose sums go to separate outputs out[part][M][N]
+    const int part_tiles = (k_tiles + gridDim.y - 1) / gridDim.y;
+    const int part_begin = blockIdx.y * part_tiles, part_end = min(k_tiles, part_begin + part_tiles);
+    const int kt_begin = part_begin + wave * tiles_per_wave, kt_end = min(part_end, kt_begin + tiles_per_wave);
+    out += (size_t)blockIdx.y * M * N;
     const bf16_t* wp = wpacked + ((size_t)nt * k_tiles * 64 + lane) * 8;
     const bf16_t* up = SWIGLU ? wpacked + ((size_t)(up_tile_offset + nt) * k_tiles * 64 + lane) * 8 : nullptr;
     const bf16_t* xp = x + (size_t)(x_ok ? i : 0) * K + jg * 8;
@@ -134,33 +137,56 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     }
 }
 
+// Four wavefronts a workgroup stream fastest when there are many row tiles (5.0 TB/s on the 24576 x 4096
+// gate|up matrix against 4.6 with eight); a long K with few row tiles wants the eight (K = 12288, 256 tiles).
+static int skinny_waves(int n, int k) { return k >= 8192 ? 8 : 4; }
+
+template <int WAVES, bool SWIGLU>
+static void launch_packed(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts,
+                          hipStream_t s) {
+    const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
+    const int part_tiles = (k_tiles + parts - 1) / parts;
+    const int tiles_per_wave = (part_tiles + WAVES - 1) / WAVES;
+    dim3 grid(row_tiles, parts);
+    if (out_dtype == RI_F32)
+        gemm_skinny_packed_kernel<WAVES, SWIGLU, float><<<grid, WAVES * 64, 0, s>>>(
+            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+    else
+        gemm_skinny_packed_kernel<WAVES, SWIGLU, bf16_t><<<grid, WAVES * 64, 0, s>>>(
+            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+}
+
 extern "C" int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
-                                          int k, int swiglu, void* stream) {
+                                          int k, int swiglu, int parts, void* stream) {
     RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_packed_bf16: %d rows of x, this kernel takes 1 to 16", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_packed_bf16: out dtype %d", out_dtype);
-    const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
-    const int tiles_per_wave = (k_tiles + SK_WAVES - 1) / SK_WAVES;
+    RI_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || (!swiglu && out_dtype == RI_F32)),
+               "gemm_skinny_packed_bf16: %d parts of K (more than one needs float32 sums and no activation)", parts);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)wpacked;
+    const bool eight = skinny_waves(n, (k + parts - 1) / parts) == 8;
     if (swiglu) {
-        if (out_dtype == RI_F32)
-            gemm_skinny_packed_kernel<true, float><<<row_tiles, SK_WAVES * 64, 0, s>>>(
-                (float*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, row_tiles);
-        else
-            gemm_skinny_packed_kernel<true, bf16_t><<<row_tiles, SK_WAVES * 64, 0, s>>>(
-                (bf16_t*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+        if (eight) launch_packed<8, true>(out, out_dtype, xb, wb, m, n, k, parts, s);
+        else       launch_packed<4, true>(out, out_dtype, xb, wb, m, n, k, parts, s);
     } else {
-        if (out_dtype == RI_F32)
-            gemm_skinny_packed_kernel<false, float><<<row_tiles, SK_WAVES * 64, 0, s>>>(
-                (float*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, 0);
-        else
-            gemm_skinny_packed_kernel<false, bf16_t><<<row_tiles, SK_WAVES * 64, 0, s>>>(
-                (bf16_t*)out, xb, wb, m, n, k, k_tiles, tiles_per_wave, 0);
+        if (eight) launch_packed<8, false>(out, out_dtype, xb, wb, m, n, k, parts, s);
+        else       launch_packed<4, false>(out, out_dtype, xb, wb, m, n, k, parts, s);
     }
     RI_LAUNCH_CHECK("gemm_skinny_packed_bf16");
     return 0;
+}
+
+template <int WAVES, bool SWIGLU>
+static void launch_skinny(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k,
+                          hipStream_t s) {
+    const int kslice = ((k + WAVES - 1) / WAVES + 31) / 32 * 32;
+    const unsigned grid = (n + 15) / 16;
+    if (out_dtype == RI_F32)
+        gemm_skinny_bf16_kernel<WAVES, SWIGLU, float><<<grid, WAVES * 64, 0, s>>>((float*)out, x, w, m, n, k, kslice);
+    else
+        gemm_skinny_bf16_kernel<WAVES, SWIGLU, bf16_t><<<grid, WAVES * 64, 0, s>>>((bf16_t*)out, x, w, m, n, k, kslice);
 }
 
 extern "C" int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
@@ -168,21 +194,16 @@ extern "C" int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, cons
     RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_bf16: %d rows of x, this kernel takes 1 to 16", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_bf16: out dtype %d", out_dtype);
-    const int kslice = ((k + SK_WAVES - 1) / SK_WAVES + 31) / 32 * 32;
-    const unsigned grid = (n + 15) / 16;
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
+    const bool eight = skinny_waves(n, k) == 8;
     if (swiglu) {
-        if (out_dtype == RI_F32)
-            gemm_skinny_bf16_kernel<true, float><<<grid, SK_WAVES * 64, 0, s>>>((float*)out, xb, wb, m, n, k, kslice);
-        else
-            gemm_skinny_bf16_kernel<true, bf16_t><<<grid, SK_WAVES * 64, 0, s>>>((bf16_t*)out, xb, wb, m, n, k, kslice);
+        if (eight) launch_skinny<8, true>(out, out_dtype, xb, wb, m, n, k, s);
+        else       launch_skinny<4, true>(out, out_dtype, xb, wb, m, n, k, s);
     } else {
-        if (out_dtype == RI_F32)
-            gemm_skinny_bf16_kernel<false, float><<<grid, SK_WAVES * 64, 0, s>>>((float*)out, xb, wb, m, n, k, kslice);
-        else
-            gemm_skinny_bf16_kernel<false, bf16_t><<<grid, SK_WAVES * 64, 0, s>>>((bf16_t*)out, xb, wb, m, n, k, kslice);
+        if (eight) launch_skinny<8, false>(out, out_dtype, xb, wb, m, n, k, s);
+        else       launch_skinny<4, false>(out, out_dtype, xb, wb, m, n, k, s);
     }
     RI_LAUNCH_CHECK("gemm_skinny_bf16");
     return 0;

@@ -34,8 +34,8 @@ extern "C" int ri_embed_gather(float* out, const void* table, int table_dtype, c
 // float32 and is not rounded before the variance is taken.
 template <typename TP, typename TO>
 __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ residual, const TP* __restrict__ pending,
-                                   const float* __restrict__ gain, float eps, const int32_t* __restrict__ rows,
-                                   int dim) {
+                                   int parts, size_t part_stride, const float* __restrict__ gain, float eps,
+                                   const int32_t* __restrict__ rows, int dim) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[row] : row) * dim;
@@ -43,7 +43,8 @@ __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ res
     float ss = 0.f;
     for (int d = threadIdx.x; d < dim; d += blockDim.x) {
         float v = residual[src + d];
-        if (pending) v += to_f32(pending[src + d]);
+        if (pending)
+            for (int p = 0; p < parts; ++p) v += to_f32(pending[p * part_stride + src + d]);
         if (write_back && pending) residual[src + d] = v;
         ss += v * v;
     }
@@ -51,7 +52,8 @@ __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ res
     TO* o = out + (size_t)row * dim;
     for (int d = threadIdx.x; d < dim; d += blockDim.x) {
         float v = residual[src + d];                       // written by this same thread when write_back
-        if (pending && !write_back) v += to_f32(pending[src + d]);
+        if (pending && !write_back)
+            for (int p = 0; p < parts; ++p) v += to_f32(pending[p * part_stride + src + d]);
         from_f32(o + d, v * inv * gain[d]);
     }
 }
@@ -77,7 +79,8 @@ __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
 template <typename TP, typename TO, int VPT>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const TP* __restrict__ pending,
-                       const float* __restrict__ gain, float eps, const int32_t* __restrict__ rows, int dim) {
+                       int parts, size_t part_stride, const float* __restrict__ gain, float eps,
+                       const int32_t* __restrict__ rows, int dim) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[row] : row) * dim;
@@ -91,8 +94,10 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
             v[i] = load4(residual + src + d);
             g[i] = load4(gain + d);
             if (pending) {
-                const float4 p = load4(pending + src + d);
-                v[i].x += p.x; v[i].y += p.y; v[i].z += p.z; v[i].w += p.w;
+                for (int q = 0; q < parts; ++q) {            // the parts of a split product, always in this order
+                    const float4 p = load4(pending + q * part_stride + src + d);
+                    v[i].x += p.x; v[i].y += p.y; v[i].z += p.z; v[i].w += p.w;
+                }
             }
         }
     }
@@ -117,39 +122,46 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
 }
 
 template <typename TP, typename TO>
-static void launch_add_rmsnorm_typed(TO* out, float* residual, const TP* pending, const float* gain, float eps,
-                                     const int32_t* rows, int n_rows, int dim, hipStream_t s) {
+static void launch_add_rmsnorm_typed(TO* out, float* residual, const TP* pending, int parts, size_t ps,
+                                     const float* gain, float eps, const int32_t* rows, int n_rows, int dim,
+                                     hipStream_t s) {
     if (dim % 4 == 0 && dim <= 1024)
-        add_rmsnorm_vec_kernel<TP, TO, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
     else if (dim % 4 == 0 && dim <= 2048)
-        add_rmsnorm_vec_kernel<TP, TO, 2><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 2><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
     else if (dim % 4 == 0 && dim <= 4096)
-        add_rmsnorm_vec_kernel<TP, TO, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
     else if (dim % 4 == 0 && dim <= 8192)
-        add_rmsnorm_vec_kernel<TP, TO, 8><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 8><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
     else
-        add_rmsnorm_kernel<TP, TO><<<n_rows, 256, 0, s>>>(out, residual, pending, gain, eps, rows, dim);
+        add_rmsnorm_kernel<TP, TO><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
 }
 
 template <typename TP>
-static void launch_add_rmsnorm(void* out, int out_dtype, float* residual, const TP* pending, const float* gain,
-                               float eps, const int32_t* rows, int n_rows, int dim, hipStream_t s) {
+static void launch_add_rmsnorm(void* out, int out_dtype, float* residual, const TP* pending, int parts, size_t ps,
+                               const float* gain, float eps, const int32_t* rows, int n_rows, int dim, hipStream_t s) {
     if (out_dtype == RI_F32)
-        launch_add_rmsnorm_typed<TP, float>((float*)out, residual, pending, gain, eps, rows, n_rows, dim, s);
+        launch_add_rmsnorm_typed<TP, float>((float*)out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, s);
     else
-        launch_add_rmsnorm_typed<TP, bf16_t>((bf16_t*)out, residual, pending, gain, eps, rows, n_rows, dim, s);
+        launch_add_rmsnorm_typed<TP, bf16_t>((bf16_t*)out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim,
+                                             s);
 }
 
 extern "C" int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype,
-                              const float* gain, float eps, const int32_t* rows, int n_rows, int dim, void* stream) {
+                              int parts, int total_rows, const float* gain, float eps, const int32_t* rows, int n_rows,
+                              int dim, void* stream) {
     RI_REQUIRE(n_rows > 0 && dim > 0, "add_rmsnorm: rows %d, dim %d", n_rows, dim);
+    RI_REQUIRE(parts >= 1 && parts <= 64 && total_rows >= 1, "add_rmsnorm: %d parts of %d rows", parts, total_rows);
+    const size_t ps = (size_t)total_rows * dim;
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "add_rmsnorm: out dtype %d", out_dtype);
     RI_REQUIRE(pending_dtype == RI_F32 || pending_dtype == RI_BF16, "add_rmsnorm: pending dtype %d", pending_dtype);
     hipStream_t s = (hipStream_t)stream;
     if (pending_dtype == RI_F32)
-        launch_add_rmsnorm<float>(out, out_dtype, residual, (const float*)pending, gain, eps, rows, n_rows, dim, s);
+        launch_add_rmsnorm<float>(out, out_dtype, residual, (const float*)pending, parts, ps, gain, eps, rows, n_rows,
+                                  dim, s);
     else
-        launch_add_rmsnorm<bf16_t>(out, out_dtype, residual, (const bf16_t*)pending, gain, eps, rows, n_rows, dim, s);
+        launch_add_rmsnorm<bf16_t>(out, out_dtype, residual, (const bf16_t*)pending, parts, ps, gain, eps, rows, n_rows,
+                                   dim, s);
     RI_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }

@@ -20,7 +20,8 @@ _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
 _SIGNATURES = {
     "ri_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
-    "ri_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p],
+    "ri_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_int,
+                       c_int, c_void_p],
     "ri_add_rows": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_qk_norm_rope_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p,
                                  c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -40,7 +41,7 @@ _SIGNATURES = {
     "ri_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_float,
                   c_void_p],
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
-    "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -110,12 +111,20 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
 def add_rmsnorm(residual: torch.Tensor, pending, gain: torch.Tensor, eps: float, out_dtype,
                 rows: torch.Tensor | None = None) -> torch.Tensor:
     """``residual += pending`` (in place, when ``rows`` is None) and the RMSNorm of the sum.
-    With ``rows`` the sum and norm are taken of those rows only and nothing is written back."""
+    With ``rows`` the sum and norm are taken of those rows only and nothing is written back.
+    ``pending`` may be ``[parts, T, dim]``: the parts of a product split along K, added in order."""
     t, dim = residual.shape
     n = t if rows is None else rows.shape[0]
+    parts = 1
+    if pending is not None and pending.dim() == 3:
+        parts = pending.shape[0]
+        if tuple(pending.shape[1:]) != (t, dim):
+            raise ShapeError(f"pending parts are {list(pending.shape)}, the stream is {[t, dim]}")
+    elif pending is not None and tuple(pending.shape) != (t, dim):
+        raise ShapeError(f"pending is {list(pending.shape)}, the stream is {[t, dim]}")
     out = torch.empty((n, dim), dtype=out_dtype, device=residual.device)
     _call("ri_add_rmsnorm", _dev(out, "out"), code(out_dtype), _dev(residual, "residual", torch.float32),
-          _opt(pending, "pending", None, (t, dim)), code(pending.dtype) if pending is not None else F32,
+          _opt(pending, "pending"), code(pending.dtype) if pending is not None else F32, parts, t,
           _dev(gain, "gain", torch.float32, (dim,)), float(eps), _opt(rows, "rows", torch.int32), n, dim, _stream())
     return out
 
@@ -325,15 +334,16 @@ def pack_for_mfma(w: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
 
 
 def gemm_skinny_packed_bf16(x: torch.Tensor, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16,
-                            swiglu: bool = False) -> torch.Tensor:
+                            swiglu: bool = False, parts: int = 1) -> torch.Tensor:
     """``x @ w.T`` for up to 16 bfloat16 rows with ``w`` packed by ``pack_for_mfma``; ``n`` is the number of
-    output columns (rows of w; of its gate half with ``swiglu``)."""
+    output columns (rows of w; of its gate half with ``swiglu``).  With ``parts > 1`` K is cut into that many
+    pieces and the result is their float32 sums ``[parts, M, n]``, for a consumer that adds them."""
     m, k = x.shape
     row_tiles = -(-n // 16)
     want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
     if tuple(wpacked.shape) != want:
         raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
-    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    out = torch.empty((m, n) if parts == 1 else (parts, m, n), dtype=out_dtype, device=x.device)
     _call("ri_gemm_skinny_packed_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
-          _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), _stream())
+          _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), int(parts), _stream())
     return out

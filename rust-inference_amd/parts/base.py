@@ -23,7 +23,10 @@ class Part:
 class Norm(Part):
     """``apply(residual, pending, out_dtype, rows=None)``: adds ``pending`` into the
     float32 residual stream (in place when ``rows`` is None) and returns the norm of
-    the sum in ``out_dtype``; with ``rows`` only those rows, nothing written back."""
+    the sum in ``out_dtype``; with ``rows`` only those rows, nothing written back.  A norm that sets
+    ``accepts_parts`` also takes ``pending`` as ``[parts, T, hidden]`` and adds the parts in order."""
+
+    accepts_parts = False
 
     def apply(self, residual, pending, out_dtype, rows=None):
         raise NotImplementedError
@@ -50,7 +53,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Token-wise ``[T, hidden] -> [T, hidden]``."""
+    """Token-wise ``[T, hidden] -> [T, hidden]``.  The result may also be ``[parts, T, hidden]`` float32:
+    partial sums that the residual stream adds up in order (a product split along K)."""
 
     def forward(self, x, ctx):
         raise NotImplementedError

@@ -18,6 +18,8 @@ class ResidualStream:
         self.pending = branch
 
     def normed(self, norm, out_dtype, rows=None):
+        if self.pending is not None and self.pending.dim() == 3 and not getattr(norm, "accepts_parts", False):
+            self.pending = self.pending.sum(0)       # a norm that does not know about parts
         out = norm.apply(self.sum, self.pending, out_dtype, rows)
         if rows is None:
             self.pending = None      # the kernel wrote sum + pending back
@@ -26,7 +28,8 @@ class ResidualStream:
     def flush(self) -> None:
         """Add the waiting branch without a norm (only arrangements that push twice need it)."""
         if self.pending is not None:
-            self.sum.add_(self.pending.to(self.sum.dtype))
+            pending = self.pending.sum(0) if self.pending.dim() == 3 else self.pending
+            self.sum.add_(pending.to(self.sum.dtype))
             self.pending = None
 
 

@@ -7,6 +7,7 @@ from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part
+from .runtime import PackedWeight
 
 
 @register_part("feed_forward", "swiglu")
@@ -31,9 +32,11 @@ class SwiGLU(FeedForward):
         p = self.prefix
         gate_up = rt.place_matrix(torch.cat([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], 0))
         self.w_gate_up = rt.pack(gate_up, swiglu=True)
-        self.w_down = rt.place_matrix(weights[p + "down_proj.weight"])
+        down = rt.place_matrix(weights[p + "down_proj.weight"])
+        # the packed copy pays only where K is long enough to be split (see PackedWeight.parts)
+        self.w_down = rt.pack(down) if self.inter >= 8192 else PackedWeight(down, None, False)
 
     def forward(self, x, ctx):
         rt = self.rt
         a = rt.linear_packed(x, self.w_gate_up)        # the activation is in the epilogue of the decode-size kernels
-        return rt.linear(a, self.w_down)
+        return rt.linear_packed(a, self.w_down, parts_ok=True)     # may come in parts: the stream's next norm adds them

@@ -12,6 +12,8 @@ class RMSNorm(Norm):
     """``y = x * (1 / sqrt(mean(x^2) + eps)) * w`` over the last axis, statistics in
     float32 (the reference: src/ops/norm.rs:7-32; fused with the add: :35-62)."""
 
+    accepts_parts = True
+
     def __init__(self, dim: int, eps: float, name: str):
         self.dim, self.eps, self.name = dim, eps, name
 

@@ -19,6 +19,7 @@ from ..kernels import ops
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
 GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
+SPLIT_K = 4096
 
 
 class PackedWeight:
@@ -29,6 +30,9 @@ class PackedWeight:
         self.w, self.packed, self.swiglu = w, packed, swiglu
         self.n = w.shape[0] // 2 if swiglu else w.shape[0]
         self.k = w.shape[1]
+        # a long K is cut into pieces of 4096 whose float32 sums the next norm adds up: more workgroups
+        # stream the weights (768 instead of 256 for 4096 x 12288), and the sum is never rounded to 16 bits
+        self.parts = self.k // SPLIT_K if (not swiglu and self.k >= 2 * SPLIT_K) else 1
 
 
 class Runtime:
@@ -79,15 +83,18 @@ class Runtime:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
 
-    def linear_packed(self, x: torch.Tensor, pw: PackedWeight, out_dtype=None) -> torch.Tensor:
+    def linear_packed(self, x: torch.Tensor, pw: PackedWeight, out_dtype=None, parts_ok: bool = False) -> torch.Tensor:
         """``x @ w.T`` (or ``silu(x @ gate.T) * (x @ up.T)`` for a fused gate|up weight) with the kernel
-        that fits the number of rows."""
+        that fits the number of rows.  With ``parts_ok`` the result may be ``[parts, M, N]`` float32, the
+        sums over pieces of K, for a consumer that adds them (the residual stream's next norm)."""
         out_dtype = out_dtype or self.dtype
         m = x.shape[0]
         if self.dtype == torch.bfloat16 and pw.k % 8 == 0:
             if m <= GEMV_MAX_ROWS:
                 return ops.gemv_bf16(x, pw.w, out_dtype, swiglu=pw.swiglu)
             if m <= SKINNY_MAX_ROWS and pw.packed is not None:
+                if parts_ok and pw.parts > 1:
+                    return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=pw.parts)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
         y = self.linear(x, pw.w, None if pw.swiglu else out_dtype)
         return ops.swiglu(y) if pw.swiglu else y

@@ -67,6 +67,22 @@ def test_add_rmsnorm(ops, dim, pending_dtype):
     close(ops.add_rows(before.clone(), pend, rows), total[[5, 0, 5]], 1e-7, "add_rows")
 
 
+def test_add_rmsnorm_adds_the_parts_of_a_split_product(ops):
+    rng = np.random.default_rng(11)
+    res, parts = t(rng.normal(size=(6, 4096))), t(rng.normal(size=(3, 6, 4096)))
+    gain = t(1 + 0.1 * rng.normal(size=4096))
+    total = f64(res) + f64(parts).sum(0)
+    out = ops.add_rmsnorm(res, parts, gain, 1e-6, torch.float32)
+    close(out, P.rms_norm(total, f64(gain), 1e-6), 2e-6, "norm over parts")
+    close(res, total, 2e-7, "residual over parts")
+    rows = t([4, 1], torch.int32)
+    res2 = t(rng.normal(size=(6, 104)))
+    p2 = t(rng.normal(size=(2, 6, 104)))
+    g2 = t(np.ones(104))
+    want = P.rms_norm((f64(res2) + f64(p2).sum(0))[[4, 1]], np.ones(104), 1e-6)
+    close(ops.add_rmsnorm(res2, p2, g2, 1e-6, torch.float32, rows), want, 2e-6, "gathered rows over parts")
+
+
 def test_add_rmsnorm_fused_equals_unfused_bit_for_bit(ops):
     # src/ops/norm.rs:84-98
     a, r = t([[0.5, -1.0, 2.0, 0.25]]), t([[1.0, 1.0, -1.0, 0.0]])
@@ -375,6 +391,10 @@ def test_gemm_skinny_packed_bf16(ops, m, n, k):
     y = f64(x) @ f64(wgu).T
     close(ops.gemm_skinny_packed_bf16(x, ops.pack_for_mfma(wgu, swiglu=True), n, torch.bfloat16, swiglu=True),
           P.silu(y[:, :n]) * y[:, n:], 5e-3, "packed, with swiglu")
+    for parts in (2, 3):                                   # K cut in pieces: the pieces add up to the product
+        got = ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32, parts=parts)
+        assert got.shape == (parts, m, n)
+        close(got.sum(0), want, 3e-6, f"{parts} parts of K")
 
 
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 1e-6), (torch.bfloat16, 5e-3)])
