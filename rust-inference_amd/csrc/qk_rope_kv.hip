@@ -1,5 +1,6 @@
 // Per-head q/k RMSNorm, rotate-half position encoding and the write of keys and values into
-// their pages, in one pass over the fused qkv projection.  One workgroup per token.
+// their pages, in one pass over the fused qkv projection.  One wavefront per (token, head) in the
+// general kernel; prompts of head sizes that allow it go through the 16-byte kernels further down.
 //
 // The reference does this in four launches and rounds to 16 bits after each
 // (src/cuda/kernels.cu:98-108 norm, :127-142 rotation, :322-336 page write); here a q or k
@@ -8,98 +9,70 @@
 #include "common.h"
 
 #define QK_MAX_PAIRS 4   // pairs per lane: head_dim / 2 <= 64 * QK_MAX_PAIRS
-#define QK_BATCH 4       // heads a wavefront loads together
 
-// One workgroup of four wavefronts per token: the token's sines and cosines are made once and shared
-// by all its heads through LDS; each wavefront then takes every fourth head.
 template <typename TA, typename TC>
-__global__ void __launch_bounds__(256)
-qk_norm_rope_kv_write_kernel(
+__global__ void qk_norm_rope_kv_write_kernel(
     TA* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ inv_freq, const int32_t* __restrict__ tok_pos,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table, int table_width,
     TC* __restrict__ k_pages, TC* __restrict__ v_pages, int tokens, int heads, int kv_heads, int head_dim,
     int page_size) {
-    __shared__ float cs_lds[RI_WAVE * QK_MAX_PAIRS], sn_lds[RI_WAVE * QK_MAX_PAIRS];
-    const int lane = threadIdx.x & (RI_WAVE - 1), wave = threadIdx.x / RI_WAVE;
+    const int lane = threadIdx.x & (RI_WAVE - 1);
+    const int waves_per_block = blockDim.x / RI_WAVE;
     const int all_heads = heads + 2 * kv_heads;
-    const int t = blockIdx.x;
+    const long item = (long)blockIdx.x * waves_per_block + threadIdx.x / RI_WAVE;
+    if (item >= (long)tokens * all_heads) return;          // whole wavefront leaves together
+    const int t = (int)(item / all_heads), hh = (int)(item % all_heads);
     const int half = head_dim / 2;
-    const int pos = tok_pos[t];
-    const int page = kv_heads > 0 ? page_table[(size_t)tok_seq[t] * table_width + pos / page_size] : 0;
-    if (inv_freq) {
-        // angle = f32(pos) * inv_freq[i] as a float32 product (the reference: src/ops/rope.rs:39)
-        for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf((float)pos * inv_freq[i], &sn_lds[i], &cs_lds[i]);
-    }
-    __syncthreads();
-    TA* row = qkv + (size_t)t * all_heads * head_dim;
+    TA* x = qkv + (size_t)t * all_heads * head_dim + (size_t)hh * head_dim;
 
-    // Each wavefront takes QK_BATCH consecutive heads at a time and loads them all before it works on
-    // any: the loads of a token's heads are in flight together.
-    for (int h0 = wave * QK_BATCH; h0 < all_heads; h0 += 4 * QK_BATCH) {
-        float x1[QK_BATCH][QK_MAX_PAIRS], x2[QK_BATCH][QK_MAX_PAIRS];
-#pragma unroll
-        for (int hb = 0; hb < QK_BATCH; ++hb) {
-            const int hh = h0 + hb;
-            const TA* x = row + (size_t)min(hh, all_heads - 1) * head_dim;
-#pragma unroll
-            for (int j = 0; j < QK_MAX_PAIRS; ++j) {
-                const int i = lane + j * RI_WAVE;
-                x1[hb][j] = x2[hb][j] = 0.f;
-                if (i < half && hh < all_heads) {
-                    x1[hb][j] = to_f32(x[i]);
-                    x2[hb][j] = to_f32(x[i + half]);
-                }
-            }
+    const int pos = tok_pos[t];
+    TC* dst = nullptr;          // where a k head goes
+    if (hh >= heads) {
+        const int kvh = (hh - heads) % kv_heads;
+        const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
+        const size_t head_base = ((size_t)page * kv_heads + kvh) * page_size * head_dim;
+        if (hh >= heads + kv_heads) {
+            // v: a copy, no norm and no rotation, transposed inside the page: [head_dim][page_size]
+            TC* vt = v_pages + head_base + pos % page_size;
+            for (int d = lane; d < head_dim; d += RI_WAVE) from_f32(vt + (size_t)d * page_size, to_f32(x[d]));
+            return;
         }
+        dst = k_pages + head_base + (size_t)(pos % page_size) * head_dim;
+    }
+
+    // lane owns pairs i = lane, lane + 64, ...: elements (i, i + half)
+    float x1[QK_MAX_PAIRS], x2[QK_MAX_PAIRS];
+    float ss = 0.f;
 #pragma unroll
-        for (int hb = 0; hb < QK_BATCH; ++hb) {
-            const int hh = h0 + hb;
-            if (hh >= all_heads) break;
-            TA* x = row + (size_t)hh * head_dim;
-            TC* dst = nullptr;          // where a k head goes
-            if (hh >= heads) {
-                const int kvh = (hh - heads) % kv_heads;
-                const size_t head_base = ((size_t)page * kv_heads + kvh) * page_size * head_dim;
-                if (hh >= heads + kv_heads) {
-                    // v: a copy, no norm and no rotation, transposed inside the page: [head_dim][page_size]
-                    TC* vt = v_pages + head_base + pos % page_size;
-#pragma unroll
-                    for (int j = 0; j < QK_MAX_PAIRS; ++j) {
-                        const int i = lane + j * RI_WAVE;
-                        if (i < half) {
-                            from_f32(vt + (size_t)i * page_size, x1[hb][j]);
-                            from_f32(vt + (size_t)(i + half) * page_size, x2[hb][j]);
-                        }
-                    }
-                    continue;
-                }
-                dst = k_pages + head_base + (size_t)(pos % page_size) * head_dim;
-            }
-            // lane owns pairs i = lane, lane + 64, ...: elements (i, i + half)
-            float ss = 0.f;
-#pragma unroll
-            for (int j = 0; j < QK_MAX_PAIRS; ++j) ss += x1[hb][j] * x1[hb][j] + x2[hb][j] * x2[hb][j];
-            const float* gain = hh < heads ? q_gain : k_gain;
-            float inv = 1.0f;
-            if (gain) inv = 1.0f / sqrtf(wave_sum(ss) / (float)head_dim + eps);
-#pragma unroll
-            for (int j = 0; j < QK_MAX_PAIRS; ++j) {
-                const int i = lane + j * RI_WAVE;
-                if (i >= half) continue;
-                float a = x1[hb][j], b = x2[hb][j];
-                if (gain) { a = a * inv * gain[i]; b = b * inv * gain[i + half]; }
-                // pairs (i, i + half): x'[i] = x[i] cos - x[i+half] sin, x'[i+half] = x[i+half] cos + x[i] sin
-                // (the reference: src/ops/rope.rs:73-74)
-                if (inv_freq) {
-                    const float cs = cs_lds[i], sn = sn_lds[i];
-                    const float ra = a * cs - b * sn, rb = b * cs + a * sn;
-                    a = ra; b = rb;
-                }
-                if (dst) { from_f32(dst + i, a); from_f32(dst + i + half, b); }
-                else     { from_f32(x + i, a);   from_f32(x + i + half, b); }
-            }
+    for (int j = 0; j < QK_MAX_PAIRS; ++j) {
+        const int i = lane + j * RI_WAVE;
+        x1[j] = x2[j] = 0.f;
+        if (i < half) {
+            x1[j] = to_f32(x[i]);
+            x2[j] = to_f32(x[i + half]);
+            ss += x1[j] * x1[j] + x2[j] * x2[j];
         }
+    }
+    const float* gain = hh < heads ? q_gain : k_gain;
+    float inv = 1.0f;
+    if (gain) inv = 1.0f / sqrtf(wave_sum(ss) / (float)head_dim + eps);
+#pragma unroll
+    for (int j = 0; j < QK_MAX_PAIRS; ++j) {
+        const int i = lane + j * RI_WAVE;
+        if (i >= half) continue;
+        float a = x1[j], b = x2[j];
+        if (gain) { a = a * inv * gain[i]; b = b * inv * gain[i + half]; }
+        // pairs (i, i + half); angle = f32(pos) * inv_freq[i] as a float32 product
+        // (the reference: src/ops/rope.rs:39, :73-74)
+        if (inv_freq) {
+            float sn, cs;
+            sincosf((float)pos * inv_freq[i], &sn, &cs);
+            const float ra = a * cs - b * sn, rb = b * cs + a * sn;
+            a = ra; b = rb;
+        }
+        if (dst) { from_f32(dst + i, a); from_f32(dst + i + half, b); }
+        else     { from_f32(x + i, a);   from_f32(x + i + half, b); }
     }
 }
 
@@ -241,7 +214,9 @@ static void launch_qk(void* qkv, const float* q_gain, const float* k_gain, float
                       int seqs, int max_new, const int32_t* page_table, int table_width, void* k_pages,
                       void* v_pages, int tokens, int heads, int kv_heads, int head_dim, int page_size,
                       hipStream_t s) {
-    if (cu_seqlens && vec_path_fits(head_dim, page_size)) {
+    // one new token per sequence: a single launch that writes the few values element by element is cheaper
+    // than two
+    if (cu_seqlens && max_new > 1 && vec_path_fits(head_dim, page_size)) {
         qk_norm_rope_k_write_vec_kernel<TA, TC><<<tokens, 256, head_dim * sizeof(float), s>>>(
             (TA*)qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, table_width, (TC*)k_pages, heads,
             kv_heads, head_dim, page_size);
@@ -252,7 +227,9 @@ static void launch_qk(void* qkv, const float* q_gain, const float* k_gain, float
             page_size);
         return;
     }
-    qk_norm_rope_kv_write_kernel<TA, TC><<<tokens, 4 * RI_WAVE, 0, s>>>(
+    const long items = (long)tokens * (heads + 2 * kv_heads);
+    const int waves = 4;
+    qk_norm_rope_kv_write_kernel<TA, TC><<<(unsigned)((items + waves - 1) / waves), waves * RI_WAVE, 0, s>>>(
         (TA*)qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, table_width,
         (TC*)k_pages, (TC*)v_pages, tokens, heads, kv_heads, head_dim, page_size);
 }
@@ -271,6 +248,7 @@ extern "C" int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q
                "qk_norm_rope_kv_write: rotation of %d of %d elements: only whole heads are rotated here", rot_dim,
                head_dim);
     RI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "qk_norm_rope_kv_write: page geometry");
+    RI_REQUIRE((long)tokens * (heads + 2 * kv_heads) / 4 < 2147483647L, "qk_norm_rope_kv_write: too many tokens");
     RI_REQUIRE(!cu_seqlens || (seqs > 0 && seqs <= 65535 && max_new > 0 && kv_heads <= 65535),
                "qk_norm_rope_kv_write: seqs %d, max_new %d", seqs, max_new);
     RI_REQUIRE(act_dtype == cache_dtype && (act_dtype == RI_F32 || act_dtype == RI_BF16),
