@@ -1,8 +1,8 @@
 // Decode-size products for bfloat16: out[M, N] = x[M, K] . w[N, K]^T with M <= 8 rows of x.
-// The weights are the traffic: each wavefront streams whole rows of w with 16-byte loads and keeps
-// M float32 accumulators, so every weight byte is read once per call.  Optional SwiGLU epilogue for
-// the fused gate|up matrix.  Lane l owns k = 8 * (l + 64 * i) ..+8: the order of each row's sum is
-// fixed by K alone.
+// The weights are the traffic: each wavefront streams a row of w (or a fixed share of one) with
+// 16-byte loads and keeps M float32 accumulators, so every weight byte is read once per call.
+// Optional SwiGLU epilogue for the fused gate|up matrix.  Lane l owns k = 8 * (l + 64 * i) ..+8: the
+// order of each row's sum is fixed by K and N alone.
 #include "api.h"
 #include "common.h"
 
@@ -19,49 +19,101 @@ __device__ __forceinline__ void unpack8(const uint4 v, float* o) {
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-template <int MT, bool SWIGLU, typename TO>
+// KS wavefronts share a row, each taking a contiguous 1/KS of K (a multiple of 512 elements, so that
+// every lane's 16-byte pieces stay aligned and the split depends on K alone); their sums are added
+// through LDS in wavefront order.  More wavefronts in flight per byte: it pays when the matrix has few
+// rows or long ones.
+template <int MT, bool SWIGLU, typename TO, int KS>
 __global__ void __launch_bounds__(GV_WAVES * RI_WAVE)
 gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K) {
+    __shared__ float red[2][GV_WAVES][MT];
     const int lane = threadIdx.x & (RI_WAVE - 1);
-    const int n = blockIdx.x * GV_WAVES + threadIdx.x / RI_WAVE;
-    if (n >= N) return;
-    const bf16_t* wr = w + (size_t)n * K;
-    const bf16_t* wu = SWIGLU ? w + (size_t)(N + n) * K : nullptr;
+    const int wave = threadIdx.x / RI_WAVE;
+    const int n = blockIdx.x * (GV_WAVES / KS) + wave / KS;
+    const int part = wave % KS;
+    const int slice = ((K + KS - 1) / KS + 511) / 512 * 512;
+    const int k_begin = part * slice, k_end = min(K, k_begin + slice);
+    const bool row_ok = n < N;
+    const bf16_t* wr = w + (size_t)(row_ok ? n : 0) * K;
+    const bf16_t* wu = SWIGLU ? w + (size_t)(N + (row_ok ? n : 0)) * K : nullptr;
     float acc[MT] = {}, accu[MT] = {};
-    for (int k = lane * 8; k < K; k += RI_WAVE * 8) {
-        float wv[8], uv[8];
-        unpack8(*reinterpret_cast<const uint4*>(wr + k), wv);
-        if (SWIGLU) unpack8(*reinterpret_cast<const uint4*>(wu + k), uv);
+    if (row_ok) {
+        for (int k = k_begin + lane * 8; k < k_end; k += RI_WAVE * 8) {
+            float wv[8], uv[8];
+            unpack8(*reinterpret_cast<const uint4*>(wr + k), wv);
+            if (SWIGLU) unpack8(*reinterpret_cast<const uint4*>(wu + k), uv);
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            if (m < M) {
-                float xv[8];
-                unpack8(*reinterpret_cast<const uint4*>(x + (size_t)m * K + k), xv);
+            for (int m = 0; m < MT; ++m) {
+                if (m < M) {
+                    float xv[8];
+                    unpack8(*reinterpret_cast<const uint4*>(x + (size_t)m * K + k), xv);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    acc[m] = fmaf(xv[e], wv[e], acc[m]);
-                    if (SWIGLU) accu[m] = fmaf(xv[e], uv[e], accu[m]);
+                    for (int e = 0; e < 8; ++e) {
+                        acc[m] = fmaf(xv[e], wv[e], acc[m]);
+                        if (SWIGLU) accu[m] = fmaf(xv[e], uv[e], accu[m]);
+                    }
                 }
             }
         }
     }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        const float g = wave_sum(acc[m]);
-        const float u = SWIGLU ? wave_sum(accu[m]) : 0.f;
-        if (lane == 0 && m < M) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_f(g) * u : g);
+        acc[m] = wave_sum(acc[m]);
+        if (SWIGLU) accu[m] = wave_sum(accu[m]);
     }
+    if (KS > 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                red[0][wave][m] = acc[m];
+                if (SWIGLU) red[1][wave][m] = accu[m];
+            }
+        }
+        __syncthreads();
+        if (part != 0) return;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            acc[m] = 0.f;
+            accu[m] = 0.f;
+            for (int p = 0; p < KS; ++p) {
+                acc[m] += red[0][wave + p][m];
+                if (SWIGLU) accu[m] += red[1][wave + p][m];
+            }
+        }
+    }
+    if (lane == 0 && row_ok) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            if (m < M) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_f(acc[m]) * accu[m] : acc[m]);
+    }
+}
+
+// How many wavefronts share a row: measured on MI355X with one row of x (decode at batch 1).
+static int gemv_k_split(int n, int k) {
+    if (k >= 8192) return 4;
+    if ((long)n * k <= 4096L * 4096L) return 2;
+    return 1;
+}
+
+template <int MT, bool SWIGLU, int KS>
+static void launch_gemv_ks(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, hipStream_t s) {
+    const int rows_per_wg = GV_WAVES / KS;
+    const unsigned grid = (n + rows_per_wg - 1) / rows_per_wg;
+    if (out_dtype == RI_F32)
+        gemv_bf16_kernel<MT, SWIGLU, float, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((float*)out, (const bf16_t*)x,
+                                                                                    (const bf16_t*)w, m, n, k);
+    else
+        gemv_bf16_kernel<MT, SWIGLU, bf16_t, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((bf16_t*)out, (const bf16_t*)x,
+                                                                                     (const bf16_t*)w, m, n, k);
 }
 
 template <int MT, bool SWIGLU>
 static void launch_gemv(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, hipStream_t s) {
-    const unsigned grid = (n + GV_WAVES - 1) / GV_WAVES;
-    if (out_dtype == RI_F32)
-        gemv_bf16_kernel<MT, SWIGLU, float><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((float*)out, (const bf16_t*)x,
-                                                                                (const bf16_t*)w, m, n, k);
-    else
-        gemv_bf16_kernel<MT, SWIGLU, bf16_t><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((bf16_t*)out, (const bf16_t*)x,
-                                                                                 (const bf16_t*)w, m, n, k);
+    switch (gemv_k_split(n, k)) {
+        case 4: launch_gemv_ks<MT, SWIGLU, 4>(out, out_dtype, x, w, m, n, k, s); break;
+        case 2: launch_gemv_ks<MT, SWIGLU, 2>(out, out_dtype, x, w, m, n, k, s); break;
+        default: launch_gemv_ks<MT, SWIGLU, 1>(out, out_dtype, x, w, m, n, k, s); break;
+    }
 }
 
 extern "C" int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
