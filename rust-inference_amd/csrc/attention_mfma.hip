@@ -346,15 +346,7 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     const int tok = b;                                       // one new token per sequence: token b is sequence b's
     const int qpos = tok_pos[tok];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) {          // whole workgroup
-        // no key of this chunk is visible: say so, and the join need not know the positions
-        if (threadIdx.x < group) {
-            float* dst = ws + (((long)b * heads + kvh * group + threadIdx.x) * max_chunks + chunk) * (DH + 2);
-            dst[DH] = -INFINITY;
-            dst[DH + 1] = 0.f;
-        }
-        return;
-    }
+    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
 
     const int page = chunk * (DECODE_CHUNK / PAGE) + wave;   // this wavefront's page
     const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
@@ -405,18 +397,23 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     }
 }
 
+// The join reads only the chunks that hold visible keys (it takes the position for that: reading every
+// chunk's marker instead was tried and was slower).
 template <int DH>
 __global__ void __launch_bounds__(DH)
-attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, int heads, int max_chunks) {
+attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
+                        int heads, int window, int max_chunks) {
     const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;      // token b is sequence b's one new token
+    const int qpos = tok_pos[b];
+    const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
+    const int c_lo = lo / DECODE_CHUNK, c_hi = qpos / DECODE_CHUNK;
     const float* base = ws + ((long)b * heads + h) * max_chunks * (DH + 2);
     float m = -INFINITY;
-    for (int c = 0; c < max_chunks; ++c) m = fmaxf(m, base[c * (DH + 2) + DH]);
+    for (int c = c_lo; c <= c_hi; ++c) m = fmaxf(m, base[c * (DH + 2) + DH]);
     float acc = 0.f, l = 0.f;
-    for (int c = 0; c < max_chunks; ++c) {                          // always in chunk order
+    for (int c = c_lo; c <= c_hi; ++c) {                            // always in chunk order
         const float mc = base[c * (DH + 2) + DH];
-        if (mc == -INFINITY) continue;                              // a chunk without a visible key
-        const float f = exp2f(mc - m);
+        const float f = mc == -INFINITY ? 0.f : exp2f(mc - m);
         acc += base[c * (DH + 2) + d] * f;
         l += base[c * (DH + 2) + DH + 1] * f;
     }
@@ -478,15 +475,7 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
     const int group = heads / kv_heads;
     const int qpos = tok_pos[b];                             // token b is sequence b's one new token
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) {          // whole workgroup
-        // no key of this chunk is visible: say so, and the join need not know the positions
-        if (threadIdx.x < group) {
-            float* dst = ws + (((long)b * heads + kvh * group + threadIdx.x) * max_chunks + chunk) * (DH + 2);
-            dst[DH] = -INFINITY;
-            dst[DH + 1] = 0.f;
-        }
-        return;
-    }
+    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
     const bool owner = chunk == qpos / DECODE_CHUNK;         // this chunk holds the new token's position
 
     // 1. this wavefront's page is on its way while the queries are made
@@ -653,7 +642,8 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
         attn_decode_mfma_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                           \
             workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
             tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks);                   \
-        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, heads, max_chunks); \
+        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos, heads,    \
+                                                                      window, max_chunks);                        \
         break;
     switch (head_dim) {
         RI_DECODE_CASE(32)
@@ -689,7 +679,8 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
         attn_decode_fused_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                          \
             workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq, (bf16_t*)k_pages,             \
             (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks); \
-        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, heads, max_chunks); \
+        attn_decode_join_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos, heads,    \
+                                                                      window, max_chunks);                        \
         break;
     switch (head_dim) {
         RI_FUSED_CASE(32)
