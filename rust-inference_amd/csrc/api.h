@@ -97,6 +97,24 @@ int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, 
 int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
                                int swiglu, int parts, void* stream);
 
+// The two decode-size products linked to the RMSNorms around them, so that those need no kernels of their
+// own.  W . norm(r) with norm(r) = r * inv * g equals inv * (W . (r * g)), inv = 1 / sqrt(mean(r^2) + eps):
+//   consumer side (ssq_in != NULL): x holds bfloat16(r * g) and ssq_in[m][n_in] partial sums of r[m]^2 over
+//     a row of `dim` elements; the result rows are scaled by inv (before the activation with swiglu).
+//   producer side (residual != NULL): the result is added into residual[m][n] (float32, in place), the new
+//     value times next_gain[n] goes to xg_out[m][n] (bfloat16) and each workgroup's sum of its squares to
+//     ssq_out[m][partials]; out is not written.  No swiglu on this side.
+// ri_*_partials: the number of partial sums a row gets from a product with these sizes.
+int ri_gemv_bf16_partials(int n, int k);
+int ri_gemv_bf16_linked(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
+                        const float* ssq_in, int n_in, float eps, int dim, float* residual, const float* next_gain,
+                        void* xg_out, float* ssq_out, void* stream);
+int ri_gemm_skinny_packed_bf16_partials(int n);
+int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
+                                      int k, int swiglu, const float* ssq_in, int n_in, float eps, int dim,
+                                      float* residual, const float* next_gain, void* xg_out, float* ssq_out,
+                                      void* stream);
+
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);
 

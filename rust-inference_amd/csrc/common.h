@@ -73,6 +73,26 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return total;
 }
 
+// How a decode-size product is linked to the RMSNorms around it, so that the norms need no kernels
+// of their own.  y = W . norm(r) with norm(r) = r * inv * g is computed as inv * (W . (r * g)): the
+// producer of r leaves xg = bfloat16(r * g) and partial sums of r^2; the consumer adds the partial
+// sums up (always in the same order), and scales its result rows by inv = 1 / sqrt(mean(r^2) + eps).
+struct NormLink {
+    // consumer side: the rows of x are xg, not yet scaled.  ssq_in: [M][n_in] partial sums of squares over
+    // a row of `dim` elements; NULL: x is what it is.
+    const float* ssq_in;
+    int n_in;
+    float eps;
+    int dim;
+    // producer side: the result is a branch's output.  residual[m][n] += result (float32, in place),
+    // xg_out[m][n] = bfloat16(residual * next_gain[n]), ssq_out[m][workgroup] = the workgroup's sum of
+    // residual^2; NULL: the result is stored as it is.
+    float* residual;
+    const float* next_gain;
+    bf16_t* xg_out;
+    float* ssq_out;
+};
+
 // ---- host side: error text of the last refused or failed call (per thread)
 void ri_set_error(const char* fmt, ...);
 

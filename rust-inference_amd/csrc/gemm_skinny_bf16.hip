@@ -79,11 +79,16 @@ gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
 // row l % 16, k 8 * (l / 16) ..+8), tiles of one row block consecutive in k.  A wavefront's loads are
 // then whole contiguous kilobytes, which is what the memory system streams fastest.
 // packed: [row_tiles][k_tiles][64 lanes][8]; for SwiGLU the up matrix's tiles follow the gate's.
+#define SK_ROWS (16 / SK_WAVES)   // rows of x whose sums of squares one wavefront adds up
+#define SK_PRE 4                  // partial sums of squares a lane fetches ahead of the weights
+
 template <int SK_WAVES, bool SWIGLU, typename TO>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked,
-                          int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset) {
+                          int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset, NormLink link) {
     __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][4][64];
+    __shared__ float inv_lds[16];
+    __shared__ float sq_lds[16][17];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, jg = lane >> 4;
@@ -99,16 +104,40 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     const bf16_t* xp = x + (size_t)(x_ok ? i : 0) * K + jg * 8;
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
+    // Loads whose values are wanted only after the weights have streamed are issued here, so that their
+    // latency hides behind the stream.  Partial sums of squares: wavefront w has the rows w, w + SK_WAVES, ...,
+    // each lane SK_PRE of a row's partial sums (more are fetched afterwards).  And the element of the
+    // residual stream and the gain that this thread's result meets.
+    float pre[SK_ROWS][SK_PRE];
+    if (link.ssq_in) {
+#pragma unroll
+        for (int j = 0; j < SK_ROWS; ++j)
+#pragma unroll
+            for (int q = 0; q < SK_PRE; ++q) {
+                const int m = wave + j * SK_WAVES, p = lane + q * 64;
+                pre[j][q] = (m < M && p < link.n_in) ? link.ssq_in[(size_t)m * link.n_in + p] : 0.f;
+            }
+    }
+    const int t = threadIdx.x;
+    const int ln = t & 63, r = (t >> 6) & 3;
+    const int nl = 4 * (ln >> 4) + r, n = nt * 16 + nl, m = ln & 15;      // D[row n, column m]
+    const bool ok = m < M && n < N;
+    float res_pre = 0.f, gain_pre = 0.f;
+    if (link.residual && t < 256 && ok) {
+        res_pre = link.residual[(size_t)m * N + n];
+        gain_pre = link.next_gain[n];
+    }
+
     floatx4 acc = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
     for (int kt = kt_begin; kt < kt_end; kt += SK_CHUNK) {
         Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];
 #pragma unroll
         for (int c = 0; c < SK_CHUNK; ++c) {
-            const bool ok = kt + c < kt_end;
-            wf[c].u = ok ? *reinterpret_cast<const uint4*>(wp + (size_t)(kt + c) * 512) : zero;
-            if (SWIGLU) uf[c].u = ok ? *reinterpret_cast<const uint4*>(up + (size_t)(kt + c) * 512) : zero;
+            const bool live = kt + c < kt_end;
+            wf[c].u = live ? *reinterpret_cast<const uint4*>(wp + (size_t)(kt + c) * 512) : zero;
+            if (SWIGLU) uf[c].u = live ? *reinterpret_cast<const uint4*>(up + (size_t)(kt + c) * 512) : zero;
             // the packed matrix is zero beyond K; x is not padded
-            xf[c].u = (ok && x_ok && (kt + c) * 32 + jg * 8 < K) ? *reinterpret_cast<const uint4*>(xp + (kt + c) * 32)
+            xf[c].u = (live && x_ok && (kt + c) * 32 + jg * 8 < K) ? *reinterpret_cast<const uint4*>(xp + (kt + c) * 32)
                                                                  : zero;
         }
 #pragma unroll
@@ -118,22 +147,58 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
         }
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        red[0][wave][r][lane] = acc[r];
-        if (SWIGLU) red[1][wave][r][lane] = accu[r];
+    for (int e = 0; e < 4; ++e) {
+        red[0][wave][e][lane] = acc[e];
+        if (SWIGLU) red[1][wave][e][lane] = accu[e];
+    }
+    // rows of x that still want their 1 / rms: the lanes' shares in the order of wave_sum, the same in every
+    // workgroup
+    if (link.ssq_in) {
+#pragma unroll
+        for (int j = 0; j < SK_ROWS; ++j) {
+            const int mr = wave + j * SK_WAVES;
+            if (mr < M) {
+                float sq = 0.f;
+#pragma unroll
+                for (int q = 0; q < SK_PRE; ++q) sq += pre[j][q];
+                for (int p = lane + SK_PRE * 64; p < link.n_in; p += 64) sq += link.ssq_in[(size_t)mr * link.n_in + p];
+                sq = wave_sum(sq);
+                if (lane == 0) inv_lds[mr] = 1.0f / sqrtf(sq / (float)link.dim + link.eps);
+            }
+        }
     }
     __syncthreads();
-    const int t = threadIdx.x;
     if (t < 256) {
-        const int ln = t & 63, r = t >> 6;
         float g = 0.f, u = 0.f;
 #pragma unroll
         for (int wv = 0; wv < SK_WAVES; ++wv) {
             g += red[0][wv][r][ln];
             if (SWIGLU) u += red[1][wv][r][ln];
         }
-        const int n = nt * 16 + 4 * (ln >> 4) + r, m = ln & 15;
-        if (m < M && n < N) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_sk(g) * u : g);
+        if (link.ssq_in && m < M) {
+            g *= inv_lds[m];
+            u *= inv_lds[m];
+        }
+        float v = SWIGLU ? silu_sk(g) * u : g;
+        if (link.residual) {
+            if (ok) {
+                const size_t at = (size_t)m * N + n;
+                v += res_pre;
+                link.residual[at] = v;                   // this element belongs to this thread alone
+                link.xg_out[at] = f32_to_bf16(v * gain_pre);
+            }
+            sq_lds[m][nl] = ok ? v * v : 0.f;
+        } else if (ok) {
+            from_f32(out + (size_t)m * N + n, v);
+        }
+    }
+    if (link.residual) {                                 // the workgroup's share of every row's sum of squares
+        __syncthreads();
+        if (t < M) {
+            float total = 0.f;
+            for (int c = 0; c < 16; ++c) total += sq_lds[t][c];
+            link.ssq_out[(size_t)t * gridDim.x + blockIdx.x] = total;
+        }
     }
 }
 
@@ -143,17 +208,33 @@ static int skinny_waves(int n, int k) { return k >= 8192 ? 8 : 4; }
 
 template <int WAVES, bool SWIGLU>
 static void launch_packed(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts,
-                          hipStream_t s) {
+                          const NormLink& link, hipStream_t s) {
     const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
     const int part_tiles = (k_tiles + parts - 1) / parts;
     const int tiles_per_wave = (part_tiles + WAVES - 1) / WAVES;
     dim3 grid(row_tiles, parts);
     if (out_dtype == RI_F32)
         gemm_skinny_packed_kernel<WAVES, SWIGLU, float><<<grid, WAVES * 64, 0, s>>>(
-            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link);
     else
         gemm_skinny_packed_kernel<WAVES, SWIGLU, bf16_t><<<grid, WAVES * 64, 0, s>>>(
-            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link);
+}
+
+static int packed_run(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k, int swiglu,
+                      int parts, const NormLink& link, hipStream_t s) {
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)wpacked;
+    const bool eight = skinny_waves(n, (k + parts - 1) / parts) == 8;
+    if (swiglu) {
+        if (eight) launch_packed<8, true>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
+        else       launch_packed<4, true>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
+    } else {
+        if (eight) launch_packed<8, false>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
+        else       launch_packed<4, false>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
+    }
+    RI_LAUNCH_CHECK("gemm_skinny_packed_bf16");
+    return 0;
 }
 
 extern "C" int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
@@ -163,19 +244,29 @@ extern "C" int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* 
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_packed_bf16: out dtype %d", out_dtype);
     RI_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || (!swiglu && out_dtype == RI_F32)),
                "gemm_skinny_packed_bf16: %d parts of K (more than one needs float32 sums and no activation)", parts);
-    hipStream_t s = (hipStream_t)stream;
-    const bf16_t* xb = (const bf16_t*)x;
-    const bf16_t* wb = (const bf16_t*)wpacked;
-    const bool eight = skinny_waves(n, (k + parts - 1) / parts) == 8;
-    if (swiglu) {
-        if (eight) launch_packed<8, true>(out, out_dtype, xb, wb, m, n, k, parts, s);
-        else       launch_packed<4, true>(out, out_dtype, xb, wb, m, n, k, parts, s);
-    } else {
-        if (eight) launch_packed<8, false>(out, out_dtype, xb, wb, m, n, k, parts, s);
-        else       launch_packed<4, false>(out, out_dtype, xb, wb, m, n, k, parts, s);
-    }
-    RI_LAUNCH_CHECK("gemm_skinny_packed_bf16");
-    return 0;
+    NormLink link = {};
+    return packed_run(out, out_dtype, x, wpacked, m, n, k, swiglu, parts, link, (hipStream_t)stream);
+}
+
+// Number of workgroups (and so of partial sums of squares per row) of a linked product with n output columns.
+extern "C" int ri_gemm_skinny_packed_bf16_partials(int n) { return (n + 15) / 16; }
+
+extern "C" int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, const void* wpacked, int m,
+                                                 int n, int k, int swiglu, const float* ssq_in, int n_in, float eps,
+                                                 int dim, float* residual, const float* next_gain, void* xg_out,
+                                                 float* ssq_out, void* stream) {
+    RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_packed_bf16_linked: %d rows of x, this kernel takes 1 to 16", m);
+    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_packed_bf16_linked: n %d, k %d (k must be a multiple of 8)", n,
+               k);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_packed_bf16_linked: out dtype %d", out_dtype);
+    RI_REQUIRE(!ssq_in || (n_in > 0 && dim > 0), "gemm_skinny_packed_bf16_linked: %d partial sums over %d elements", n_in,
+               dim);
+    RI_REQUIRE(!residual || (next_gain && xg_out && ssq_out && !swiglu),
+               "gemm_skinny_packed_bf16_linked: a product that feeds the residual stream needs the next gain and both "
+               "outputs");
+    RI_REQUIRE(residual || out, "gemm_skinny_packed_bf16_linked: no output");
+    NormLink link = {ssq_in, n_in, eps, dim, residual, next_gain, (bf16_t*)xg_out, ssq_out};
+    return packed_run(out, out_dtype, x, wpacked, m, n, k, swiglu, 1, link, (hipStream_t)stream);
 }
 
 template <int WAVES, bool SWIGLU>

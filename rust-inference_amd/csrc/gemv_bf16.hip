@@ -23,10 +23,15 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 // every lane's 16-byte pieces stay aligned and the split depends on K alone); their sums are added
 // through LDS in wavefront order.  More wavefronts in flight per byte: it pays when the matrix has few
 // rows or long ones.
+#define GV_PRE 4              // partial sums of squares a thread fetches ahead of the weights
+
 template <int MT, bool SWIGLU, typename TO, int KS>
 __global__ void __launch_bounds__(GV_WAVES * RI_WAVE)
-gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K) {
+gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K,
+                 NormLink link) {
     __shared__ float red[2][GV_WAVES][MT];
+    __shared__ float scratch[16];
+    __shared__ float sq_lds[GV_WAVES][MT];
     const int lane = threadIdx.x & (RI_WAVE - 1);
     const int wave = threadIdx.x / RI_WAVE;
     const int n = blockIdx.x * (GV_WAVES / KS) + wave / KS;
@@ -36,6 +41,27 @@ gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_
     const bool row_ok = n < N;
     const bf16_t* wr = w + (size_t)(row_ok ? n : 0) * K;
     const bf16_t* wu = SWIGLU ? w + (size_t)(N + (row_ok ? n : 0)) * K : nullptr;
+
+    // Loads whose values are wanted only after the weights have streamed are issued here, so that their
+    // latency hides behind the stream: a row's partial sums of squares (up to GV_PRE per thread; more are
+    // fetched afterwards), and the element of the residual stream and the gain that the result meets.
+    float pre[MT][GV_PRE];
+    if (link.ssq_in) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < GV_PRE; ++j) {
+                const int p = threadIdx.x + j * GV_WAVES * RI_WAVE;
+                pre[m][j] = (m < M && p < link.n_in) ? link.ssq_in[(size_t)m * link.n_in + p] : 0.f;
+            }
+    }
+    float res_pre[MT], gain_pre = 0.f;
+    if (link.residual && row_ok && part == 0) {
+        gain_pre = link.next_gain[n];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) res_pre[m] = m < M ? link.residual[(size_t)m * N + n] : 0.f;
+    }
+
     float acc[MT] = {}, accu[MT] = {};
     if (row_ok) {
         for (int k = k_begin + lane * 8; k < k_end; k += RI_WAVE * 8) {
@@ -70,21 +96,64 @@ gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_
             }
         }
         __syncthreads();
-        if (part != 0) return;
+        if (part == 0) {
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            acc[m] = 0.f;
-            accu[m] = 0.f;
-            for (int p = 0; p < KS; ++p) {
-                acc[m] += red[0][wave + p][m];
-                if (SWIGLU) accu[m] += red[1][wave + p][m];
+            for (int m = 0; m < MT; ++m) {
+                acc[m] = 0.f;
+                accu[m] = 0.f;
+                for (int p = 0; p < KS; ++p) {
+                    acc[m] += red[0][wave + p][m];
+                    if (SWIGLU) accu[m] += red[1][wave + p][m];
+                }
             }
         }
     }
-    if (lane == 0 && row_ok) {
+    // rows of x that still want their 1 / rms: add up the partial sums of squares, always in this order
+    float inv[MT];
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
-            if (m < M) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_f(acc[m]) * accu[m] : acc[m]);
+    for (int m = 0; m < MT; ++m) inv[m] = 1.0f;
+    if (link.ssq_in) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (m < M) {
+                float sq = 0.f;
+#pragma unroll
+                for (int j = 0; j < GV_PRE; ++j) sq += pre[m][j];
+                for (int p = threadIdx.x + GV_PRE * GV_WAVES * RI_WAVE; p < link.n_in; p += GV_WAVES * RI_WAVE)
+                    sq += link.ssq_in[(size_t)m * link.n_in + p];
+                inv[m] = 1.0f / sqrtf(block_sum(sq, scratch) / (float)link.dim + link.eps);
+            }
+        }
+    }
+    const bool writer = lane == 0 && row_ok && part == 0;
+    float sq[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        sq[m] = 0.f;
+        if (writer && m < M) {
+            float v = SWIGLU ? silu_f(acc[m] * inv[m]) * (accu[m] * inv[m]) : acc[m] * inv[m];
+            if (link.residual) {
+                const size_t at = (size_t)m * N + n;
+                v += res_pre[m];
+                link.residual[at] = v;                      // this element belongs to this wavefront alone
+                link.xg_out[at] = f32_to_bf16(v * gain_pre);
+                sq[m] = v * v;
+            } else {
+                from_f32(out + (size_t)m * N + n, v);
+            }
+        }
+    }
+    if (link.residual) {                                    // the workgroup's share of every row's sum of squares
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) sq_lds[wave][m] = sq[m];
+        }
+        __syncthreads();
+        if (threadIdx.x < MT && threadIdx.x < M) {
+            float total = 0.f;
+            for (int wv = 0; wv < GV_WAVES; ++wv) total += sq_lds[wv][threadIdx.x];
+            link.ssq_out[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = total;
+        }
     }
 }
 
@@ -95,38 +164,40 @@ static int gemv_k_split(int n, int k) {
     return 1;
 }
 
+static unsigned gemv_grid(int n, int k) {
+    const int rows_per_wg = GV_WAVES / gemv_k_split(n, k);
+    return (unsigned)((n + rows_per_wg - 1) / rows_per_wg);
+}
+
 template <int MT, bool SWIGLU, int KS>
-static void launch_gemv_ks(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, hipStream_t s) {
-    const int rows_per_wg = GV_WAVES / KS;
-    const unsigned grid = (n + rows_per_wg - 1) / rows_per_wg;
+static void launch_gemv_ks(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
+                           const NormLink& link, hipStream_t s) {
+    const unsigned grid = gemv_grid(n, k);
     if (out_dtype == RI_F32)
         gemv_bf16_kernel<MT, SWIGLU, float, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((float*)out, (const bf16_t*)x,
-                                                                                    (const bf16_t*)w, m, n, k);
+                                                                                    (const bf16_t*)w, m, n, k, link);
     else
-        gemv_bf16_kernel<MT, SWIGLU, bf16_t, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((bf16_t*)out, (const bf16_t*)x,
-                                                                                     (const bf16_t*)w, m, n, k);
+        gemv_bf16_kernel<MT, SWIGLU, bf16_t, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>(
+            (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, m, n, k, link);
 }
 
 template <int MT, bool SWIGLU>
-static void launch_gemv(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, hipStream_t s) {
+static void launch_gemv(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
+                        const NormLink& link, hipStream_t s) {
     switch (gemv_k_split(n, k)) {
-        case 4: launch_gemv_ks<MT, SWIGLU, 4>(out, out_dtype, x, w, m, n, k, s); break;
-        case 2: launch_gemv_ks<MT, SWIGLU, 2>(out, out_dtype, x, w, m, n, k, s); break;
-        default: launch_gemv_ks<MT, SWIGLU, 1>(out, out_dtype, x, w, m, n, k, s); break;
+        case 4: launch_gemv_ks<MT, SWIGLU, 4>(out, out_dtype, x, w, m, n, k, link, s); break;
+        case 2: launch_gemv_ks<MT, SWIGLU, 2>(out, out_dtype, x, w, m, n, k, link, s); break;
+        default: launch_gemv_ks<MT, SWIGLU, 1>(out, out_dtype, x, w, m, n, k, link, s); break;
     }
 }
 
-extern "C" int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
-                            void* stream) {
-    RI_REQUIRE(m > 0 && m <= 8, "gemv_bf16: %d rows of x, this kernel takes 1 to 8", m);
-    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemv_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
-    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemv_bf16: out dtype %d", out_dtype);
-    hipStream_t s = (hipStream_t)stream;
+static int gemv_run(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
+                    const NormLink& link, hipStream_t s) {
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
-#define RI_GEMV_CASE(MT)                                                       \
-    case MT:                                                                   \
-        if (swiglu) launch_gemv<MT, true>(out, out_dtype, x, w, m, n, k, s);   \
-        else        launch_gemv<MT, false>(out, out_dtype, x, w, m, n, k, s);  \
+#define RI_GEMV_CASE(MT)                                                             \
+    case MT:                                                                         \
+        if (swiglu) launch_gemv<MT, true>(out, out_dtype, x, w, m, n, k, link, s);   \
+        else        launch_gemv<MT, false>(out, out_dtype, x, w, m, n, k, link, s);  \
         break;
     switch (mt) {
         RI_GEMV_CASE(1)
@@ -137,4 +208,30 @@ extern "C" int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void*
 #undef RI_GEMV_CASE
     RI_LAUNCH_CHECK("gemv_bf16");
     return 0;
+}
+
+extern "C" int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
+                            void* stream) {
+    RI_REQUIRE(m > 0 && m <= 8, "gemv_bf16: %d rows of x, this kernel takes 1 to 8", m);
+    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemv_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemv_bf16: out dtype %d", out_dtype);
+    NormLink link = {};
+    return gemv_run(out, out_dtype, x, w, m, n, k, swiglu, link, (hipStream_t)stream);
+}
+
+// Number of workgroups (and so of partial sums of squares per row) of a linked product with n output columns.
+extern "C" int ri_gemv_bf16_partials(int n, int k) { return (int)gemv_grid(n, k); }
+
+extern "C" int ri_gemv_bf16_linked(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
+                                   int swiglu, const float* ssq_in, int n_in, float eps, int dim, float* residual,
+                                   const float* next_gain, void* xg_out, float* ssq_out, void* stream) {
+    RI_REQUIRE(m > 0 && m <= 8, "gemv_bf16_linked: %d rows of x, this kernel takes 1 to 8", m);
+    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemv_bf16_linked: n %d, k %d (k must be a multiple of 8)", n, k);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemv_bf16_linked: out dtype %d", out_dtype);
+    RI_REQUIRE(!ssq_in || (n_in > 0 && dim > 0), "gemv_bf16_linked: %d partial sums over %d elements", n_in, dim);
+    RI_REQUIRE(!residual || (next_gain && xg_out && ssq_out && !swiglu),
+               "gemv_bf16_linked: a product that feeds the residual stream needs the next gain and both outputs");
+    RI_REQUIRE(residual || out, "gemv_bf16_linked: no output");
+    NormLink link = {ssq_in, n_in, eps, dim, residual, next_gain, (bf16_t*)xg_out, ssq_out};
+    return gemv_run(out, out_dtype, x, w, m, n, k, swiglu, link, (hipStream_t)stream);
 }

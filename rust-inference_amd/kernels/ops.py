@@ -42,6 +42,12 @@ _SIGNATURES = {
                   c_void_p],
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemv_bf16_partials": [c_int, c_int],
+    "ri_gemm_skinny_packed_bf16_partials": [c_int],
+    "ri_gemv_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
+                            c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "ri_gemm_skinny_packed_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                          c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -347,3 +353,57 @@ def gemm_skinny_packed_bf16(x: torch.Tensor, wpacked: torch.Tensor, n: int, out_
     _call("ri_gemm_skinny_packed_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
           _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), int(parts), _stream())
     return out
+
+
+class NormedLater:
+    """Rows of a residual stream whose RMSNorm is left to the product that reads them:
+    ``xg = bfloat16(r * gain)`` and partial sums of ``r^2`` per row, ``[M, partials]``; the
+    normed rows are ``xg / sqrt(ssq.sum(1) / dim + eps)``."""
+
+    def __init__(self, xg: torch.Tensor, ssq: torch.Tensor, eps: float, dim: int):
+        self.xg, self.ssq, self.eps, self.dim = xg, ssq, float(eps), int(dim)
+        self.shape, self.dtype, self.device = xg.shape, xg.dtype, xg.device
+
+
+def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfloat16, swiglu: bool = False,
+                   residual: torch.Tensor | None = None, next_gain: torch.Tensor | None = None,
+                   next_eps: float = 0.0):
+    """A decode-size product that does the RMSNorm before it, the residual add and the RMSNorm's
+    preparation after it, or both, in the same kernel.
+
+    ``x`` is bfloat16 rows or a ``NormedLater``; ``w`` the row-major weight (``packed`` false: up to 8
+    rows, one wavefront per weight row) or its MFMA tiles (``packed`` true: up to 16 rows).  With
+    ``residual`` (float32 ``[M, n]``, updated in place to ``residual + x @ w.T``) the result is the
+    ``NormedLater`` of the new residual for a norm with ``next_gain`` and ``next_eps``; else the product."""
+    later = x if isinstance(x, NormedLater) else None
+    xr = later.xg if later else x
+    m, k = xr.shape
+    name = "ri_gemm_skinny_packed_bf16" if packed else "ri_gemv_bf16"
+    if packed:
+        want = (-(-n // 16) * (2 if swiglu else 1), -(-k // 32), 64, 8)
+        if tuple(w.shape) != want:
+            raise ShapeError(f"packed weight is {list(w.shape)}, a product with n {n}, k {k} wants {list(want)}")
+        wd = _dev(w, "wpacked", torch.bfloat16)
+    else:
+        wd = _dev(w, "w", torch.bfloat16, (n * (2 if swiglu else 1), k))
+    if later is not None:
+        ssq_in = _dev(later.ssq, "ssq", torch.float32, (m, later.ssq.shape[1]))
+        n_in, eps, dim = later.ssq.shape[1], later.eps, later.dim
+        if dim != k:
+            raise ShapeError(f"rows normed over {dim} elements into a product over {k}")
+    else:
+        ssq_in, n_in, eps, dim = None, 0, 0.0, 0
+    if residual is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=xr.device)
+        _call(name + "_linked", _dev(out, "out"), code(out_dtype), _dev(xr, "x", torch.bfloat16, (m, k)), wd, m, n, k,
+              int(swiglu), ssq_in, n_in, eps, dim, None, None, None, None, _stream())
+        return out
+    if swiglu:
+        raise ShapeError("a gate|up product does not feed the residual stream")
+    partials = _get("ri_gemm_skinny_packed_bf16_partials")(n) if packed else _get("ri_gemv_bf16_partials")(n, k)
+    xg = torch.empty((m, n), dtype=torch.bfloat16, device=xr.device)
+    ssq = torch.empty((m, partials), dtype=torch.float32, device=xr.device)
+    _call(name + "_linked", None, code(torch.bfloat16), _dev(xr, "x", torch.bfloat16, (m, k)), wd, m, n, k, 0,
+          ssq_in, n_in, eps, dim, _dev(residual, "residual", torch.float32, (m, n)),
+          _dev(next_gain, "next_gain", torch.float32, (n,)), _dev(xg, "xg"), _dev(ssq, "ssq"), _stream())
+    return NormedLater(xg, ssq, next_eps, n)

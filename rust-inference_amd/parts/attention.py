@@ -34,6 +34,8 @@ class GroupedQueryAttention(Mixer):
     ``[q; k; v]``: every output row's dot product is the same as with three products.
     """
 
+    links_norms = True
+
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, prefix: str, qk_norm: bool = True,
                  eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None):
         if heads < 1 or kv_heads < 1 or heads % kv_heads:
@@ -74,7 +76,7 @@ class GroupedQueryAttention(Mixer):
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window)
 
-    def forward(self, x, ctx, store, page_table):
+    def forward(self, x, ctx, store, page_table, link=None):
         rt = self.rt
         qkv = rt.linear(x, self.w_qkv)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
@@ -86,11 +88,11 @@ class GroupedQueryAttention(Mixer):
                                                 self.position.rotation_table(), store.k_pages, store.v_pages,
                                                 ctx.tok_pos, page_table, ctx.B, ctx.max_len, self.heads,
                                                 self.kv_heads, self.head_dim, self.window, self.scale)
-            return rt.linear_packed(o, self.w_o)
+            return rt.linear_packed(o, self.w_o, link=link)
         ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
                                   ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
                                   self.heads, self.kv_heads, self.head_dim, ctx.cu_seqlens, ctx.max_new)
-        return rt.linear_packed(self.attend(qkv, ctx, store, page_table), self.w_o)
+        return rt.linear_packed(self.attend(qkv, ctx, store, page_table), self.w_o, link=link)
 
     def attend(self, qkv, ctx, store, page_table):
         """The attention kernel that fits the step: matrix cores for bfloat16 (one new token per

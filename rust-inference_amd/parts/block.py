@@ -1,23 +1,61 @@
 """Arrangements: how a layer wires its norms, mixer and feed-forward around the residual stream."""
 from __future__ import annotations
 
+from ..kernels.ops import NormedLater
 from .registry import build_part, register_part
+
+# A decode step of at most this many tokens leaves its norms to the products around them (the
+# products that can do it take no more rows).
+LINK_MAX_TOKENS = 16
+
+
+class NormLink:
+    """An offer to a branch's last product: add your result into ``residual`` yourself and prepare
+    the rows for ``norm``, which then needs no kernel of its own."""
+
+    def __init__(self, residual, norm):
+        self.residual, self.norm = residual, norm
+        self.gain, self.eps = norm.gain, norm.eps
 
 
 class ResidualStream:
     """The float32 sum that runs through the layers, with at most one branch output
-    waiting to be added.  The add is done by the next norm, in the same kernel."""
+    waiting to be added.  The add is done by the next norm, in the same kernel, or, in
+    small decode steps, by the product that made the branch output: then what waits is
+    the prepared input of one norm (``later``) and the sum is already up to date."""
 
     def __init__(self, hidden):
         self.sum = hidden            # [T, hidden] float32
         self.pending = None
+        self.later = None            # (NormedLater, the norm it was prepared for)
+        self.next_entry_norm = None  # the norm that reads the stream after the current layer, if known
+
+    def link(self, norm, act_dtype):
+        """A ``NormLink`` for the branch that is about to run, if ``norm`` is the next reader of the
+        stream and can be left to a product."""
+        import torch
+        if (norm is None or not getattr(norm, "linkable", False) or self.pending is not None or self.later is not None
+                or act_dtype != torch.bfloat16 or self.sum.shape[0] > LINK_MAX_TOKENS
+                or norm.dim != self.sum.shape[1]):
+            return None
+        return NormLink(self.sum, norm)
 
     def push(self, branch) -> None:
-        if self.pending is not None:
+        if self.pending is not None or self.later is not None:
             self.flush()
-        self.pending = branch
+        if isinstance(branch, tuple):        # (NormedLater, norm): the product took a NormLink
+            self.later = branch
+        else:
+            self.pending = branch
 
-    def normed(self, norm, out_dtype, rows=None):
+    def normed(self, norm, out_dtype, rows=None, later_ok: bool = False):
+        """The stream through ``norm``.  With ``later_ok`` the caller takes a ``NormedLater`` too."""
+        if self.later is not None:
+            later, for_norm = self.later
+            self.later = None
+            if later_ok and for_norm is norm and rows is None:
+                return later
+            # prepared for another reader: the sum is complete, norm it the plain way
         if self.pending is not None and self.pending.dim() == 3 and not getattr(norm, "accepts_parts", False):
             self.pending = self.pending.sum(0)       # a norm that does not know about parts
         out = norm.apply(self.sum, self.pending, out_dtype, rows)
@@ -27,6 +65,7 @@ class ResidualStream:
 
     def flush(self) -> None:
         """Add the waiting branch without a norm (only arrangements that push twice need it)."""
+        self.later = None            # its sum is in the stream already
         if self.pending is not None:
             pending = self.pending.sum(0) if self.pending.dim() == 3 else self.pending
             self.sum.add_(pending.to(self.sum.dtype))
@@ -48,8 +87,23 @@ class PreNormBlock:
     def parts(self):
         return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
 
+    def entry_norm(self):
+        """The norm through which this layer first reads the stream."""
+        return self.mixer_norm
+
     def forward(self, stream: ResidualStream, ctx, store, page_table, act_dtype) -> None:
-        h = stream.normed(self.mixer_norm, act_dtype)
-        stream.push(self.mixer.forward(h, ctx, store, page_table))
-        h = stream.normed(self.feed_forward_norm, act_dtype)
-        stream.push(self.feed_forward.forward(h, ctx))
+        # a part with ``links_norms`` takes a NormedLater as input and a NormLink for its output
+        if getattr(self.mixer, "links_norms", False):
+            h = stream.normed(self.mixer_norm, act_dtype, later_ok=True)
+            link = stream.link(self.feed_forward_norm, act_dtype)
+            stream.push(self.mixer.forward(h, ctx, store, page_table, link=link))
+        else:
+            h = stream.normed(self.mixer_norm, act_dtype)
+            stream.push(self.mixer.forward(h, ctx, store, page_table))
+        if getattr(self.feed_forward, "links_norms", False):
+            h = stream.normed(self.feed_forward_norm, act_dtype, later_ok=True)
+            link = stream.link(stream.next_entry_norm, act_dtype)
+            stream.push(self.feed_forward.forward(h, ctx, link=link))
+        else:
+            h = stream.normed(self.feed_forward_norm, act_dtype)
+            stream.push(self.feed_forward.forward(h, ctx))

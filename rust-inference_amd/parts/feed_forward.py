@@ -16,6 +16,8 @@ class SwiGLU(FeedForward):
     (the reference: src/models/qwen3.rs:112-117; src/ops/elementwise.rs:9-12).  Gate and
     up are one product with the row-concatenated weight ``[gate; up]``."""
 
+    links_norms = True
+
     def __init__(self, hidden: int, inter: int, prefix: str):
         self.hidden, self.inter, self.prefix = hidden, inter, prefix
 
@@ -36,7 +38,8 @@ class SwiGLU(FeedForward):
         # (22 us against 27 us, also with K split into parts)
         self.w_down = PackedWeight(rt.place_matrix(weights[p + "down_proj.weight"]), None, False)
 
-    def forward(self, x, ctx):
+    def forward(self, x, ctx, link=None):
         rt = self.rt
         a = rt.linear_packed(x, self.w_gate_up)        # the activation is in the epilogue of the decode-size kernels
-        return rt.linear_packed(a, self.w_down, parts_ok=True)     # may come in parts: the stream's next norm adds them
+        # may come in parts: the stream's next norm adds them
+        return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)

@@ -130,8 +130,11 @@ class DecoderModel:
         """float32 logits ``[n_want, vocab]`` for the wanted rows of this step's tokens."""
         rt = self.rt
         stream = ResidualStream(self.embedding.forward(ctx.tokens))
-        for run in self.schedule:
+        for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]
+            follower = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
+            entry = getattr(follower, "entry_norm", None)
+            stream.next_entry_norm = entry() if entry else None
             store, table = None, None
             if run.cache is not None:
                 need = cache.needs[run.cache]

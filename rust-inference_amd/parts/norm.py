@@ -13,6 +13,7 @@ class RMSNorm(Norm):
     float32 (the reference: src/ops/norm.rs:7-32; fused with the add: :35-62)."""
 
     accepts_parts = True
+    linkable = True          # gain, eps and dim are all a product needs to do this norm itself
 
     def __init__(self, dim: int, eps: float, name: str):
         self.dim, self.eps, self.name = dim, eps, name

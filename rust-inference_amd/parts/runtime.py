@@ -74,8 +74,19 @@ class Runtime:
             return ops.gemm_f32(x, w)
         m, k = x.shape
         if m <= GEMV_MAX_ROWS and k % 8 == 0:
+            if isinstance(x, ops.NormedLater):
+                return ops.linked_product(x, w, w.shape[0], False, out_dtype)
             return ops.gemv_bf16(x, w, out_dtype)
-        return self._library_mm(x, w, out_dtype)
+        return self._library_mm(self.normed_now(x), w, out_dtype)
+
+    @staticmethod
+    def normed_now(x):
+        """The rows of a ``NormedLater`` for a product that cannot do the norm itself (``xg`` was
+        rounded once already, so this differs from the plain norm by one more rounding)."""
+        if not isinstance(x, ops.NormedLater):
+            return x
+        inv = torch.rsqrt(x.ssq.sum(1, keepdim=True) / x.dim + x.eps)
+        return (x.xg.float() * inv).to(x.xg.dtype)
 
     def pack(self, w: torch.Tensor, swiglu: bool = False) -> PackedWeight:
         """A placed weight with its packed copy for decode-size products (bfloat16 compute only)."""
@@ -83,17 +94,33 @@ class Runtime:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
 
-    def linear_packed(self, x: torch.Tensor, pw: PackedWeight, out_dtype=None, parts_ok: bool = False) -> torch.Tensor:
+    def linear_packed(self, x, pw: PackedWeight, out_dtype=None, parts_ok: bool = False, link=None):
         """``x @ w.T`` (or ``silu(x @ gate.T) * (x @ up.T)`` for a fused gate|up weight) with the kernel
         that fits the number of rows.  With ``parts_ok`` the result may be ``[parts, M, N]`` float32, the
-        sums over pieces of K, for a consumer that adds them (the residual stream's next norm)."""
+        sums over pieces of K, for a consumer that adds them (the residual stream's next norm).
+
+        ``x`` may be a ``NormedLater``.  With ``link`` (the residual stream's offer to the last product of
+        a branch) a kernel that can adds the result into the stream and prepares the next norm; the
+        return value is then ``(NormedLater, norm)`` for the stream instead of a tensor."""
         out_dtype = out_dtype or self.dtype
         m = x.shape[0]
         if self.dtype == torch.bfloat16 and pw.k % 8 == 0:
+            later = isinstance(x, ops.NormedLater)
+            mine = None
             # two rows of the gate|up matrix: the matrix-core kernel is already ahead (40 us against 47 us)
             if m == 1 or (m <= GEMV_MAX_ROWS and not (pw.swiglu and pw.packed is not None)):
-                return ops.gemv_bf16(x, pw.w, out_dtype, swiglu=pw.swiglu)
-            if m <= SKINNY_MAX_ROWS and pw.packed is not None:
+                mine = (pw.w, False)
+            elif m <= SKINNY_MAX_ROWS and pw.packed is not None:
+                mine = (pw.packed, True)
+            if mine is not None:
+                if link is not None and not pw.swiglu and link.residual.shape == (m, pw.n):
+                    made = ops.linked_product(x, mine[0], pw.n, mine[1], residual=link.residual,
+                                              next_gain=link.gain, next_eps=link.eps)
+                    return (made, link.norm)
+                if later:
+                    return ops.linked_product(x, mine[0], pw.n, mine[1], out_dtype, swiglu=pw.swiglu)
+                if not mine[1]:
+                    return ops.gemv_bf16(x, pw.w, out_dtype, swiglu=pw.swiglu)
                 if parts_ok and pw.parts > 1:
                     return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=pw.parts)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)

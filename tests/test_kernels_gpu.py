@@ -397,6 +397,46 @@ def test_gemm_skinny_packed_bf16(ops, m, n, k):
         close(got.sum(0), want, 3e-6, f"{parts} parts of K")
 
 
+@pytest.mark.parametrize("packed, m", [(False, 1), (False, 2), (False, 5), (True, 1), (True, 3), (True, 16)])
+@pytest.mark.parametrize("hidden, k, inter", [(104, 72, 56), (4096, 4096, 1000), (584, 12288, 37)])
+def test_products_linked_to_norms(ops, packed, m, hidden, k, inter):
+    """A branch's last product adds into the residual stream and prepares the next RMSNorm; the
+    product after it finishes that norm.  Checked against add, norm and products done one by one."""
+    rng = np.random.default_rng(m + hidden)
+    eps = 1e-5
+    x = t(rng.normal(size=(m, k)), torch.bfloat16)
+    w_out = t(rng.normal(size=(hidden, k)) / np.sqrt(k), torch.bfloat16)
+    r0 = t(rng.normal(size=(m, hidden)) * 3)
+    gain = t(1 + 0.3 * rng.normal(size=hidden))
+    w_next = t(rng.normal(size=(inter, hidden)), torch.bfloat16)
+    w_gu = t(rng.normal(size=(2 * inter, hidden)) * (4.0 / np.sqrt(hidden)), torch.bfloat16)
+    prep = (lambda w, **kw: ops.pack_for_mfma(w, **kw)) if packed else (lambda w, **kw: w)
+
+    r1 = f64(r0) + f64(x) @ f64(w_out).T
+    residual = r0.clone()
+    later = ops.linked_product(x, prep(w_out), hidden, packed, residual=residual, next_gain=gain, next_eps=eps)
+    close(residual, r1, 3e-6, "residual after the linked product")
+    close(later.xg, f64(residual) * f64(gain), 4e-3, "rows times gain")       # one rounding to bfloat16
+    close(later.ssq.sum(1), (f64(residual) ** 2).sum(1), 1e-5, "sums of squares")
+    assert later.dim == hidden and later.eps == eps
+    # a second call leaves the same partial sums: they do not depend on scheduling
+    again = ops.linked_product(x, prep(w_out), hidden, packed, residual=r0.clone(), next_gain=gain, next_eps=eps)
+    assert torch.equal(again.ssq, later.ssq) and torch.equal(again.xg, later.xg)
+
+    normed = P.rms_norm(f64(residual), f64(gain), eps)
+    close(ops.linked_product(later, prep(w_next), inter, packed, torch.float32), normed @ f64(w_next).T, 6e-3,
+          "product that finishes the norm")
+    y = normed @ f64(w_gu).T
+    close(ops.linked_product(later, prep(w_gu, swiglu=True) if packed else w_gu, inter, packed, torch.bfloat16,
+                             swiglu=True), P.silu(y[:, :inter]) * y[:, inter:], 1e-2, "the same with swiglu")
+    # both sides at once: the next branch's product reads prepared rows and prepares the following norm
+    w_back = t(rng.normal(size=(hidden, hidden)) / np.sqrt(hidden), torch.bfloat16)
+    r2 = f64(residual) + normed @ f64(w_back).T
+    chained = ops.linked_product(later, prep(w_back), hidden, packed, residual=residual, next_gain=gain, next_eps=eps)
+    close(residual, r2, 6e-3, "residual after two linked products")
+    close(chained.ssq.sum(1), (f64(residual) ** 2).sum(1), 1e-5, "sums of squares, second link")
+
+
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 1e-6), (torch.bfloat16, 5e-3)])
 def test_swiglu(ops, dtype, rel):
     assert f64(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])))[0, 0] == 0.0                 # src/ops/elementwise.rs:59-70
