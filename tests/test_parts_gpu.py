@@ -115,6 +115,62 @@ def test_swiglu_part(dtype, bound, rows):
     assert rel_to_max(f64(ff.forward(x, None)), want) < bound
 
 
+@pytest.mark.parametrize("rows", [1, 2, 5, 16, 17])
+def test_prenorm_block_leaves_norms_to_the_products(rows):
+    """Small bfloat16 steps: the branch's last product adds into the stream and prepares the next norm.
+    The block must give the plain block's stream whether the link is taken (up to 16 rows), not offered
+    (17 rows), or its preparation is for a norm that turns out not to read the stream next."""
+    from rust_inference_amd.kernels.ops import NormedLater
+    from rust_inference_amd.parts import PartSpec, Runtime, build_part
+    from rust_inference_amd.parts.block import ResidualStream
+    rng = np.random.default_rng(rows)
+    rt, hidden, inter, eps = Runtime(DEV, torch.bfloat16), 104, 232, 1e-5
+    ff = build_part("feed_forward", PartSpec("swiglu", {"hidden": hidden, "inter": inter, "prefix": "m."}))
+    w = {n: torch.tensor(0.1 * rng.normal(size=s.shape)).to(torch.bfloat16) for n, s in ff.tensors().items()}
+    norms = []
+    for name in ("a", "b", "c"):
+        norm = build_part("norm", PartSpec("rmsnorm", {"dim": hidden, "eps": eps, "name": name}))
+        w[name] = torch.tensor(1 + 0.2 * rng.normal(size=hidden)).to(torch.bfloat16)
+        norm.bind(w, rt)
+        norms.append(norm)
+    ff.bind(w, rt)
+    w64 = {k: v.to(torch.float64).numpy() for k, v in w.items()}
+    h0 = rng.normal(size=(rows, hidden))
+
+    def plain_branch(h, gain):
+        return h + P.swiglu_mlp(P.rms_norm(h, w64[gain], eps), w64["m.gate_proj.weight"], w64["m.up_proj.weight"],
+                                w64["m.down_proj.weight"])
+
+    # two feed-forward branches in a row, the first told that norm b reads the stream next
+    stream = ResidualStream(t(h0))
+    link = stream.link(norms[1], torch.bfloat16)
+    assert (link is not None) == (rows <= 16)
+    stream.push(ff.forward(stream.normed(norms[0], torch.bfloat16), None, link=link))
+    h1 = plain_branch(h0, "a")
+    if rows <= 2:                                 # these sizes' down product can take the link
+        assert stream.later is not None and stream.pending is None
+        assert rel_to_max(f64(stream.sum), h1) < 5e-3
+    assert stream.link(norms[2], torch.bfloat16) is None          # something waits: no second offer
+    x = stream.normed(norms[1], torch.bfloat16, later_ok=True)
+    assert isinstance(x, NormedLater) == (rows <= 2)
+    stream.push(ff.forward(x, None))
+    stream.flush()
+    assert rel_to_max(f64(stream.sum), plain_branch(h1, "b")) < 2e-2
+
+    # prepared for b, read by c: the preparation is dropped and c norms the complete sum itself
+    stream = ResidualStream(t(h0))
+    stream.push(ff.forward(stream.normed(norms[0], torch.bfloat16), None, link=stream.link(norms[1], torch.bfloat16)))
+    x = stream.normed(norms[2], torch.bfloat16, later_ok=True)
+    assert not isinstance(x, NormedLater)
+    assert rel_to_max(f64(x), P.rms_norm(h1, w64["c"], eps)) < 1e-2
+    # and a reader of single rows (the output head's norm) gets plain rows too
+    stream = ResidualStream(t(h0))
+    stream.push(ff.forward(stream.normed(norms[0], torch.bfloat16), None, link=stream.link(norms[1], torch.bfloat16)))
+    rows_wanted = torch.tensor([rows - 1], dtype=torch.int32, device=DEV)
+    x = stream.normed(norms[1], torch.bfloat16, rows=rows_wanted, later_ok=True)
+    assert rel_to_max(f64(x), P.rms_norm(h1[-1:], w64["b"], eps)) < 1e-2
+
+
 # ------------------------------------------------------------------------------------------------ the toy architecture
 TOY = {"architectures": ["ToyMixForCausalLM"], "vocab_size": 130, "hidden_size": 48, "inter": 80, "heads": 4,
        "kv_heads": 2, "head_dim": 16, "window": 24, "eps": 1e-5, "theta": 10000.0}
