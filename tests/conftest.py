@@ -35,18 +35,26 @@ TINY_C = {
     "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 48,
     "rope_theta": 50000.0, "rms_norm_eps": 3e-6, "tie_word_embeddings": False, "max_position_embeddings": 1024,
 }
+# The head size and grouping of the large models (128, four query heads per kv head), where the
+# bfloat16 path takes its matrix-core attention kernels and packed weights.
+TINY_D = {
+    "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+    "vocab_size": 500, "hidden_size": 128, "intermediate_size": 384, "num_hidden_layers": 2,
+    "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 128,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 512,
+}
 
 
 @pytest.fixture(scope="session")
 def model_dirs(tmp_path_factory):
     """Model folders with random weights for the tiny configurations, made once per session.
-    A is stored in float32, B and C in bfloat16.  Weights are larger than the benchmark's
+    A is stored in float32, the others in bfloat16.  Weights are larger than the benchmark's
     N(0, 0.02) so that logits are of order one and differences show."""
     import torch
     from rust_inference_amd.weights import write_random_model
     base = tmp_path_factory.mktemp("models")
     out = {}
     for name, cfg, seed, dtype in (("A", TINY_A, 0, torch.float32), ("B", TINY_B, 1, torch.bfloat16),
-                                   ("C", TINY_C, 2, torch.bfloat16)):
+                                   ("C", TINY_C, 2, torch.bfloat16), ("D", TINY_D, 3, torch.bfloat16)):
         out[name] = write_random_model(str(base / name), cfg, seed, dtype, matrix_std=0.12, gain_std=0.1)
     return out

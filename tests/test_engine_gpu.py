@@ -66,7 +66,7 @@ def check_against_plain(model_dir, got, requests, dtype_name, what):
         assert_logits_close(got[rid], plain_logits(model_dir, toks), dtype_name, f"{what}, request {rid}")
 
 
-CASES = [("A", [5, 11, 1, 17], 0), ("B", [33, 2, 40], 1), ("C", [70, 45, 3], 2)]
+CASES = [("A", [5, 11, 1, 17], 0), ("B", [33, 2, 40], 1), ("C", [70, 45, 3], 2), ("D", [300, 37, 130], 3)]
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])

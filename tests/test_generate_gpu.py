@@ -46,6 +46,7 @@ def prompts_for(cfg, lengths, seed):
 @pytest.mark.parametrize("name, lengths, steps, dtype_name", [
     ("A", [5, 11, 1, 17], 8, "float32"), ("A", [5, 11, 1, 17], 8, "bfloat16"),
     ("B", [33, 2, 40], 16, "float32"), ("B", [33, 2, 40], 16, "bfloat16"),
+    ("D", [70, 2, 40], 16, "bfloat16"),
 ])
 def test_greedy_generation_through_the_entry_point(model_dirs, name, lengths, steps, dtype_name, use_graphs):
     from rust_inference_amd import Model
@@ -75,16 +76,17 @@ def test_stop_tokens_and_batches_one_after_another(model_dirs):
     assert all(s not in toks for toks in res.tokens for s in stop)
 
 
-def test_graph_and_eager_decoding_give_the_same_logits(model_dirs):
+@pytest.mark.parametrize("name, lengths, room", [("B", [33, 2, 40], 96), ("D", [270, 2, 40], 320)])
+def test_graph_and_eager_decoding_give_the_same_logits(model_dirs, name, lengths, room):
     import torch
     from rust_inference_amd.engine import Engine, StepEntry
     from rust_inference_amd.parts import load_model
-    model = load_model(model_dirs["B"], torch.bfloat16)
-    cfg, _ = read_model_f64(model_dirs["B"])
-    prompts = prompts_for(cfg, [33, 2, 40], 5)
+    model = load_model(model_dirs[name], torch.bfloat16)
+    cfg, _ = read_model_f64(model_dirs[name])
+    prompts = prompts_for(cfg, lengths, 5)
     outs = []
     for graphs in (False, True):
-        eng = Engine(model, model.new_cache(max_tokens=3 * 96, num_slots=3, max_seq_len=96), use_graphs=graphs)
+        eng = Engine(model, model.new_cache(max_tokens=3 * room, num_slots=3, max_seq_len=room), use_graphs=graphs)
         slots = [eng.cache.acquire() for _ in prompts]
         eng.step([StepEntry(s, p, "last") for s, p in zip(slots, prompts)])
         rows = []
