@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
-The default run has the layer sizes of the Qwen3-8B row of BASELINE.json with random weights
+The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
 context of 4,096.  A step is one decode step: every live sequence gets one more token, chosen
 greedily on the device.  Prints one JSON line: decoded tokens a second at batch 8 (`value`), the

@@ -17,6 +17,10 @@ from ..kernels import ops
 #              plus an activation kernel; 3.0 against 2.2 TB/s on the 4096 x 4096 matrix).  Elsewhere
 #              the vendor library's product is as fast or faster (4.5 to 4.9 TB/s) and is used.
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
+#              A form of the packed kernel for up to 64 rows (every weight tile used for four tiles of x
+#              taken from the L2 cache) was tried and lost to the library from 24 rows on at every one of
+#              these matrices (q|k|v at 32 rows: 23 us against 16 us): it would need x staged through LDS
+#              and larger workgroup tiles, which is the library's own design.
 GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
 SPLIT_K = 4096
