@@ -1,7 +1,9 @@
 """Each part alone against its plain counterpart, and the parts' generality: a toy architecture,
 registered here and nowhere in the package, with a windowed attention layer that runs twice (its
 weights shared, a cache entry per run), a toy mixer that keeps a state of its own per sequence, and
-no position encoding in one layer; built and stepped through the unchanged engine."""
+no position encoding in one layer, a position encoding of another kind (a learned table added to q and
+k) and a feed-forward that routes every token to two of four experts in another; built and stepped
+through the unchanged engine."""
 import json
 import os
 from dataclasses import dataclass
@@ -173,14 +175,62 @@ def test_prenorm_block_leaves_norms_to_the_products(rows):
 
 # ------------------------------------------------------------------------------------------------ the toy architecture
 TOY = {"architectures": ["ToyMixForCausalLM"], "vocab_size": 130, "hidden_size": 48, "inter": 80, "heads": 4,
-       "kv_heads": 2, "head_dim": 16, "window": 24, "eps": 1e-5, "theta": 10000.0}
+       "kv_heads": 2, "head_dim": 16, "window": 24, "eps": 1e-5, "theta": 10000.0, "experts": 4, "period": 37}
 
 
 def register_toy():
     from rust_inference_amd.cache import StateNeed
     from rust_inference_amd.config import ModelConfig, register_architecture
-    from rust_inference_amd.parts import LayerSpec, Mixer, ModelSpec, PartSpec, Run, register_part
+    from rust_inference_amd.parts import (FeedForward, LayerSpec, Mixer, ModelSpec, PartSpec, PositionEncoding, Run,
+                                          register_part)
     from rust_inference_amd.weights import MATRIX, TensorSpec
+
+    @register_part("position", "toy_additive")
+    class AdditivePosition(PositionEncoding):
+        """q and k of the token at position p get row ``p % period`` of a learned table added, in
+        every head: an encoding that does not rotate and has a tensor of its own."""
+        def __init__(self, head_dim, period, name):
+            self.head_dim, self.period, self.name = head_dim, period, name
+
+        def tensors(self):
+            return {self.name: TensorSpec((self.period, self.head_dim), MATRIX)}
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.table = weights[self.name].to(rt.device, torch.float32)
+
+        def apply(self, qkv, ctx, heads, kv_heads, head_dim):
+            add = self.table[ctx.tok_pos.long() % self.period]                     # [T, head_dim]
+            qk = qkv[:, :(heads + kv_heads) * head_dim].unflatten(1, (heads + kv_heads, head_dim))
+            qk.copy_((qk.float() + add[:, None, :]).to(qkv.dtype))                 # a view: in place, one rounding
+
+    @register_part("feed_forward", "toy_top2")
+    class Top2Experts(FeedForward):
+        """Four square experts; a token goes to the two with the largest router probability and
+        weights them by their lead over the third, ``p_e - p_(3)``: zero for every other expert, and
+        continuous in x, so that rounding cannot flip a result.  Router logits and softmax in
+        float32.  (Every expert sees every token here, masked: the toy keeps to shapes that do not
+        depend on the data.)"""
+        def __init__(self, hidden, experts, prefix):
+            self.hidden, self.experts, self.prefix = hidden, experts, prefix
+
+        def tensors(self):
+            t = {self.prefix + "router.weight": TensorSpec((self.experts, self.hidden), MATRIX)}
+            for e in range(self.experts):
+                t[f"{self.prefix}experts.{e}.weight"] = TensorSpec((self.hidden, self.hidden), MATRIX)
+            return t
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.router = weights[self.prefix + "router.weight"].to(rt.device, torch.float32)
+            self.w = torch.stack([weights[f"{self.prefix}experts.{e}.weight"] for e in range(self.experts)]).to(
+                rt.device, torch.float32)
+
+        def forward(self, x, ctx):
+            p = torch.softmax(x.float() @ self.router.T, dim=-1)                   # [T, E]
+            third = torch.topk(p, 3, dim=-1).values[:, 2:3]
+            weight = torch.clamp(p - third, min=0.0)                               # two experts at most are non-zero
+            return torch.einsum("te,ehd,td->th", weight, self.w, x.float())       # float32: the stream takes it as it is
 
     @register_part("mixer", "toy_running_mean")
     class RunningMean(Mixer):
@@ -221,6 +271,8 @@ def register_toy():
         window: int = 0
         eps: float = 1e-5
         theta: float = 1e4
+        experts: int = 0
+        period: int = 0
         ARCHITECTURE: ClassVar[str] = "ToyMixForCausalLM"
         MODEL_TYPE: ClassVar[str] = "toy_mix"
 
@@ -248,12 +300,19 @@ def register_toy():
             mixer_norm=norm("l2.n1"), feed_forward_norm=norm("l2.n2"), feed_forward=ff("l2.ff."),
             mixer=PartSpec("attention", {"hidden": d, "heads": 2, "kv_heads": 1, "head_dim": 32, "prefix": "l2.attn.",
                                          "qk_norm": True, "eps": c.eps, "window": None, "position": PartSpec("none")}))
+        routed = LayerSpec(
+            mixer_norm=norm("l3.n1"), feed_forward_norm=norm("l3.n2"),
+            feed_forward=PartSpec("toy_top2", {"hidden": d, "experts": c.experts, "prefix": "l3.moe."}),
+            mixer=PartSpec("attention", {"hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                         "prefix": "l3.attn.", "qk_norm": False, "eps": c.eps, "window": None,
+                                         "position": PartSpec("toy_additive", {"head_dim": c.head_dim, "period": c.period,
+                                                                               "name": "l3.attn.position.weight"})}))
         return ModelSpec(
             architecture="ToyMixForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
             embedding=PartSpec("table", {"vocab": c.vocab_size, "dim": d, "name": "embed.weight"}),
-            layers=(windowed, stateful, unrotated),
+            layers=(windowed, stateful, unrotated, routed),
             # layer 0 runs twice with the same weights; each run has a cache entry of its own
-            schedule=(Run(0, 0), Run(1, 1), Run(0, 2), Run(2, 3)),
+            schedule=(Run(0, 0), Run(1, 1), Run(0, 2), Run(2, 3), Run(3, 4)),
             final_norm=norm("final.weight"),
             head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": False}),
             max_positions=512)
@@ -292,10 +351,31 @@ def toy_plain(w, ids):
         v = (x @ w["l2.attn.v_proj.weight"].T).reshape(s, 1, 32)
         return P.attention(q, k, v).reshape(s, -1) @ w["l2.attn.o_proj.weight"].T
 
+    def additive(x):
+        s = x.shape[0]
+        add = w["l3.attn.position.weight"][pos % c["period"]][:, None, :]
+        q = (x @ w["l3.attn.q_proj.weight"].T).reshape(s, c["heads"], c["head_dim"]) + add
+        k = (x @ w["l3.attn.k_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"]) + add
+        v = (x @ w["l3.attn.v_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        return P.attention(q, k, v).reshape(s, -1) @ w["l3.attn.o_proj.weight"].T
+
+    def top2(x):
+        logits = x @ w["l3.moe.router.weight"].T
+        p = np.exp(logits - logits.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        out = np.zeros_like(x)
+        for t in range(x.shape[0]):                          # token by token: the two chosen experts only
+            order = np.argsort(-p[t])
+            for e in order[:2]:
+                out[t] += (p[t, e] - p[t, order[2]]) * (w[f"l3.moe.experts.{e}.weight"] @ x[t])
+        return out
+
     h = block(h, "l0", windowed)
     h = block(h, "l1", running_mean)
     h = block(h, "l0", windowed)
     h = block(h, "l2", unrotated)
+    r = h + additive(P.rms_norm(h, w["l3.n1"], c["eps"]))
+    h = r + top2(P.rms_norm(r, w["l3.n2"], c["eps"]))
     return P.rms_norm(h, w["final.weight"], c["eps"]) @ w["head.weight"].T
 
 
@@ -304,7 +384,7 @@ def toy_dir(tmp_path_factory):
     register_toy()
     from rust_inference_amd.weights import write_random_model
     return write_random_model(str(tmp_path_factory.mktemp("toy") / "m"), TOY, seed=7, dtype=torch.float32,
-                              matrix_std=0.15)
+                              matrix_std=0.12)     # the scale of the other test models
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
@@ -316,6 +396,7 @@ def test_toy_architecture_builds_and_steps_through_the_unchanged_engine(toy_dir,
     model = load_model(toy_dir, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
     needs = model.cache_needs()
     assert needs[0] == needs[2] == KVNeed(2, 16, 24) and isinstance(needs[1], StateNeed) and needs[3] == KVNeed(1, 32, None)
+    assert needs[4] == KVNeed(2, 16, None)
     with safe_open(os.path.join(toy_dir, "model.safetensors"), framework="pt") as f:
         w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
     rng = np.random.default_rng(8)
@@ -326,7 +407,7 @@ def test_toy_architecture_builds_and_steps_through_the_unchanged_engine(toy_dir,
                                  {k: (v, max(1, len(v) - 20)) for k, v in list(reqs.items())[:2]},
                                  {k: (v, max(1, len(v) - 33)) for k, v in list(reqs.items())[2:]}]))):
         engine = engine_for_trace(model, plans.max_live_tokens(steps))
-        assert len(engine.cache.groups) == 2                     # the windowed entries and the full one: own storage
+        assert len(engine.cache.groups) == 3                     # the windowed entries and the two full kinds: own storage
         player, outs = Replayer(engine), {}
         for s in steps:
             logits = player.feed(s)
