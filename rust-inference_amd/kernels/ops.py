@@ -42,6 +42,7 @@ _SIGNATURES = {
                   c_void_p],
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_attention_decode_chunks": [c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
     "ri_gemm_skinny_packed_bf16_partials": [c_int],
     "ri_gemv_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
@@ -223,7 +224,6 @@ def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, k
 
 
 MFMA_HEAD_DIMS = (32, 64, 128)
-DECODE_CHUNK = 256
 
 
 def mfma_attention_fits(dtype, head_dim: int, group: int, page_size: int, decode: bool) -> bool:
@@ -252,7 +252,7 @@ def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table
     tokens, stride = qkv.shape
     if tokens != seqs:
         raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
-    chunks = -(-max_len // DECODE_CHUNK)
+    chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
     out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
     ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
     _call("ri_attention_decode_bf16", _dev(out, "out"), _dev(ws, "workspace"), _dev(qkv, "qkv", torch.bfloat16), stride,
@@ -275,7 +275,7 @@ def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_p
     if (hkv, dh) != (kv_heads, head_dim) or tuple(v_pages.shape) != (num_pages, hkv, dh, page_size):
         raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv heads "
                          f"of {head_dim}")
-    chunks = -(-max_len // DECODE_CHUNK)
+    chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
     out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
     ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
     half = head_dim // 2
