@@ -13,7 +13,8 @@
 // Nothing is sorted.  The order is a 56-bit key per candidate (the float's bits made monotone, then
 // 2^24 - 1 - id), and "the first candidate whose running count or mass passes a target" is found by
 // descending that key eight bits at a time: a histogram of the candidates that share the prefix found
-// so far, then a scan of its 256 bins from the top.  Masses are 40-bit fixed-point integers, so every
+// so far, then a scan of its 256 bins from the top (the id bits are settled in one step as a rule: see
+// descend).  Masses are 40-bit fixed-point integers, so every
 // sum is exact and independent of the order of addition: the same logits and the same r give the
 // same token on every run.  Lanes add into 16 copies of the histogram, so that
 // the many candidates that share a bin do not queue up on one LDS address.
@@ -24,6 +25,7 @@
 #define SMP_COPIES 16
 #define SMP_ID_BITS 24
 #define SMP_FIXED 1099511627776.0f      // 2^40
+#define SMP_TIES 2048                   // candidates of one value whose ids are listed rather than descended
 
 typedef unsigned long long u64;
 
@@ -37,37 +39,161 @@ struct RowView {
     const float* logits;
     const uint8_t* seen;     // may be NULL
     float penalty, inv_temperature;
-    __device__ __forceinline__ float penalised(int i) const {
-        float l = logits[i];
-        if (seen && seen[i]) l = l > 0.f ? l / penalty : l * penalty;
-        return l;
+    bool wide;               // the row starts on a 16-byte boundary and the vocabulary is a multiple of 4
+    __device__ __forceinline__ float penalise(float l, bool was_seen) const {
+        return was_seen ? (l > 0.f ? l / penalty : l * penalty) : l;
     }
-    __device__ __forceinline__ float scaled(int i) const { return penalised(i) * inv_temperature; }
 };
+
+// f(i, penalised logit of token i) for every token of the row, each token once, the workgroup's threads
+// sharing the work.  One pass over a row is bound by the latency of its loads, not by their volume (a
+// row is a few hundred KB in the L2 cache), so the loads are 16 bytes wide where the row allows it and
+// SMP_UNROLL of them are in flight per thread before the first value is used.
+#define SMP_UNROLL 4
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const RowView& row, int vocab, F&& f) {
+    if (row.wide) {
+        const float4* lp = reinterpret_cast<const float4*>(row.logits);
+        const uint32_t* sp = reinterpret_cast<const uint32_t*>(row.seen);
+        const int n4 = vocab / 4;
+        for (int i0 = threadIdx.x; i0 < n4; i0 += SMP_THREADS * SMP_UNROLL) {
+            float4 v[SMP_UNROLL];
+            uint32_t sn[SMP_UNROLL];
+#pragma unroll
+            for (int u = 0; u < SMP_UNROLL; ++u) {
+                const int i = i0 + u * SMP_THREADS;
+                v[u] = i < n4 ? lp[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                sn[u] = (sp && i < n4) ? sp[i] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < SMP_UNROLL; ++u) {
+                const int i = i0 + u * SMP_THREADS;
+                if (i < n4) {
+                    f(4 * i, row.penalise(v[u].x, sn[u] & 0x000000FFu));
+                    f(4 * i + 1, row.penalise(v[u].y, sn[u] & 0x0000FF00u));
+                    f(4 * i + 2, row.penalise(v[u].z, sn[u] & 0x00FF0000u));
+                    f(4 * i + 3, row.penalise(v[u].w, sn[u] & 0xFF000000u));
+                }
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < vocab; i += SMP_THREADS) f(i, row.penalise(row.logits[i], row.seen && row.seen[i]));
+    }
+}
+
+// The fixed-point mass of a candidate, exp(s - smax) * 2^40 cut to an integer: one function, used wherever
+// a mass is wanted, so that every pass sees the same number.  The exponential is the hardware's base-2
+// one (its argument is at most 0, its last bit or two are its own: the masses define the distribution that
+// is drawn from, and they differ from the exact ones by parts in ten million).  The float, at least 1
+// and below 2^41, is widened by hand: 24 bits of mantissa shifted into place.
+__device__ __forceinline__ u64 fixed_mass(float s, float smax) {
+    const float x = __builtin_amdgcn_exp2f((s - smax) * 1.44269504088896341f) * SMP_FIXED;
+    const uint32_t bits = __float_as_uint(x);
+    const int e = (int)(bits >> 23) - 127;                   // x is not negative and not above 2^40 (1 + 2^-22)
+    if (e < 0) return 0;
+    const u64 mant = (u64)((bits & 0x007FFFFFu) | 0x00800000u);
+    return e >= 23 ? mant << (e - 23) : mant >> (23 - e);
+}
 
 __device__ __forceinline__ u64 composite(float s, int id) {
     return ((u64)ordered_bits(s) << SMP_ID_BITS) | (u64)((1 << SMP_ID_BITS) - 1 - id);
 }
 
+__device__ __forceinline__ float value_of_ordered(uint32_t ob) {      // the inverse of ordered_bits
+    return __uint_as_float((ob & 0x80000000u) ? (ob & 0x7FFFFFFFu) : ~ob);
+}
+
+// One digit of a descent: from the 256 bins of the candidates that share the prefix found so far, the
+// highest bin b whose candidates bring the running weight past the target:
+//   shared[0] = weight above bin b, shared[1] = b, shared[2] = weight down to and including bin b.
+// The first wavefront does it, four bins a lane, with a suffix sum over the lanes.
+__device__ __forceinline__ void pick_bin(const u64* bins, u64 above, u64 target, u64* shared) {
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const u64 b0 = bins[4 * lane], b1 = bins[4 * lane + 1], b2 = bins[4 * lane + 2], b3 = bins[4 * lane + 3];
+        const u64 mine = b0 + b1 + b2 + b3;
+        u64 sfx = mine;                                         // this lane's bins and all higher lanes'
+        for (int d = 1; d < 64; d <<= 1) {
+            const u64 o = __shfl_down(sfx, d, 64);
+            if (lane + d < 64) sfx += o;
+        }
+        const u64 a3 = above + (sfx - mine);                    // weight above bin 4 lane + 3
+        const u64 a2 = a3 + b3, a1 = a2 + b2, a0 = a1 + b1;
+        int hit = -1;
+        u64 hit_above = 0, hit_bin = 0;
+        if (a3 + b3 > target)      { hit = 4 * lane + 3; hit_above = a3; hit_bin = b3; }
+        else if (a2 + b2 > target) { hit = 4 * lane + 2; hit_above = a2; hit_bin = b2; }
+        else if (a1 + b1 > target) { hit = 4 * lane + 1; hit_above = a1; hit_bin = b1; }
+        else if (a0 + b0 > target) { hit = 4 * lane;     hit_above = a0; hit_bin = b0; }
+        const u64 any = __ballot(hit >= 0);
+        const int top = any ? 63 - __clzll((long long)any) : 0;       // nothing passes the target: bin 0
+        if (lane == top) {
+            if (!any) { hit = 0; hit_above = a0; hit_bin = b0; }
+            shared[0] = hit_above;
+            shared[1] = (u64)hit;
+            shared[2] = hit_above + hit_bin;
+        }
+    }
+}
+
 // Finds the key c* with  sum_{c > c*} w  <=  target  <  sum_{c >= c*} w  over the candidates with
 // key >= floor_key, w = 1 (count) or the fixed-point mass.  Returns c*; *incl = sum_{c >= c*} w.
+//
+// Four passes settle the 32 value bits.  What is left are the candidates whose value is exactly that
+// (nearly always one): a fifth pass lists their ids, they all weigh the same, and the one wanted is found
+// by its rank.  Only if the list overflows (a row of equal logits) the id bits are descended like the
+// value bits.
 template <bool MASS>
 __device__ u64 descend(const RowView& row, int vocab, float smax, u64 floor_key, u64 target, u64* hist, u64* bins,
-                       u64* shared, u64* incl) {
+                       u64* shared, int* ties, int* tie_count, u64* incl) {
     u64 prefix = 0;            // the bits of c* found so far, in place
     u64 above = 0;             // weight of the candidates above the prefix's bucket
     for (int shift = 48; shift >= 0; shift -= 8) {
+        if (shift == SMP_ID_BITS - 8) {                       // the value is known: list the ids that have it
+            if (threadIdx.x == 0) *tie_count = 0;
+            __syncthreads();
+            const uint32_t value_bits = (uint32_t)(prefix >> SMP_ID_BITS);
+            for_each_logit(row, vocab, [&](int i, float l) {
+                const float s = l * row.inv_temperature;
+                if (ordered_bits(s) == value_bits && composite(s, i) >= floor_key) {
+                    const int k = atomicAdd(tie_count, 1);
+                    if (k < SMP_TIES) ties[k] = i;
+                }
+            });
+            __syncthreads();
+            const int n = *tie_count;
+            if (n >= 1 && n <= SMP_TIES) {                      // (none: cannot be, the bucket was chosen for its weight)
+                const float s = value_of_ordered(value_bits);
+                const u64 w = MASS ? fixed_mass(s, smax) : 1;
+                u64 j = w ? (target - above) / w : 0;           // so many of the tied candidates lie above c*
+                if (j > (u64)(n - 1)) j = (u64)(n - 1);
+                for (int k = threadIdx.x; k < n; k += SMP_THREADS) {      // ids rise as keys fall: the j-th smallest id
+                    const int id = ties[k];
+                    int rank = 0;
+                    for (int q = 0; q < n; ++q) rank += ties[q] < id;
+                    if ((u64)rank == j) {
+                        shared[0] = prefix | (u64)((1 << SMP_ID_BITS) - 1 - id);
+                        shared[1] = above + (j + 1) * w;
+                    }
+                }
+                __syncthreads();
+                prefix = shared[0];
+                *incl = shared[1];
+                __syncthreads();
+                return prefix;
+            }
+        }
         for (int i = threadIdx.x; i < 256 * SMP_COPIES; i += SMP_THREADS) hist[i] = 0;
         __syncthreads();
         const u64 hi_mask = shift == 48 ? 0 : (~(u64)0) << (shift + 8);
-        for (int i = threadIdx.x; i < vocab; i += SMP_THREADS) {
-            const float s = row.scaled(i);
+        for_each_logit(row, vocab, [&](int i, float l) {
+            const float s = l * row.inv_temperature;
             const u64 c = composite(s, i);
             if (c >= floor_key && (c & hi_mask) == (prefix & hi_mask)) {
-                const u64 w = MASS ? (u64)(expf(s - smax) * SMP_FIXED) : 1;
+                const u64 w = MASS ? fixed_mass(s, smax) : 1;
                 atomicAdd(&hist[((c >> shift) & 255) * SMP_COPIES + (threadIdx.x & (SMP_COPIES - 1))], w);
             }
-        }
+        });
         __syncthreads();
         if (threadIdx.x < 256) {
             u64 t = 0;
@@ -75,17 +201,7 @@ __device__ u64 descend(const RowView& row, int vocab, float smax, u64 floor_key,
             bins[threadIdx.x] = t;
         }
         __syncthreads();
-        if (threadIdx.x == 0) {
-            u64 acc = above;
-            int b = 255;
-            for (; b > 0; --b) {
-                if (acc + bins[b] > target) break;
-                acc += bins[b];
-            }
-            shared[0] = acc;                   // weight above bucket b
-            shared[1] = (u64)b;
-            shared[2] = acc + bins[b];         // weight down to and including bucket b
-        }
+        pick_bin(bins, above, target, shared);
         __syncthreads();
         above = shared[0];
         prefix |= shared[1] << shift;
@@ -102,6 +218,8 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
     __shared__ u64 hist[256 * SMP_COPIES];
     __shared__ u64 bins[256];
     __shared__ u64 shared[4];
+    __shared__ int ties[SMP_TIES];
+    __shared__ int tie_count;
     __shared__ float fscratch[16];
     __shared__ int iscratch[16];
     RowView row;
@@ -110,14 +228,14 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
                    ? seen + (size_t)(seen_rows ? seen_rows[blockIdx.x] : (int)blockIdx.x) * vocab : nullptr;
     row.penalty = penalty;
     row.inv_temperature = temperature > 0.f ? 1.0f / temperature : 1.0f;
+    row.wide = vocab % 4 == 0 && ((uintptr_t)row.logits & 15) == 0 && ((uintptr_t)row.seen & 3) == 0;
 
     if (!(temperature > 0.f)) {                            // greedy: the first maximum (src/sampling.rs:131-139)
         float v = -INFINITY;
         int idx = 0x7FFFFFFF;
-        for (int i = threadIdx.x; i < vocab; i += SMP_THREADS) {
-            const float l = row.penalised(i);
+        for_each_logit(row, vocab, [&](int i, float l) {
             if (l > v || (l == v && i < idx)) { v = l; idx = i; }
-        }
+        });
         for (int m = RI_WAVE / 2; m > 0; m >>= 1) {
             const float ov = __shfl_xor(v, m, RI_WAVE);
             const int oi = __shfl_xor(idx, m, RI_WAVE);
@@ -134,19 +252,19 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
     }
 
     float smax = -INFINITY;
-    for (int i = threadIdx.x; i < vocab; i += SMP_THREADS) smax = fmaxf(smax, row.scaled(i));
+    for_each_logit(row, vocab, [&](int, float l) { smax = fmaxf(smax, l * row.inv_temperature); });
     smax = block_max(smax, fscratch);
 
     u64 floor_key = 0, incl = 0;
     if (top_k > 0 && top_k < vocab)                       // the k-th candidate of the order closes the kept set
-        floor_key = descend<false>(row, vocab, smax, 0, (u64)(top_k - 1), hist, bins, shared, &incl);
+        floor_key = descend<false>(row, vocab, smax, 0, (u64)(top_k - 1), hist, bins, shared, ties, &tie_count, &incl);
     // total mass of the kept set: descend to the very last candidate (target = everything but one unit)
     // would cost seven more passes; one exact integer sum does it
     u64 z = 0;
-    for (int i = threadIdx.x; i < vocab; i += SMP_THREADS) {
-        const float s = row.scaled(i);
-        if (composite(s, i) >= floor_key) z += (u64)(expf(s - smax) * SMP_FIXED);
-    }
+    for_each_logit(row, vocab, [&](int i, float l) {
+        const float s = l * row.inv_temperature;
+        if (composite(s, i) >= floor_key) z += fixed_mass(s, smax);
+    });
     for (int m = RI_WAVE / 2; m > 0; m >>= 1) z += __shfl_xor(z, m, RI_WAVE);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) bins[threadIdx.x >> 6] = z;
@@ -159,11 +277,12 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
         u64 want = (u64)ceil((double)top_p * (double)z);
         if (want < 1) want = 1;
         if (want > z) want = z;
-        floor_key = descend<true>(row, vocab, smax, floor_key, want - 1, hist, bins, shared, &incl);
+        floor_key = descend<true>(row, vocab, smax, floor_key, want - 1, hist, bins, shared, ties, &tie_count, &incl);
         z = incl;                                          // the kept mass, to be normalised by
     }
     const u64 target = (u64)((double)uniform[blockIdx.x] * (double)z);     // r < 1, so target < z
-    const u64 pick = descend<true>(row, vocab, smax, floor_key, target < z ? target : z - 1, hist, bins, shared, &incl);
+    const u64 pick = descend<true>(row, vocab, smax, floor_key, target < z ? target : z - 1, hist, bins, shared, ties,
+                                  &tie_count, &incl);
     if (threadIdx.x == 0) out[blockIdx.x] = (1 << SMP_ID_BITS) - 1 - (int)(pick & ((1 << SMP_ID_BITS) - 1));
 }
 

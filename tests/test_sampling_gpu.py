@@ -27,9 +27,10 @@ def plain_pick(logits, r, temperature, top_k, top_p, penalty, history):
     (0.8, 0, 1.0, 1.0), (1.3, 5, 1.0, 1.0), (0.7, 0, 0.8, 1.0), (1.0, 12, 0.6, 1.3), (0.0, 0, 1.0, 1.7),
     (1.0, 1, 1.0, 1.0), (0.5, 0, 0.05, 1.0), (2.0, 400, 0.999, 1.0),
 ])
-def test_same_token_as_the_plain_sampler(ops, temperature, top_k, top_p, penalty):
+@pytest.mark.parametrize("vocab", [411, 4096])                  # no power of two; and rows read 16 bytes at a time,
+def test_same_token_as_the_plain_sampler(ops, temperature, top_k, top_p, penalty, vocab):   # more ties than are listed
     rng = np.random.default_rng(int(temperature * 10) + top_k)
-    vocab, rows = 411, 24                                       # a vocabulary that is no power of two
+    rows = 24
     logits = (3.0 * rng.normal(size=(rows, vocab))).astype(np.float32)
     logits[:, 10] = logits[:, 20]                               # ties inside every row
     logits[3, :] = 0.25                                         # a row of equal logits: the id order decides alone
