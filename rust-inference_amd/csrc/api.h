@@ -130,6 +130,15 @@ int ri_sample(int32_t* out, const float* logits, const uint8_t* seen, const int3
               int rows, int vocab, float temperature, int top_k, float top_p, float penalty, void* stream);
 
 // seen[rows[i], tokens[i]] = 1 for i < n.
+// The same selection (temperature > 0 only) with every row cut over many workgroups and one launch per
+// pass: the form for large vocabularies, where one workgroup's loads in flight bound a pass.  The same
+// token as ri_sample for the same arguments.  workspace: ri_sample_split_workspace_bytes(rows) bytes, any
+// contents.
+long ri_sample_split_workspace_bytes(int rows);
+int ri_sample_split(int32_t* out, const float* logits, const uint8_t* seen, const int32_t* seen_rows,
+                    const float* uniform, void* workspace, int rows, int vocab, float temperature, int top_k,
+                    float top_p, float penalty, void* stream);
+
 int ri_mark_seen(uint8_t* seen, const int32_t* rows, const int32_t* tokens, int n, int vocab, void* stream);
 
 #ifdef __cplusplus

@@ -41,6 +41,8 @@ _SIGNATURES = {
     "ri_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_float,
                   c_void_p],
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "ri_sample_split": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
+                        c_float, c_float, c_void_p],
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
@@ -167,13 +169,32 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return ids
 
 
+# From this vocabulary size on a sampled row is cut over many workgroups (at 151,936 entries: 8 short
+# launches instead of one long one).
+SPLIT_SAMPLER_MIN_VOCAB = 16384
+
+
 def sample(logits: torch.Tensor, uniform, temperature: float, top_k: int = 0, top_p: float = 1.0,
-           penalty: float = 1.0, seen: torch.Tensor | None = None, seen_rows: torch.Tensor | None = None) -> torch.Tensor:
+           penalty: float = 1.0, seen: torch.Tensor | None = None, seen_rows: torch.Tensor | None = None,
+           split: bool | None = None) -> torch.Tensor:
     """int32 token per row of float32 ``logits``: repetition penalty over the ids marked in ``seen``
     (uint8 ``[*, vocab]``), greedy when the temperature is not positive, else temperature, top-k, top-p
-    and one draw with ``uniform[r]`` in [0, 1)."""
+    and one draw with ``uniform[r]`` in [0, 1).  ``split``: the many-workgroups form (the same token;
+    by default for large vocabularies)."""
     rows, vocab = logits.shape
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    if split is None:
+        split = vocab >= SPLIT_SAMPLER_MIN_VOCAB
+    if split and temperature > 0:
+        lib = load()
+        lib.ri_sample_split_workspace_bytes.restype = ctypes.c_long
+        lib.ri_sample_split_workspace_bytes.argtypes = [c_int]
+        ws = torch.empty((lib.ri_sample_split_workspace_bytes(rows),), dtype=torch.uint8, device=logits.device)
+        _call("ri_sample_split", _dev(out, "out"), _dev(logits, "logits", torch.float32),
+              _opt(seen, "seen", torch.uint8), _opt(seen_rows, "seen_rows", torch.int32, (rows,)),
+              _dev(uniform, "uniform", torch.float32, (rows,)), _dev(ws, "workspace"), rows, vocab, float(temperature),
+              int(top_k), float(top_p), float(penalty), _stream())
+        return out
     _call("ri_sample", _dev(out, "out"), _dev(logits, "logits", torch.float32),
           _opt(seen, "seen", torch.uint8), _opt(seen_rows, "seen_rows", torch.int32, (rows,)),
           _opt(uniform, "uniform", torch.float32, (rows,)), rows, vocab, float(temperature), int(top_k), float(top_p),

@@ -27,8 +27,9 @@ def plain_pick(logits, r, temperature, top_k, top_p, penalty, history):
     (0.8, 0, 1.0, 1.0), (1.3, 5, 1.0, 1.0), (0.7, 0, 0.8, 1.0), (1.0, 12, 0.6, 1.3), (0.0, 0, 1.0, 1.7),
     (1.0, 1, 1.0, 1.0), (0.5, 0, 0.05, 1.0), (2.0, 400, 0.999, 1.0),
 ])
+@pytest.mark.parametrize("split", [False, True])                 # a workgroup a row; a row over many workgroups
 @pytest.mark.parametrize("vocab", [411, 4096])                  # no power of two; and rows read 16 bytes at a time,
-def test_same_token_as_the_plain_sampler(ops, temperature, top_k, top_p, penalty, vocab):   # more ties than are listed
+def test_same_token_as_the_plain_sampler(ops, temperature, top_k, top_p, penalty, vocab, split):   # more ties than are listed
     rng = np.random.default_rng(int(temperature * 10) + top_k)
     rows = 24
     logits = (3.0 * rng.normal(size=(rows, vocab))).astype(np.float32)
@@ -44,7 +45,7 @@ def test_same_token_as_the_plain_sampler(ops, temperature, top_k, top_p, penalty
     ht = [t for r in range(rows) for t in history[r]]
     ops.mark_seen(seen, torch.tensor(hr, dtype=torch.int32, device=DEV), torch.tensor(ht, dtype=torch.int32, device=DEV))
     got = ops.sample(torch.tensor(logits, device=DEV), torch.tensor(rs, dtype=torch.float32, device=DEV), temperature,
-                     top_k, top_p, penalty, seen if penalty != 1.0 else None).tolist()
+                     top_k, top_p, penalty, seen if penalty != 1.0 else None, split=split).tolist()
     want = [plain_pick(logits[r], rs[r], temperature, top_k, top_p, penalty, history[r]) for r in range(rows)]
     # the device sums masses exactly, the plain sampler in float32 in drawing order: a draw that falls within
     # float32 rounding of a boundary may land on the neighbour; allow that for at most one row, and only then
@@ -68,6 +69,38 @@ def test_large_vocabulary_and_distribution(ops):
     assert abs(np.mean([p == 150000 for p in picks]) - 0.75) < 0.03
     again = ops.sample(logits.expand(4000, vocab).contiguous(), rs, 1.0).tolist()
     assert picks == again                                         # the same draws, the same tokens
+    assert picks == ops.sample(logits.expand(4000, vocab).contiguous(), rs, 1.0, split=False).tolist()
+
+
+def test_both_forms_pick_the_same_tokens_of_a_large_vocabulary(ops):
+    """Logits like a model's over 151,936 entries, with ties, penalty, top-k and top-p: the row cut over many
+    workgroups gives the token that the single workgroup gives, and a few rows are checked against the
+    plain sampler."""
+    rng = np.random.default_rng(11)
+    vocab, rows = 151936, 16
+    logits = (2.5 * rng.normal(size=(rows, vocab))).astype(np.float32)
+    logits[:, 5000:5400] = logits[:, 5000:5001]                  # 400 tied candidates in every row
+    logits[2, :] = 1.5                                           # more ties than are listed
+    logits[3, 70000] = 30.0                                      # one token owns the row
+    history = [[int(t) for t in rng.integers(0, vocab, 50)] for _ in range(rows)]
+    seen = torch.zeros((rows, vocab), dtype=torch.uint8, device=DEV)
+    ops.mark_seen(seen, torch.tensor([r for r in range(rows) for _ in history[r]], dtype=torch.int32, device=DEV),
+                  torch.tensor([t for r in range(rows) for t in history[r]], dtype=torch.int32, device=DEV))
+    gen = PlainRng(3)
+    rs = [gen.next_f32() for _ in range(rows)]
+    dl, dr = torch.tensor(logits, device=DEV), torch.tensor(rs, dtype=torch.float32, device=DEV)
+    # (47 kept of a row of equal logits: 0.9 of them is no whole number, so float32 sums cannot sit on the edge)
+    for temperature, top_k, top_p, penalty in ((0.8, 0, 1.0, 1.0), (1.0, 47, 0.9, 1.2), (1.5, 0, 0.95, 1.0),
+                                               (0.7, 3000, 1.0, 1.1)):
+        sn = seen if penalty != 1.0 else None
+        one = ops.sample(dl, dr, temperature, top_k, top_p, penalty, sn, split=False).tolist()
+        many = ops.sample(dl, dr, temperature, top_k, top_p, penalty, sn, split=True).tolist()
+        assert one == many, (temperature, top_k, top_p, penalty)
+        for r in (0, 2, 3):
+            want = plain_pick(logits[r], rs[r], temperature, top_k, top_p, penalty, history[r])
+            if many[r] != want:                                   # only within float32 rounding of a boundary
+                order, probs = candidates(penalise(logits[r], history[r], penalty), temperature, top_k, top_p)
+                assert np.min(np.abs(np.cumsum(probs.astype(np.float64)) - rs[r])) < 1e-5, (r, many[r], want)
 
 
 def test_top_p_drops_the_tail_and_top_k_one_is_greedy(ops):
