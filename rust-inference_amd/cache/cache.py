@@ -170,6 +170,14 @@ class Cache:
     def has_state(self, entry: int) -> bool:
         return entry in self._state
 
+    def snapshot_state(self) -> dict[int, torch.Tensor]:
+        """Copies of all state arenas (for a step that has to be run twice and count once)."""
+        return {e: arena.clone() for e, arena in self._state.items()}
+
+    def restore_state(self, snapshot: dict[int, torch.Tensor]) -> None:
+        for e, saved in snapshot.items():
+            self._state[e].copy_(saved)
+
     # ---- accounting
     def free_pages(self) -> list[int]:
         return [g.pool.free_count for g in self.groups]

@@ -182,8 +182,11 @@ class Engine:
         ctx = self.build_context(entries, staging=dg.staging, full_width=True)
         if dg.graph is None:
             # once eagerly (libraries set themselves up outside the capture), then capture; writing
-            # the same keys and values to the same places twice changes nothing
+            # the same keys and values to the same places twice changes nothing, and per-sequence
+            # state is put back to where it was before the rehearsal
+            saved = self.cache.snapshot_state()
             self.model.forward(ctx, self.cache)
+            self.cache.restore_state(saved)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):

@@ -42,7 +42,9 @@ class Mixer(Part):
     step's page table of its group; it returns ``[T, hidden]``.  Tokens of a
     sequence are contiguous and in order (``ctx.cu_seqlens``); a mixer with state
     reads its slot's row, consumes the sequence's tokens in order and writes the
-    row back.
+    row back.  Decode steps may be captured as a graph and replayed for other slots
+    and positions: a mixer that is to run there takes them from the context's device
+    tensors (``ctx.slots``, ``ctx.tok_pos``, the page table), not from its host lists.
     """
 
     def cache_need(self):

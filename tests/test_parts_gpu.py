@@ -249,6 +249,12 @@ def register_toy():
             return StateNeed((self.hidden + 1,), torch.float32)
 
         def forward(self, x, ctx, store, page_table):
+            if ctx.is_decode:       # one token a sequence: all on the device, so that the step can be captured as a graph
+                rows = ctx.slots.long()
+                state = store.index_select(0, rows)
+                total, count = state[:, :-1] + x.float(), state[:, -1] + 1
+                store.index_copy_(0, rows, torch.cat([total, count[:, None]], 1))
+                return ((total / count[:, None]) @ self.w.T).to(x.dtype)
             out = torch.empty_like(x)
             begin = 0
             for slot, n in zip(ctx.slot_list, ctx.new_counts):        # a sequence's tokens are contiguous, in order
@@ -425,3 +431,25 @@ def test_toy_architecture_builds_and_steps_through_the_unchanged_engine(toy_dir,
     windowed = next(g for g in engine.cache.groups if g.need.window)
     full = next(g for g in engine.cache.groups if not g.need.window)
     assert len(windowed.pool.pages_of(slot)) == 2 and len(full.pool.pages_of(slot)) == 4
+
+
+def test_toy_model_decodes_the_same_through_graphs(toy_dir):
+    """Decode steps captured as graphs: the mixer with state is rehearsed once before the capture, and its
+    state must count that step once; sequences leave, so another batch size gets a graph of its own."""
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.parts import load_model
+    model = load_model(toy_dir, torch.bfloat16)
+    rng = np.random.default_rng(9)
+    prompts = [[int(x) for x in rng.integers(0, TOY["vocab_size"], n)] for n in (40, 3, 17)]
+    outs = []
+    for graphs in (False, True):
+        eng = Engine(model, model.new_cache(max_tokens=3 * 128, num_slots=3, max_seq_len=128), use_graphs=graphs)
+        slots = [eng.cache.acquire() for _ in prompts]
+        eng.step([StepEntry(s, p, "last") for s, p in zip(slots, prompts)])
+        rows = []
+        for step in range(14):
+            live = slots if step < 8 else slots[1:]
+            rows.append(eng.step([StepEntry(s, [(5 * step + s) % TOY["vocab_size"]], "last") for s in live]).clone())
+        outs.append(rows)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
