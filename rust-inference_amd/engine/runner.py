@@ -1,9 +1,9 @@
 """The command line, in the manner of the reference's runner (src/bin/runner.rs:24-123): the same
 option names and meanings where it has them.
 
-    runner <MODEL_DIR> [-p PROMPT] [-n N] [--temperature T] [--top-k K] [--top-p P]
+    runner <MODEL_DIR> [-p PROMPT] [-n N] [--chat [--think]] [--temperature T] [--top-k K] [--top-p P]
            [--repetition-penalty R] [--seed S] [--ignore-eos] [--max-pages N] [--pages-per-seq N]
-           [--dtype bfloat16|float32] [--profile]
+           [-t THREADS] [--dtype bfloat16|float32] [--profile]
 
 The prompt is text when the model folder has a tokenizer.json (read with the `tokenizers` package),
 else a list of token ids (`-p "5 17 3"` or `--prompt-ids 5,17,3`); it is read from standard input when
@@ -27,10 +27,13 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--prompt-ids", action="append", help="a prompt as comma-separated token ids")
     ap.add_argument("--batch", action="store_true", help="read one prompt per line of standard input")
     ap.add_argument("-n", "--max-new-tokens", type=int, default=600, help="number of tokens to generate")
+    ap.add_argument("--chat", action="store_true", help="wrap the prompt in the Qwen chat template")
+    ap.add_argument("--think", action="store_true", help="with --chat, leave thinking mode enabled")
     ap.add_argument("--ignore-eos", action="store_true", help="keep generating past end-of-sequence tokens")
     ap.add_argument("--tokenizer", help="directory holding tokenizer.json, if not the model directory")
     ap.add_argument("--max-pages", type=int, default=256, help="KV cache pages per layer (32 tokens each)")
     ap.add_argument("--pages-per-seq", type=int, default=128, help="maximum KV pages per sequence")
+    ap.add_argument("-t", "--threads", type=int, default=None, help="host worker threads (defaults to all cores)")
     ap.add_argument("--profile", action="store_true", help="print a per-step timing summary at the end")
     ap.add_argument("--temperature", type=float, default=0.0, help="sampling temperature; 0 = greedy")
     ap.add_argument("--top-k", type=int, default=0, help="keep only the k most likely tokens (0 = off)")
@@ -43,6 +46,34 @@ def build_parser() -> argparse.ArgumentParser:
                     "(default: eos_token_id of generation_config.json or config.json, if present)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     return ap
+
+
+def chat_prompt(user: str, enable_thinking: bool) -> str:
+    """The Qwen chat format for a single user turn; without thinking, an empty think block opens the
+    answer (src/tokenizer/mod.rs:402-408)."""
+    text = f"<|im_start|>user\n{user}<|im_end|>\n<|im_start|>assistant\n"
+    if not enable_thinking:
+        text += "<think>\n\n</think>\n\n"
+    return text
+
+
+class StreamPrinter:
+    """Prints a sequence's text as its tokens arrive, holding back bytes that do not yet form whole
+    characters (the reference's StreamDecoder: src/tokenizer/mod.rs:411-416)."""
+
+    def __init__(self, tokenizer, out=sys.stdout):
+        self.tokenizer, self.out, self.ids, self.printed = tokenizer, out, [], 0
+
+    def push(self, token: int) -> None:
+        if self.tokenizer is None:
+            self.out.write(f"{token} ")
+        else:
+            self.ids.append(token)
+            text = self.tokenizer.decode(self.ids)
+            if not text.endswith("\ufffd"):                 # an unfinished character decodes to U+FFFD: wait for the rest
+                self.out.write(text[self.printed:])
+                self.printed = len(text)
+        self.out.flush()
 
 
 def load_tokenizer(folder: str):
@@ -72,8 +103,17 @@ def parse_ids(text: str) -> list[int]:
 
 
 def main(argv=None) -> int:
-    args = build_parser().parse_args(argv)
+    ap = build_parser()
+    args = ap.parse_args(argv)
+    if args.think and not args.chat:
+        ap.error("--think requires --chat")
+    if args.threads:
+        import torch
+        torch.set_num_threads(args.threads)
     tokenizer = load_tokenizer(args.tokenizer or args.model_dir)
+    if args.chat and tokenizer is None:
+        print("error: --chat wraps text and needs a tokenizer.json", file=sys.stderr)
+        return 1
     raw = list(args.prompt or [])
     id_prompts = [parse_ids(p) for p in (args.prompt_ids or [])]
     if not raw and not id_prompts:
@@ -81,6 +121,8 @@ def main(argv=None) -> int:
         raw = [ln for ln in lines if ln.strip()] if args.batch else ["\n".join(lines).strip()]
     prompts = list(id_prompts)
     for p in raw:
+        if args.chat:
+            p = chat_prompt(p, args.think)                             # src/bin/runner.rs:233
         prompts.append(tokenizer.encode(p).ids if tokenizer is not None else parse_ids(p))
     if not prompts or any(len(p) == 0 for p in prompts):
         print("error: empty prompt", file=sys.stderr)                  # src/bin/runner.rs:235-237
@@ -100,11 +142,11 @@ def main(argv=None) -> int:
     stop = parse_ids(args.stop_token_ids) if args.stop_token_ids is not None else default_stop_ids(args.model_dir)
 
     single = len(prompts) == 1
+    printer = StreamPrinter(tokenizer)
 
     def on_token(request, token):
         if single:                                                     # streamed, as the reference prints
-            sys.stdout.write(tokenizer.decode([token]) if tokenizer is not None else f"{token} ")
-            sys.stdout.flush()
+            printer.push(token)
 
     try:
         res = model.generate(prompts, max_new_tokens=args.max_new_tokens, temperature=args.temperature,

@@ -108,3 +108,25 @@ def test_temperature_sampling_is_seeded(model_dirs):
     c = model.generate(prompts, max_new_tokens=12, temperature=0.8, seed=2).tokens
     alone = model.generate(prompts[:1], max_new_tokens=12, temperature=0.8, seed=1).tokens
     assert a == b and a != c and alone[0] == a[0]
+
+
+def test_the_command_line_generates_what_the_plain_implementation_does(model_dirs):
+    """bin/runner with prompts as token ids (the folder has no tokenizer.json): greedy, float32; one prompt
+    is streamed to standard output, two are printed a line each; a stop token from the command line."""
+    cfg, _ = read_model_f64(model_dirs["A"])
+    prompts = prompts_for(cfg, [7, 12], 9)
+    want = plain_greedy_with_margins(model_dirs["A"], prompts, 6)
+    base = [sys.executable, os.path.join(ROOT, "bin", "runner"), model_dirs["A"], "--dtype", "float32", "-n", "6"]
+    one = subprocess.run(base + ["-p", " ".join(map(str, prompts[0]))], capture_output=True, text=True, timeout=120)
+    assert one.returncode == 0, one.stderr
+    assert [int(t) for t in one.stdout.split()] == want[0][0]
+    assert "prefill: 7 tokens" in one.stderr and "decode: 5 tokens" in one.stderr      # src/bin/runner.rs:243-251
+    two = subprocess.run(base + ["--prompt-ids", ",".join(map(str, prompts[0])), "--prompt-ids",
+                                 ",".join(map(str, prompts[1])), "--profile"], capture_output=True, text=True, timeout=120)
+    assert two.returncode == 0, two.stderr
+    assert [[int(t) for t in ln.split()] for ln in two.stdout.strip().splitlines()] == [w[0] for w in want]
+    assert "profile: 1 batches, 5 decode steps" in two.stderr
+    stop = want[1][0][2]
+    cut = subprocess.run(base + ["-p", " ".join(map(str, prompts[1])), "--stop-token-ids", str(stop)],
+                         capture_output=True, text=True, timeout=120)
+    assert cut.returncode == 0 and [int(t) for t in cut.stdout.split()] == want[1][0][:want[1][0].index(stop)]

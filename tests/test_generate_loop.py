@@ -148,3 +148,51 @@ def test_plan_step_layout():
         plan_step([StepEntry(0, [1], [1])], [0], VOCAB)
     with pytest.raises(ShapeError, match="no token"):
         plan_step([StepEntry(0, [])], [0], VOCAB)
+
+
+# ------------------------------------------------------------------------------------------------ the command line
+def test_runner_options_are_the_references():
+    """Names, short forms and defaults of src/bin/runner.rs:24-123 for the options this build has."""
+    from rust_inference_amd.engine.runner import build_parser
+    a = build_parser().parse_args(["some/dir"])
+    assert (a.model_dir, a.prompt, a.max_new_tokens, a.chat, a.think, a.ignore_eos) == ("some/dir", None, 600, False, False, False)
+    assert (a.max_pages, a.pages_per_seq, a.threads, a.profile) == (256, 128, None, False)
+    assert (a.temperature, a.top_k, a.top_p, a.repetition_penalty, a.seed) == (0.0, 0, 1.0, 1.0, 0x5EED)
+    b = build_parser().parse_args(["d", "-p", "hello", "-n", "7", "-t", "3", "--temperature", "0.5", "--top-k", "4", "--top-p",
+                                   "0.9", "--repetition-penalty", "1.1", "--seed", "0x10", "--chat", "--think",
+                                   "--ignore-eos", "--tokenizer", "tok", "--max-pages", "9", "--pages-per-seq", "2"])
+    assert (b.prompt, b.max_new_tokens, b.threads, b.seed, b.tokenizer) == (["hello"], 7, 3, 16, "tok")
+    assert b.chat and b.think and b.ignore_eos and (b.max_pages, b.pages_per_seq) == (9, 2)
+
+
+def test_chat_prompt_and_streamed_text():
+    from rust_inference_amd.engine.runner import StreamPrinter, chat_prompt
+    # src/tokenizer/mod.rs:402-408
+    assert chat_prompt("hi", True) == "<|im_start|>user\nhi<|im_end|>\n<|im_start|>assistant\n"
+    assert chat_prompt("hi", False) == "<|im_start|>user\nhi<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\n"
+
+    class TwoByteTokenizer:                                  # ids are bytes: a character may span two tokens
+        def decode(self, ids):
+            return bytes(ids).decode("utf-8", errors="replace")
+
+    import io
+    out = io.StringIO()
+    printer = StreamPrinter(TwoByteTokenizer(), out)
+    pieces = []
+    for b in "aé!".encode():
+        printer.push(b)
+        pieces.append(out.getvalue())
+    assert pieces == ["a", "a", "aé", "aé!"]                 # nothing is printed for half a character
+    out = io.StringIO()
+    StreamPrinter(None, out).push(17)
+    assert out.getvalue() == "17 "
+
+
+def test_runner_refuses_what_it_cannot_do(tmp_path, capsys):
+    from rust_inference_amd.engine.runner import main
+    with pytest.raises(SystemExit):
+        main([str(tmp_path), "-p", "1 2", "--think"])        # --think requires --chat
+    assert main([str(tmp_path), "-p", "hello", "--chat"]) == 1          # no tokenizer.json in the folder
+    assert "tokenizer.json" in capsys.readouterr().err
+    assert main([str(tmp_path), "-p", ""]) == 1
+    assert "empty prompt" in capsys.readouterr().err
