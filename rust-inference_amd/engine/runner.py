@@ -3,7 +3,7 @@ option names and meanings where it has them.
 
     runner <MODEL_DIR> [-p PROMPT] [-n N] [--chat [--think]] [--temperature T] [--top-k K] [--top-p P]
            [--repetition-penalty R] [--seed S] [--ignore-eos] [--max-pages N] [--pages-per-seq N]
-           [-t THREADS] [--dtype bfloat16|float32] [--profile]
+           [-t THREADS] [--dtype bfloat16|float32] [--profile] [--random [--random-seed S]]
 
 The prompt is text when the model folder has a tokenizer.json (read with the `tokenizers` package),
 else a list of token ids (`-p "5 17 3"` or `--prompt-ids 5,17,3`); it is read from standard input when
@@ -45,6 +45,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--stop-token-ids", default=None, help="comma-separated ids that end a sequence "
                     "(default: eos_token_id of generation_config.json or config.json, if present)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    ap.add_argument("--random", action="store_true", help="MODEL_DIR needs only a config.json (or is one): the weights "
+                    "are made in memory, N(0, 0.02) with gains 1 + N(0, 0.1), from --random-seed")
+    ap.add_argument("--random-seed", type=int, default=0, help="seed of the weights made by --random")
     return ap
 
 
@@ -133,9 +136,15 @@ def main(argv=None) -> int:
     t0 = time.perf_counter()
     try:
         per_seq = args.pages_per_seq * 32
-        model = Model.load(args.model_dir, dtype=args.dtype, max_batch=min(len(prompts), 64), max_seq_len=per_seq,
-                           max_tokens=args.max_pages * 32, use_graphs=not args.no_graphs)
-    except InferenceError as e:
+        options = dict(max_batch=min(len(prompts), 64), max_seq_len=per_seq, max_tokens=args.max_pages * 32,
+                       use_graphs=not args.no_graphs)
+        if args.random:
+            path = args.model_dir if os.path.isfile(args.model_dir) else os.path.join(args.model_dir, "config.json")
+            with open(path) as f:
+                model = Model.random(json.load(f), seed=args.random_seed, dtype=args.dtype, **options)
+        else:
+            model = Model.load(args.model_dir, dtype=args.dtype, **options)
+    except (InferenceError, OSError, json.JSONDecodeError) as e:
         print(f"error: {e}", file=sys.stderr)
         return 1
     print(f"loaded {args.model_dir} in {time.perf_counter() - t0:.2f} s", file=sys.stderr)

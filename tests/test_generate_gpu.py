@@ -130,3 +130,18 @@ def test_the_command_line_generates_what_the_plain_implementation_does(model_dir
     cut = subprocess.run(base + ["-p", " ".join(map(str, prompts[1])), "--stop-token-ids", str(stop)],
                          capture_output=True, text=True, timeout=120)
     assert cut.returncode == 0 and [int(t) for t in cut.stdout.split()] == want[1][0][:want[1][0].index(stop)]
+
+
+def test_the_command_line_with_random_weights(tmp_path):
+    """--random: a config.json is enough; the same seed gives the same tokens, another seed others."""
+    from conftest import TINY_C
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(TINY_C, f)
+    base = [sys.executable, os.path.join(ROOT, "bin", "runner"), "-p", "5 17 3 250", "-n", "12", "--random"]
+    runs = [subprocess.run(base + [where, "--random-seed", seed], capture_output=True, text=True, timeout=120)
+            for where, seed in ((str(tmp_path), "4"), (str(tmp_path / "config.json"), "4"), (str(tmp_path), "5"))]
+    assert all(r.returncode == 0 for r in runs), [r.stderr for r in runs]
+    outs = [[int(t) for t in r.stdout.split()] for r in runs]
+    assert len(outs[0]) == 12 and outs[0] == outs[1] and outs[0] != outs[2]
+    missing = subprocess.run(base + [str(tmp_path / "nowhere")], capture_output=True, text=True, timeout=120)
+    assert missing.returncode == 1 and "error:" in missing.stderr
