@@ -8,6 +8,8 @@ of all later queries.
 """
 from __future__ import annotations
 
+import numpy as np
+
 from ..errors import CacheError
 
 UNMAPPED = -1
@@ -22,7 +24,8 @@ class PagePool:
         self.max_pages_per_slot, self.window = max_pages_per_slot, window
         self._free = list(range(num_pages - 1, -1, -1))
         self._owner = [UNMAPPED] * num_pages             # page -> slot, to catch double frees
-        self.tables = [[UNMAPPED] * max_pages_per_slot for _ in range(num_slots)]
+        # slot -> its pages by logical number: one array, so that a step's tables are one gather
+        self.tables = np.full((num_slots, max_pages_per_slot), UNMAPPED, dtype=np.int32)
 
     @property
     def free_count(self) -> int:
@@ -34,9 +37,10 @@ class PagePool:
 
     def pages_needed(self, slot: int, length_before: int, new_tokens: int) -> int:
         """How many pages ``reserve`` would take from the pool."""
-        table = self.tables[slot]
         first, last = length_before // self.page_size, -(-(length_before + new_tokens) // self.page_size)
-        return sum(1 for p in range(first, min(last, self.max_pages_per_slot)) if table[p] == UNMAPPED)
+        if last - first == 1 and last <= self.max_pages_per_slot:          # the usual step: one token more
+            return int(self.tables[slot, first] == UNMAPPED)
+        return int((self.tables[slot, first:min(last, self.max_pages_per_slot)] == UNMAPPED).sum())
 
     def reserve(self, slot: int, length_before: int, new_tokens: int) -> None:
         """Map pages for positions ``length_before .. length_before + new_tokens - 1``."""
@@ -51,16 +55,16 @@ class PagePool:
                     raise CacheError(f"cache out of pages ({self.num_pages} of {self.page_size} tokens in all)")
                 page = self._free.pop()
                 self._owner[page] = slot
-                table[logical] = page
+                table[logical] = page                                              # (a view: writes the array)
 
     def _give_back(self, slot: int, logical: int) -> None:
-        page = self.tables[slot][logical]
+        page = int(self.tables[slot, logical])
         if page == UNMAPPED:
             return
         if self._owner[page] != slot:
             raise CacheError(f"page {page} is in slot {slot}'s table but owned by {self._owner[page]}")
         self._owner[page] = UNMAPPED
-        self.tables[slot][logical] = UNMAPPED
+        self.tables[slot, logical] = UNMAPPED
         self._free.append(page)
 
     def trim_behind_window(self, slot: int, length: int) -> None:
@@ -72,16 +76,21 @@ class PagePool:
             self._give_back(slot, logical)
 
     def release(self, slot: int) -> None:
-        for logical in range(self.max_pages_per_slot):
+        for logical in np.nonzero(self.tables[slot] != UNMAPPED)[0].tolist():
             self._give_back(slot, logical)
 
     def pages_of(self, slot: int) -> list[int]:
-        return [p for p in self.tables[slot] if p != UNMAPPED]
+        row = self.tables[slot]
+        return row[row != UNMAPPED].tolist()
+
+    def gather(self, slots, width: int) -> np.ndarray:
+        """The tables of these slots, ``[len(slots), width]``, unmapped places as -1."""
+        return self.tables[np.asarray(slots, dtype=np.int64), :width]
 
     def check_consistent(self) -> None:
         """Every page is either free or in exactly one table; used by the tests."""
         seen = {}
-        for slot, table in enumerate(self.tables):
+        for slot, table in enumerate(self.tables.tolist()):
             for page in table:
                 if page == UNMAPPED:
                     continue

@@ -13,6 +13,9 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Sequence, Union
 
+import itertools
+
+import numpy as np
 import torch
 
 from ..errors import ShapeError
@@ -45,25 +48,31 @@ def wanted_indices(n: int, want: Want) -> list[int]:
 
 
 def plan_step(entries: Sequence[StepEntry], lengths: Sequence[int], vocab_size: int):
-    """The host-side layout of a step: flat tokens, each token's sequence and position,
-    the wanted rows.  ``lengths[i]`` is entry i's cache length before the step."""
+    """The host-side layout of a step: flat tokens, each token's sequence and position, where
+    each sequence starts among them, and the wanted rows, as int32 arrays.  ``lengths[i]`` is
+    entry i's cache length before the step."""
     if not entries:
         raise ShapeError("a step needs at least one entry")
-    tokens, tok_seq, tok_pos, cu, want_rows = [], [], [], [0], []
-    for b, (e, start) in enumerate(zip(entries, lengths)):
-        n = len(e.tokens)
+    counts = [len(e.tokens) for e in entries]
+    for b, (e, n) in enumerate(zip(entries, counts)):
         if n < 1:
             raise ShapeError(f"entry {b} (slot {e.slot}) brings no token")
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise ShapeError(f"token id {t} is outside the vocabulary of {vocab_size}")   # src/ops/embedding.rs:20-22
-        base = cu[-1]
-        tokens.extend(int(t) for t in e.tokens)
-        tok_seq.extend([b] * n)
-        tok_pos.extend(range(start, start + n))
-        want_rows.extend(base + i for i in wanted_indices(n, e.want))
-        cu.append(base + n)
-    return tokens, tok_seq, tok_pos, cu, want_rows
+    total = sum(counts)
+    tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int64, count=total)
+    if tokens.min() < 0 or tokens.max() >= vocab_size:
+        bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
+        raise ShapeError(f"token id {bad} is outside the vocabulary of {vocab_size}")       # src/ops/embedding.rs:20-22
+    cu = np.zeros(len(entries) + 1, dtype=np.int32)
+    np.cumsum(counts, out=cu[1:])
+    if total == len(entries):                                  # one token each: the common step
+        tok_seq = np.arange(total, dtype=np.int32)
+        tok_pos = np.asarray(lengths, dtype=np.int32)
+    else:
+        tok_seq = np.repeat(np.arange(len(entries), dtype=np.int32), counts)
+        tok_pos = (np.arange(total, dtype=np.int32) - np.repeat(cu[:-1] - np.asarray(lengths, dtype=np.int32), counts))
+    want_rows = np.asarray([int(cu[b]) + i for b, (e, n) in enumerate(zip(entries, counts))
+                            for i in wanted_indices(n, e.want)], dtype=np.int32)
+    return tokens.astype(np.int32), tok_seq, tok_pos.astype(np.int32), cu, want_rows
 
 
 class _Staging:
@@ -73,16 +82,21 @@ class _Staging:
     def __init__(self, capacity: int, device, depth: int = 4):
         self.capacity, self.device, self.turn = capacity, device, 0
         self.host = [torch.empty(capacity, dtype=torch.int32, pin_memory=True) for _ in range(depth)]
+        self.views = [h.numpy() for h in self.host]            # the same memory, for numpy to fill
         self.events = [None] * depth
         self.dev = torch.zeros(capacity, dtype=torch.int32, device=device)
 
-    def upload(self, values: list[int]) -> torch.Tensor:
-        n = len(values)
+    def begin(self, n: int) -> np.ndarray:
+        """The next host buffer's first ``n`` words, free to be written."""
         i = self.turn
-        self.turn = (i + 1) % len(self.host)
         if self.events[i] is not None:
             self.events[i].synchronize()
-        self.host[i][:n] = torch.tensor(values, dtype=torch.int32)
+        return self.views[i][:n]
+
+    def upload(self, n: int) -> torch.Tensor:
+        """Send what ``begin`` handed out; returns the device buffer."""
+        i = self.turn
+        self.turn = (i + 1) % len(self.host)
         self.dev[:n].copy_(self.host[i][:n], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
@@ -134,21 +148,28 @@ class Engine:
         len_after = [s + n for s, n in zip(starts, counts)]
         max_len = max(len_after)
         width = cache.max_pages_per_slot if full_width else -(-max_len // cache.page_size)
+        T, B = len(tokens), len(entries)
+        # one block of int32 words for everything the kernels read of the layout, every piece on a
+        # 16-byte boundary: tokens, sequence and position of each, sequence starts, slots, lengths
+        # after the step, wanted rows, then a page table per key/value group
         pieces = [tokens, tok_seq, tok_pos, cu, slots, len_after, want_rows]
-        for g in cache.groups:
-            rows = g.table_rows(slots, width)
-            pieces.append([p for row in rows for p in (row + [-1] * (width - len(row)))])
-        flat, offsets = [], []
-        for p in pieces:
-            offsets.append(len(flat))
-            flat.extend(p)
-            flat.extend([0] * (-len(flat) % 4))           # keep every piece 16-byte aligned
-        dev = (staging or self._stage(len(flat))).upload(flat)
+        sizes = [len(p) for p in pieces] + [B * width] * len(cache.groups)
+        offsets, at = [], 0
+        for n in sizes:
+            offsets.append(at)
+            at += -(-n // 4) * 4
+        stage = staging or self._stage(at)
+        words = stage.begin(at)
+        for p, off in zip(pieces, offsets):
+            words[off:off + len(p)] = p
+        for gi, g in enumerate(cache.groups):
+            off = offsets[len(pieces) + gi]
+            words[off:off + B * width].reshape(B, width)[:] = g.table_rows(slots, width)
+        dev = stage.upload(at)
 
         def piece(i, n):
             return dev[offsets[i]:offsets[i] + n]
 
-        T, B = len(tokens), len(entries)
         ctx = StepContext(T=T, B=B, new_counts=counts, slot_list=slots, starts=starts,
                           tokens=piece(0, T), tok_seq=piece(1, T), tok_pos=piece(2, T), cu_seqlens=piece(3, B + 1),
                           slots=piece(4, B), len_after=piece(5, B), want_rows=piece(6, len(want_rows)),

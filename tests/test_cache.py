@@ -31,9 +31,9 @@ def test_pages_are_mapped_lazily_vector_of_the_reference():
     # src/kvcache.rs:216-227: 4 pages, 1 sequence, 3 pages per sequence
     p = PagePool(num_pages=4, page_size=32, num_slots=1, max_pages_per_slot=3)
     p.reserve(0, 0, 1)
-    assert p.tables[0] == [0, -1, -1]
+    assert p.tables[0].tolist() == [0, -1, -1]
     p.reserve(0, 0, 33)
-    assert p.tables[0] == [0, 1, -1] and p.free_count == 2
+    assert p.tables[0].tolist() == [0, 1, -1] and p.free_count == 2
     with pytest.raises(CacheError, match="per sequence"):
         p.reserve(0, 0, 97)
     p.release(0)
@@ -90,7 +90,7 @@ def test_groups_with_different_needs_have_storage_of_their_own():
     # all keys: 4 pages held; window of 40 at length 100: the next query (position 100) sees 61..100,
     # so the page of positions 0..31 went back
     assert c.free_pages() == [4, 5, 4]
-    assert c.groups[1].pool.tables[s][:4] == [-1, 1, 2, 3]
+    assert c.groups[1].pool.tables[s][:4].tolist() == [-1, 1, 2, 3]
     c.release(s)
     assert c.free_pages() == [8, 8, 8]
     c.check_consistent()

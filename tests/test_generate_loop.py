@@ -138,7 +138,7 @@ def test_temperature_sampling_is_per_sequence_and_seeded():
 
 def test_plan_step_layout():
     entries = [StepEntry(3, [5, 6, 7], [0, 2]), StepEntry(0, [9], "last"), StepEntry(1, [1, 2], "none")]
-    tokens, seq, pos, cu, want = plan_step(entries, [10, 0, 4], VOCAB)
+    tokens, seq, pos, cu, want = (a.tolist() for a in plan_step(entries, [10, 0, 4], VOCAB))
     assert tokens == [5, 6, 7, 9, 1, 2] and seq == [0, 0, 0, 1, 2, 2] and pos == [10, 11, 12, 0, 4, 5]
     assert cu == [0, 3, 4, 6] and want == [0, 2, 3]
     assert wanted_indices(4, "all") == [0, 1, 2, 3]
@@ -148,6 +148,8 @@ def test_plan_step_layout():
         plan_step([StepEntry(0, [1], [1])], [0], VOCAB)
     with pytest.raises(ShapeError, match="no token"):
         plan_step([StepEntry(0, [])], [0], VOCAB)
+    one_each = plan_step([StepEntry(2, [5]), StepEntry(0, [6])], [7, 3], VOCAB)      # the decode step's short cut
+    assert [a.tolist() for a in one_each] == [[5, 6], [0, 1], [7, 3], [0, 1, 2], [0, 1]]
 
 
 # ------------------------------------------------------------------------------------------------ the command line
