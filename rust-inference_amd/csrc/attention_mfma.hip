@@ -341,7 +341,7 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     __shared__ float ml_lds[DECODE_WAVES][2][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int chunk = blockIdx.x, b = blockIdx.y, kvh = blockIdx.z;
+    const int b = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;      // chunks last: the empty ones start last
     const int group = heads / kv_heads;
     const int tok = b;                                       // one new token per sequence: token b is sequence b's
     const int qpos = tok_pos[tok];
@@ -474,7 +474,7 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
     __shared__ __attribute__((aligned(16))) bf16_t vnew[DH];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int chunk = blockIdx.x, b = blockIdx.y, kvh = blockIdx.z;
+    const int b = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;      // chunks last: the empty ones start last
     const int group = heads / kv_heads;
     const int qpos = tok_pos[b];                             // token b is sequence b's one new token
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
@@ -635,9 +635,9 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
     if (check_common("attention_decode_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
     const int group = heads / kv_heads;
     RI_REQUIRE(group <= 16, "attention_decode_bf16: %d query heads per kv head (at most 16)", group);
-    RI_REQUIRE(seqs > 0 && seqs <= 65535 && max_chunks > 0 && heads <= 65535,
+    RI_REQUIRE(seqs > 0 && max_chunks > 0 && max_chunks <= 65535 && heads <= 65535,
                "attention_decode_bf16: seqs %d, chunks %d, heads %d", seqs, max_chunks, heads);
-    dim3 grid(max_chunks, seqs, kv_heads);
+    dim3 grid(seqs, kv_heads, max_chunks);
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
 #define RI_DECODE_CASE(DH)                                                                                        \
@@ -670,11 +670,11 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
         return 1;
     const int group = heads / kv_heads;
     RI_REQUIRE(group <= 16, "attention_decode_fused_bf16: %d query heads per kv head (at most 16)", group);
-    RI_REQUIRE(seqs > 0 && seqs <= 65535 && max_chunks > 0 && heads <= 65535,
+    RI_REQUIRE(seqs > 0 && max_chunks > 0 && max_chunks <= 65535 && heads <= 65535,
                "attention_decode_fused_bf16: seqs %d, chunks %d, heads %d", seqs, max_chunks, heads);
     RI_REQUIRE(q_stride >= (heads + 2 * kv_heads) * head_dim, "attention_decode_fused_bf16: qkv row stride %d",
                q_stride);
-    dim3 grid(max_chunks, seqs, kv_heads);
+    dim3 grid(seqs, kv_heads, max_chunks);
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
 #define RI_FUSED_CASE(DH)                                                                                         \
