@@ -215,3 +215,32 @@ def test_trace_run_program(model_dirs, tmp_path, dtype_name):
     got = plans.collect(steps, lambda i: np.fromfile(os.path.join(out_dir, f"{i}.f32"), dtype="<f4"), vocab)
     check_against_plain(model_dirs["B"], got, reqs, dtype_name, "bin/trace_run")
     assert not os.path.exists(os.path.join(out_dir, f"{len(steps)}.f32"))
+
+
+# ---------------------------------------------------------------- sizes drawn at random
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Every size a configuration may have, drawn from lists that mix what the fast kernels take (head
+    sizes 32, 64, 128, widths that are multiples of 8) with what only the general ones do (head sizes 48,
+    80, 160, 256, odd widths, seven query heads a group): whole, last 32 one by one and an unequal
+    batch, in both dtypes, against the plain implementation."""
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    rng = np.random.default_rng(1000 + seed)
+    kv, group = int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 2, 3, 4, 7, 8, 16]))
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": int(rng.integers(50, 700)),
+           "hidden_size": int(rng.choice([33, 50, 72, 75, 104, 129, 136, 264])),
+           "intermediate_size": int(rng.choice([9, 37, 88, 101, 232, 250])),
+           "num_hidden_layers": int(rng.integers(1, 4)), "num_attention_heads": kv * group, "num_key_value_heads": kv,
+           "head_dim": int(rng.choice([16, 32, 48, 64, 80, 128, 160, 256])),
+           "rope_theta": float(rng.choice([1e4, 5e4, 1e6])), "rms_norm_eps": float(rng.choice([1e-6, 1e-5, 3e-6])),
+           "tie_word_embeddings": bool(rng.integers(0, 2)), "max_position_embeddings": 512}
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=seed, dtype=torch.bfloat16, matrix_std=0.12, gain_std=0.1)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for i, n in enumerate(rng.integers(1, 200, 3))}
+    for dtype_name in ("float32", "bfloat16"):
+        model = load_model(folder, DTYPES[dtype_name])
+        for what, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 32)),
+                            ("batch", plans.unequal_batches([{k: (v, max(1, len(v) - 7)) for k, v in reqs.items()}]))):
+            got = replay_in_process(model, steps)
+            check_against_plain(folder, got, reqs, dtype_name, f"{cfg}, {what}")
