@@ -19,8 +19,11 @@ from ..kernels import ops
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
 #              A form of the packed kernel for up to 64 rows (every weight tile used for four tiles of x
 #              taken from the L2 cache) was tried and lost to the library from 24 rows on at every one of
-#              these matrices (q|k|v at 32 rows: 23 us against 16 us): it would need x staged through LDS
-#              and larger workgroup tiles, which is the library's own design.
+#              these matrices (q|k|v at 32 rows: 23 us against 16 us).  So did one whose workgroups own
+#              four row tiles and all tiles of x, with K cut into parts for the narrow matrices (at 64
+#              rows: down 36 us against 39 us, o 20 against 15, gate|up 80 against 52): one workgroup a
+#              compute unit, its stream and its reduction one after the other.  Beating the library here
+#              takes the library's own design: x staged through LDS, persistent workgroups.
 GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
 SPLIT_K = 4096
