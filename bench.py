@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|32b]
 
 The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
@@ -25,6 +25,16 @@ QWEN3_8B = {
 }
 
 
+# The other two shapes that the baseline names, for `--model`: the small model whose decode step is bound
+# by launches and latencies, and the large one (64 GB of weights).
+QWEN3_0_6B = dict(QWEN3_8B, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                  num_key_value_heads=8, tie_word_embeddings=True)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
+                 num_key_value_heads=8)
+MODELS = {"8b": ("Qwen3-8B shapes", QWEN3_8B), "0.6b": ("Qwen3-0.6B shapes", QWEN3_0_6B),
+          "32b": ("Qwen3-32B shapes", QWEN3_32B)}
+
+
 def layer_matrix_params(c):
     d, dh = c["hidden_size"], c["head_dim"]
     qkv = (c["num_attention_heads"] + 2 * c["num_key_value_heads"]) * dh * d
@@ -34,7 +44,8 @@ def layer_matrix_params(c):
 def decode_bytes(c, layers, batch, mean_context):
     """Bytes a decode step has to read: every weight it uses once, and the cache of the live requests."""
     d = c["hidden_size"]
-    weights = 2 * (layers * layer_matrix_params(c) + c["vocab_size"] * d + batch * d)        # bf16
+    weights = 2 * (layers * layer_matrix_params(c) + c["vocab_size"] * d + batch * d)        # bf16 (the head's matrix
+    # is read once whether it is the embedding table or its own; of the table only the batch's rows are)
     gains = 4 * (layers * (2 * d + 2 * c["head_dim"]) + d)
     kv = batch * mean_context * layers * 2 * c["num_key_value_heads"] * c["head_dim"] * 2
     return weights + gains + kv
@@ -55,6 +66,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--model", choices=sorted(MODELS), default="8b", help="which shapes (default: Qwen3-8B)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
     args = ap.parse_args()
@@ -67,7 +79,8 @@ def main() -> int:
     from rust_inference_amd.kernels import ops
     from rust_inference_amd.parts import random_model
 
-    cfg = dict(QWEN3_8B)
+    model_name, shapes = MODELS[args.model]
+    cfg = dict(shapes)
     full_layers = cfg["num_hidden_layers"]
     layers = args.layers or full_layers
     cfg["num_hidden_layers"] = layers
@@ -135,15 +148,15 @@ def main() -> int:
 
     flops = prefill_flops(cfg, layers, args.prompt)
     out = {
-        "metric": "decode tok/s at batch 8, Qwen3-8B shapes bf16 (prefill 2048 and batch 1/64 alongside)",
+        "metric": f"decode tok/s at batch {args.batch}, {model_name} bf16 (prefill {args.prompt} and batch 1/64 alongside)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(1e3 * dt / args.steps, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights (seed 2), uniform random token ids",
         "config": {
-            "model": "Qwen3-8B shapes", "layers": layers, "layers_full": full_layers, "hidden": cfg["hidden_size"],
+            "model": model_name, "layers": layers, "layers_full": full_layers, "hidden": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
             "intermediate": cfg["intermediate_size"], "vocab": vocab, "rope_theta": cfg["rope_theta"],
-            "rms_norm_eps": cfg["rms_norm_eps"], "tied": False, "global_batch": args.batch, "seq_len": args.context,
+            "rms_norm_eps": cfg["rms_norm_eps"], "tied": cfg["tie_word_embeddings"], "global_batch": args.batch, "seq_len": args.context,
             "prompt_len": args.prompt, "mean_decode_context": round(mean_context, 1), "page_size": 32,
             "parallelism": "single GPU",
         },

@@ -67,7 +67,7 @@ class GroupedQueryAttention(Mixer):
         self.rt = rt
         p = self.prefix
         qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
-        self.w_qkv = rt.place_matrix(qkv)
+        self.w_qkv = rt.pack(rt.place_matrix(qkv))
         self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]))
         self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
         self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
@@ -78,7 +78,7 @@ class GroupedQueryAttention(Mixer):
 
     def forward(self, x, ctx, store, page_table, link=None):
         rt = self.rt
-        qkv = rt.linear(x, self.w_qkv)
+        qkv = rt.linear_packed(x, self.w_qkv)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
         group = self.heads // self.kv_heads
         if (ctx.is_decode and ctx.B <= FUSED_DECODE_MAX_SEQS

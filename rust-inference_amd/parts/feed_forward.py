@@ -7,7 +7,6 @@ from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part
-from .runtime import PackedWeight
 
 
 @register_part("feed_forward", "swiglu")
@@ -34,9 +33,7 @@ class SwiGLU(FeedForward):
         p = self.prefix
         gate_up = rt.place_matrix(torch.cat([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], 0))
         self.w_gate_up = rt.pack(gate_up, swiglu=True)
-        # no packed copy of the down matrix: at 4096 x 12288 the library's product streams it faster
-        # (22 us against 27 us, also with K split into parts)
-        self.w_down = PackedWeight(rt.place_matrix(weights[p + "down_proj.weight"]), None, False)
+        self.w_down = rt.pack(rt.place_matrix(weights[p + "down_proj.weight"]))
 
     def forward(self, x, ctx, link=None):
         rt = self.rt

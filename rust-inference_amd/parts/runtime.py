@@ -27,6 +27,15 @@ from ..kernels import ops
 GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
 SPLIT_K = 4096
+# Which matrices get a packed copy for 3 to 16 rows (the gate|up matrix always does: its activation
+# rides in the kernel).  Measured at 4, 8 and 16 rows, packed kernel against library, in us:
+#   4096 x 1024 (8 MB) 4.5 : 7.5     1024 x 3072 (6 MB) 7.4 : 12.0    2048 x 2048 (8 MB) 5.9 : 11.1
+#   4096 x 4096 (34 MB) 10.8 : 15.4  6144 x 4096 (50 MB) 16.2 : 15.3  2560 x 9728 (50 MB) 19.7 : 18.3
+#   4096 x 12288 (101 MB) 27 : 22    10240 x 5120 (105 MB) 32 : 24    5120 x 8192 (84 MB) 29 : 20
+#   5120 x 25600 (262 MB) 90 : 136, and 74 with K cut into parts
+# so: the small ones, and the very long rows.
+PACKED_MAX_BYTES = 40_000_000
+PACKED_LONG_K = 16384
 
 
 class PackedWeight:
@@ -96,8 +105,11 @@ class Runtime:
         return (x.xg.float() * inv).to(x.xg.dtype)
 
     def pack(self, w: torch.Tensor, swiglu: bool = False) -> PackedWeight:
-        """A placed weight with its packed copy for decode-size products (bfloat16 compute only)."""
-        if self.dtype != torch.bfloat16 or w.shape[1] % 8:
+        """A placed weight, with a packed copy where the packed kernel is the faster one for 3 to 16
+        rows (bfloat16 compute only)."""
+        n, k = w.shape
+        pays = swiglu or n * k * 2 <= PACKED_MAX_BYTES or k >= PACKED_LONG_K
+        if self.dtype != torch.bfloat16 or k % 8 or not pays:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
 
@@ -120,16 +132,18 @@ class Runtime:
             elif m <= SKINNY_MAX_ROWS and pw.packed is not None:
                 mine = (pw.packed, True)
             if mine is not None:
-                if link is not None and not pw.swiglu and link.residual.shape == (m, pw.n):
+                in_parts = mine[1] and parts_ok and pw.parts > 1        # very long rows: parts beat the link
+                if link is not None and not pw.swiglu and not in_parts and link.residual.shape == (m, pw.n):
                     made = ops.linked_product(x, mine[0], pw.n, mine[1], residual=link.residual,
                                               next_gain=link.gain, next_eps=link.eps)
                     return (made, link.norm)
+                if in_parts:
+                    return ops.gemm_skinny_packed_bf16(self.normed_now(x), pw.packed, pw.n, torch.float32,
+                                                       parts=pw.parts)
                 if later:
                     return ops.linked_product(x, mine[0], pw.n, mine[1], out_dtype, swiglu=pw.swiglu)
                 if not mine[1]:
                     return ops.gemv_bf16(x, pw.w, out_dtype, swiglu=pw.swiglu)
-                if parts_ok and pw.parts > 1:
-                    return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=pw.parts)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
         y = self.linear(x, pw.w, None if pw.swiglu else out_dtype)
         return ops.swiglu(y) if pw.swiglu else y
