@@ -591,8 +591,19 @@ static int check_common(const char* name, int heads, int kv_heads, int head_dim,
     return 0;
 }
 
-// column tiles per wavefront: 64 columns for head_dim up to 64, 32 for 128 (registers)
-static int prefill_tiles(int head_dim) { return head_dim <= 64 ? 4 : 2; }
+// Column tiles per wavefront: at most 64 columns for head_dim up to 64, 32 for 128 (registers); fewer when
+// that leaves the launch with less than two workgroups a compute unit (few query heads per kv head, a
+// short prompt): a column's arithmetic does not depend on the tile it sits in, only the grid does.
+static int prefill_tiles(int head_dim, int group, int max_new, int seqs, int kv_heads) {
+    int nt = head_dim <= 64 ? 4 : 2;
+    while (nt > 1 && group <= 16 * (nt / 2)) {
+        const int tile_tokens = (16 * nt) / group;
+        const long wgs = (long)((max_new + 4 * tile_tokens - 1) / (4 * tile_tokens)) * seqs * kv_heads;
+        if (wgs >= 512) break;
+        nt /= 2;
+    }
+    return nt;
+}
 
 extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const void* k_pages,
                                          const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
@@ -601,24 +612,29 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
                                          float scale, void* stream) {
     if (check_common("attention_prefill_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
     const int group = heads / kv_heads;
-    const int nt_tiles = prefill_tiles(head_dim);
+    RI_REQUIRE(seqs > 0 && seqs <= 65535 && max_new > 0, "attention_prefill_bf16: seqs %d, max_new %d", seqs, max_new);
+    const int nt_tiles = prefill_tiles(head_dim, group, max_new, seqs, kv_heads);
     RI_REQUIRE(group <= 16 * nt_tiles, "attention_prefill_bf16: %d query heads per kv head (at most %d)", group,
                16 * nt_tiles);
-    RI_REQUIRE(seqs > 0 && seqs <= 65535 && max_new > 0, "attention_prefill_bf16: seqs %d, max_new %d", seqs, max_new);
     const int tile_tokens = (16 * nt_tiles) / group;
     dim3 grid((max_new + 4 * tile_tokens - 1) / (4 * tile_tokens), seqs, kv_heads);
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
 #define RI_PREFILL_CASE(DH, NT)                                                                                  \
-    case DH:                                                                                                     \
+    case DH * 8 + NT:                                                                                            \
         attn_prefill_mfma_kernel<DH, NT><<<grid, 256, 0, s>>>(                                                   \
             (bf16_t*)out, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,          \
             cu_seqlens, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2);                  \
         break;
-    switch (head_dim) {
+    switch (head_dim * 8 + nt_tiles) {
         RI_PREFILL_CASE(32, 4)
+        RI_PREFILL_CASE(32, 2)
+        RI_PREFILL_CASE(32, 1)
         RI_PREFILL_CASE(64, 4)
+        RI_PREFILL_CASE(64, 2)
+        RI_PREFILL_CASE(64, 1)
         RI_PREFILL_CASE(128, 2)
+        RI_PREFILL_CASE(128, 1)
     }
 #undef RI_PREFILL_CASE
     RI_LAUNCH_CHECK("attention_prefill_bf16");
