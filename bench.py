@@ -66,6 +66,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--prompt-range", type=int, nargs=2, metavar=("LOW", "HIGH"), default=None,
+                    help="decode after prompts of unequal lengths drawn uniformly from LOW..HIGH instead of --prompt")
     ap.add_argument("--model", choices=sorted(MODELS), default="8b", help="which shapes (default: Qwen3-8B)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-graphs", action="store_true", help="launch every kernel of a decode step from the host")
@@ -91,6 +93,10 @@ def main() -> int:
     gen = torch.Generator().manual_seed(2)
 
     def prompts(batch, n):
+        if args.prompt_range and batch > 1:                       # unequal lengths, prefilled together
+            low, high = args.prompt_range
+            lens = torch.randint(low, high + 1, (batch,), generator=gen).tolist()
+            return [torch.randint(0, vocab, (m,), generator=gen).tolist() for m in lens]
         return torch.randint(0, vocab, (batch, n), generator=gen).tolist()
 
     def fresh_engine(batch):
@@ -125,7 +131,7 @@ def main() -> int:
         for _ in range(warmup):
             nxt = ops.argmax(engine.step([StepEntry(s, [t], "last") for s, t in zip(slots, nxt)])).tolist()
         sync()
-        first_context = engine.cache.length(slots[0]) + 1
+        first_context = sum(engine.cache.length(s) for s in slots) / batch + 1
         t0 = time.perf_counter()
         for _ in range(steps):
             nxt = ops.argmax(engine.step([StepEntry(s, [t], "last") for s, t in zip(slots, nxt)])).tolist()
@@ -157,7 +163,7 @@ def main() -> int:
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
             "intermediate": cfg["intermediate_size"], "vocab": vocab, "rope_theta": cfg["rope_theta"],
             "rms_norm_eps": cfg["rms_norm_eps"], "tied": cfg["tie_word_embeddings"], "global_batch": args.batch, "seq_len": args.context,
-            "prompt_len": args.prompt, "mean_decode_context": round(mean_context, 1), "page_size": 32,
+            "prompt_len": "{}..{}".format(*args.prompt_range) if args.prompt_range else args.prompt, "mean_decode_context": round(mean_context, 1), "page_size": 32,
             "parallelism": "single GPU",
         },
         "prefill": {"value": round(args.prompt / prefill_s, 1), "tokens": args.prompt, "ms": round(1e3 * prefill_s, 2),
