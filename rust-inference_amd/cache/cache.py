@@ -17,11 +17,13 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..errors import CacheError
+from . import native
 from .pages import PagePool, UNMAPPED
-from .slots import SlotAllocator
+from .slots import SlotAllocator, _Core
 
 PAGE_SIZE = 32   # tokens per page, as in the reference (src/kvcache.rs:12)
 
@@ -90,8 +92,6 @@ class Cache:
         self.page_size, self.num_slots = page_size, num_slots
         self.max_seq_len = max_seq_len
         self.device, self.dtype = device, dtype
-        self.slots = SlotAllocator(num_slots)
-        self.lengths = [0] * num_slots
         self.max_pages_per_slot = -(-max_seq_len // page_size)
         num_pages = -(-max_tokens // page_size)
         self.needs = list(needs)
@@ -111,53 +111,38 @@ class Cache:
             for e in entries:
                 self._kv_of_entry[e] = (len(self.groups), g.index_of[e])
             self.groups.append(g)
+        # slots, lengths and the groups' pools together: native bookkeeping (csrc/host_cache.hip)
+        self.core = _Core([g.pool for g in self.groups], num_slots, max_seq_len)
+        self.slots = SlotAllocator(num_slots, self.core)
+        self._lib = native.lib()
 
     # ---- slots
     def acquire(self) -> int:
-        slot = self.slots.acquire()
-        self.lengths[slot] = 0
+        slot = self.slots.acquire()                 # comes back with length 0
         for arena in self._state.values():
             arena[slot].zero_()
         return slot
 
     def release(self, slot: int) -> None:
-        self.slots.release(slot)
-        for g in self.groups:
-            g.pool.release(slot)
-        self.lengths[slot] = 0
+        self.slots.release(slot)                    # its pages go back to every pool, its length to 0
 
     def length(self, slot: int) -> int:
-        self.slots.check_held(slot)
-        return self.lengths[slot]
+        n = self._lib.ri_cache_length(self.core.handle, int(slot))
+        if n < 0:
+            raise native.fail()
+        return n
 
     # ---- steps
     def reserve(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         """Map pages for the tokens a step is about to write.  Either every sequence
         gets its pages or the cache is left as it was."""
-        if len(set(slots)) != len(slots):
-            raise CacheError("a slot appears twice in one step")
-        for s, n in zip(slots, new_tokens):
-            self.slots.check_held(s)
-            if n < 1:
-                raise CacheError(f"slot {s}: a step needs at least one token")
-            if self.lengths[s] + n > self.max_seq_len:
-                raise CacheError(f"slot {s} would reach {self.lengths[s] + n} tokens, "
-                                 f"the cache holds {self.max_seq_len} per sequence")
-        for g in self.groups:
-            want = sum(g.pool.pages_needed(s, self.lengths[s], n) for s, n in zip(slots, new_tokens))
-            if want > g.pool.free_count:
-                raise CacheError(f"cache out of pages: the step needs {want} more, {g.pool.free_count} of "
-                                 f"{g.pool.num_pages} are free ({g.page_size} tokens each)")
-        for g in self.groups:
-            for s, n in zip(slots, new_tokens):
-                g.pool.reserve(s, self.lengths[s], n)
+        s, n = np.asarray(slots, dtype=np.int32), np.asarray(new_tokens, dtype=np.int32)
+        native.check(self._lib.ri_cache_reserve(self.core.handle, s.ctypes.data, n.ctypes.data, len(s)))
 
     def commit(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         """The step has written its tokens: advance the lengths, drop what fell out of a window."""
-        for s, n in zip(slots, new_tokens):
-            self.lengths[s] += n
-            for g in self.groups:
-                g.pool.trim_behind_window(s, self.lengths[s])
+        s, n = np.asarray(slots, dtype=np.int32), np.asarray(new_tokens, dtype=np.int32)
+        native.check(self._lib.ri_cache_commit(self.core.handle, s.ctypes.data, n.ctypes.data, len(s)))
 
     # ---- views for mixers
     def kv(self, entry: int) -> KVView:
@@ -184,14 +169,8 @@ class Cache:
         return [g.pool.free_count for g in self.groups]
 
     def check_consistent(self) -> None:
-        for g in self.groups:
-            g.pool.check_consistent()
-            for s in range(self.num_slots):
-                if not self.slots.is_held(s) and g.pool.pages_of(s):
-                    raise CacheError(f"slot {s} is free but still holds pages")
-        held = len(self.slots.held_slots())
-        if held + self.slots.free_count != self.num_slots:
-            raise CacheError("a slot is lost")
+        """No slot lost or held twice; no page lost, held twice or held by a free slot."""
+        native.check(self._lib.ri_cache_check(self.core.handle))
 
 
 __all__ = ["Cache", "KVNeed", "StateNeed", "KVGroup", "KVView", "PAGE_SIZE", "UNMAPPED"]

@@ -2,45 +2,59 @@
 
 A slot is the sequence's handle into every store of the cache (its row of each
 page table, its row of each state arena).  It is acquired when the sequence
-starts and released when it ends; a released slot is handed out again.
+starts and released when it ends; a released slot is handed out again, lowest
+number first.  The bookkeeping is native (csrc/host_cache.hip); a ``SlotAllocator``
+made by itself has a core of its own, the cache's shares the cache's.
 """
 from __future__ import annotations
 
 from ..errors import CacheError
+from . import native
+
+
+class _Core:
+    """Owner of a native cache core (slots, lengths, and the pools it was given)."""
+
+    def __init__(self, pools, num_slots: int, max_seq_len: int):
+        if num_slots < 1:
+            raise CacheError("a cache needs at least one slot")
+        lib = native.lib()
+        handles = (native.c_void_p * max(1, len(pools)))(*[p.handle for p in pools])
+        self.pools = list(pools)                       # the core points into them: keep them alive
+        self.handle = lib.ri_cache_new(handles, len(pools), num_slots, max_seq_len)
+        if not self.handle:
+            raise native.fail()
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            native.lib().ri_cache_delete(self.handle)
+            self.handle = None
 
 
 class SlotAllocator:
-    def __init__(self, num_slots: int):
-        if num_slots < 1:
-            raise CacheError("a cache needs at least one slot")
+    def __init__(self, num_slots: int, core: _Core | None = None):
         self.num_slots = num_slots
-        self._free = list(range(num_slots - 1, -1, -1))   # popped from the back: slot 0 first
-        self._held = [False] * num_slots
+        self._core = core or _Core([], num_slots, 1)
+        self._lib = native.lib()
 
     def acquire(self) -> int:
-        if not self._free:
-            raise CacheError(f"no free slot: all {self.num_slots} are held by live sequences")
-        slot = self._free.pop()
-        self._held[slot] = True
+        slot = self._lib.ri_cache_acquire(self._core.handle)
+        if slot < 0:
+            raise native.fail()
         return slot
 
     def release(self, slot: int) -> None:
-        self.check_held(slot)
-        self._held[slot] = False
-        self._free.append(slot)
+        native.check(self._lib.ri_cache_release(self._core.handle, int(slot)))
 
     def check_held(self, slot: int) -> None:
-        if not (0 <= slot < self.num_slots):
-            raise CacheError(f"slot {slot} does not exist (the cache has {self.num_slots})")
-        if not self._held[slot]:
-            raise CacheError(f"slot {slot} is not held (never acquired, or released already)")
+        native.check(self._lib.ri_cache_check_held(self._core.handle, int(slot)))
 
     def is_held(self, slot: int) -> bool:
-        return 0 <= slot < self.num_slots and self._held[slot]
+        return bool(self._lib.ri_cache_is_held(self._core.handle, int(slot)))
 
     @property
     def free_count(self) -> int:
-        return len(self._free)
+        return self._lib.ri_cache_free_slots(self._core.handle)
 
     def held_slots(self) -> list[int]:
-        return [s for s in range(self.num_slots) if self._held[s]]
+        return [s for s in range(self.num_slots) if self.is_held(s)]

@@ -141,6 +141,39 @@ int ri_sample_split(int32_t* out, const float* logits, const uint8_t* seen, cons
 
 int ri_mark_seen(uint8_t* seen, const int32_t* rows, const int32_t* tokens, int n, int vocab, void* stream);
 
+// ---- the host side of the cache (no device call; handles are opaque; int results: 0, or 1 with the error
+// text set, unless said otherwise)
+// A pool of pages and every slot's table of them [num_slots][max_pages_per_slot] (-1: unmapped), pages handed
+// out lowest number first.  window 0: every key stays; else pages behind the window go back at ri_pool_trim.
+void* ri_pool_new(int num_pages, int page_size, int num_slots, int max_pages_per_slot, int window);   // NULL: error
+void ri_pool_delete(void* pool);
+int32_t* ri_pool_tables(void* pool);
+int ri_pool_free_count(void* pool);
+int ri_pool_pages_needed(void* pool, int slot, long length_before, long new_tokens);                  // the count
+int ri_pool_reserve(void* pool, int slot, long length_before, long new_tokens);
+int ri_pool_trim(void* pool, int slot, long length);
+int ri_pool_release(void* pool, int slot);
+int ri_pool_check(void* pool);
+// Slots, every slot's length, and the pools (not owned) that the slots hold pages in.
+void* ri_cache_new(void* const* pools, int num_pools, int num_slots, int max_seq_len);                // NULL: error
+void ri_cache_delete(void* cache);
+int ri_cache_acquire(void* cache);                                       // the slot, or -1
+int ri_cache_release(void* cache, int slot);
+int ri_cache_is_held(void* cache, int slot);                             // 0 or 1
+int ri_cache_check_held(void* cache, int slot);
+int ri_cache_free_slots(void* cache);                                    // the count
+long ri_cache_length(void* cache, int slot);                             // the length, or -1
+int ri_cache_reserve(void* cache, const int32_t* slots, const int32_t* counts, int n);     // all or nothing
+int ri_cache_commit(void* cache, const int32_t* slots, const int32_t* counts, int n);
+int ri_cache_check(void* cache);
+// A step's layout as one block of int32 words, every piece on a 16-byte boundary: tokens, each token's
+// sequence and position, sequence starts (n + 1), slots, lengths after the step, wanted rows, one page
+// table [n][width] per pool; offsets[7 + pools] says where each piece begins.  Returns the words used, -1 on
+// error.  Between ri_cache_reserve and ri_cache_commit of the same step.
+long ri_cache_plan_step(void* cache, const int32_t* slots, const int32_t* counts, int n, const int32_t* tokens,
+                        const int32_t* want_rows, int n_want, int vocab, int width, int32_t* words, long capacity,
+                        int64_t* offsets);
+
 #ifdef __cplusplus
 }
 #endif

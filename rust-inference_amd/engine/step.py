@@ -18,6 +18,7 @@ import itertools
 import numpy as np
 import torch
 
+from ..cache import native as cache_native
 from ..errors import ShapeError
 from ..parts.context import StepContext
 
@@ -139,43 +140,56 @@ class Engine:
 
     def build_context(self, entries: Sequence[StepEntry], staging: _Staging | None = None,
                       full_width: bool = False) -> StepContext:
+        """Reserve the step's pages and send its layout to the device: one block of int32 words
+        (tokens, sequence and position of each, sequence starts, slots, lengths after the step,
+        wanted rows, a page table per key/value group), laid out by the cache's native side
+        straight into a pinned buffer."""
         cache = self.cache
+        B = len(entries)
+        if B == 0:
+            raise ShapeError("a step needs at least one entry")
         slots = [e.slot for e in entries]
-        starts = [cache.length(s) for s in slots]
         counts = [len(e.tokens) for e in entries]
-        tokens, tok_seq, tok_pos, cu, want_rows = plan_step(entries, starts, self.model.spec.vocab_size)
+        for b, (e, n) in enumerate(zip(entries, counts)):
+            if n < 1:
+                raise ShapeError(f"entry {b} (slot {e.slot}) brings no token")
+        T = sum(counts)
+        starts = [cache.length(s) for s in slots]
+        cu, want = [0], []
+        for e, n in zip(entries, counts):
+            want.extend(cu[-1] + i for i in wanted_indices(n, e.want))
+            cu.append(cu[-1] + n)
+        tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int64, count=T)
+        if T and (tokens.min() < 0 or tokens.max() >= self.model.spec.vocab_size):
+            bad = int(tokens[(tokens < 0) | (tokens >= self.model.spec.vocab_size)][0])
+            raise ShapeError(f"token id {bad} is outside the vocabulary of {self.model.spec.vocab_size}")
+        tokens = tokens.astype(np.int32)
         cache.reserve(slots, counts)
-        len_after = [s + n for s, n in zip(starts, counts)]
-        max_len = max(len_after)
+        max_len = max(s + n for s, n in zip(starts, counts))
         width = cache.max_pages_per_slot if full_width else -(-max_len // cache.page_size)
-        T, B = len(tokens), len(entries)
-        # one block of int32 words for everything the kernels read of the layout, every piece on a
-        # 16-byte boundary: tokens, sequence and position of each, sequence starts, slots, lengths
-        # after the step, wanted rows, then a page table per key/value group
-        pieces = [tokens, tok_seq, tok_pos, cu, slots, len_after, want_rows]
-        sizes = [len(p) for p in pieces] + [B * width] * len(cache.groups)
-        offsets, at = [], 0
-        for n in sizes:
-            offsets.append(at)
-            at += -(-n // 4) * 4
-        stage = staging or self._stage(at)
-        words = stage.begin(at)
-        for p, off in zip(pieces, offsets):
-            words[off:off + len(p)] = p
-        for gi, g in enumerate(cache.groups):
-            off = offsets[len(pieces) + gi]
-            words[off:off + B * width].reshape(B, width)[:] = g.table_rows(slots, width)
-        dev = stage.upload(at)
+        G = len(cache.groups)
+        capacity = 3 * (T + 4) + (B + 5) + 2 * (B + 4) + (len(want) + 4) + G * (B * width + 4)
+        stage = staging or self._stage(capacity)
+        words = stage.begin(capacity)
+        offsets = np.empty(7 + G, dtype=np.int64)
+        s_arr, c_arr, w_arr = (np.asarray(a, dtype=np.int32) for a in (slots, counts, want))
+        used = cache_native.lib().ri_cache_plan_step(
+            cache.core.handle, s_arr.ctypes.data, c_arr.ctypes.data, B, tokens.ctypes.data, w_arr.ctypes.data, len(want),
+            self.model.spec.vocab_size, width, words.ctypes.data, capacity, offsets.ctypes.data)
+        if used < 0:
+            raise ShapeError(cache_native.lib().ri_last_error().decode())
+        dev = stage.upload(used)
+        off = offsets.tolist()
 
         def piece(i, n):
-            return dev[offsets[i]:offsets[i] + n]
+            return dev[off[i]:off[i] + n]
 
         ctx = StepContext(T=T, B=B, new_counts=counts, slot_list=slots, starts=starts,
                           tokens=piece(0, T), tok_seq=piece(1, T), tok_pos=piece(2, T), cu_seqlens=piece(3, B + 1),
-                          slots=piece(4, B), len_after=piece(5, B), want_rows=piece(6, len(want_rows)),
-                          n_want=len(want_rows), max_new=max(counts),
+                          slots=piece(4, B), len_after=piece(5, B), want_rows=piece(6, len(want)),
+                          n_want=len(want), max_new=max(counts),
                           max_len=cache.max_seq_len if full_width else max_len)
-        ctx.page_tables = [piece(7 + gi, B * width).view(B, width) for gi in range(len(cache.groups))]
+        ctx.page_tables = [piece(7 + gi, B * width).view(B, width) for gi in range(G)]
         return ctx
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -196,7 +210,7 @@ class Engine:
         if dg is None:
             dg = self._graphs[batch] = _DecodeGraph(batch, self.device)
             width = self.cache.max_pages_per_slot
-            need = 7 * (batch + 4) + len(self.cache.groups) * (batch * width + 4)
+            need = 7 * (batch + 5) + len(self.cache.groups) * (batch * width + 4)
             dg.staging = _Staging(need, self.device)
         # the layout of a decode step depends on the batch size alone, so the buffers a captured
         # graph reads are refilled in place

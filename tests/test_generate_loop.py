@@ -152,6 +152,38 @@ def test_plan_step_layout():
     assert [a.tolist() for a in one_each] == [[5, 6], [0, 1], [7, 3], [0, 1, 2], [0, 1]]
 
 
+def test_native_step_layout_is_the_plain_one():
+    """The cache's native side lays a step out into one block of words; piece by piece it is what
+    plan_step says, with the page tables of the step's slots behind."""
+    import numpy as np
+    from rust_inference_amd.cache import native
+    cache = Cache([KVNeed(1, 16), KVNeed(2, 16, 40)], 4, 1024, 256, dtype=torch.float32, device="cpu", allocate=False)
+    slots = [cache.acquire() for _ in range(3)]
+    cache.reserve(slots[:2], [70, 5]); cache.commit(slots[:2], [70, 5])
+    entries = [StepEntry(slots[2], [5, 6, 7], [0, 2]), StepEntry(slots[0], [9], "last"), StepEntry(slots[1], [1, 2], "none")]
+    order, counts = [e.slot for e in entries], [len(e.tokens) for e in entries]
+    want_plain = plan_step(entries, [cache.length(s) for s in order], VOCAB)
+    cache.reserve(order, counts)
+    width, words, offsets = 3, np.zeros(400, dtype=np.int32), np.zeros(7 + len(cache.groups), dtype=np.int64)
+    arr = lambda a: np.asarray(a, dtype=np.int32)
+    s_arr, c_arr, t_arr, w_arr = arr(order), arr(counts), want_plain[0], want_plain[4]
+    used = native.lib().ri_cache_plan_step(cache.core.handle, s_arr.ctypes.data, c_arr.ctypes.data, 3, t_arr.ctypes.data,
+                                           w_arr.ctypes.data, len(w_arr), VOCAB, width, words.ctypes.data, len(words),
+                                           offsets.ctypes.data)
+    assert used > 0 and all(o % 4 == 0 for o in offsets.tolist())
+    sizes = [6, 6, 6, 4, 3, 3, len(w_arr)]
+    got = [words[o:o + n].tolist() for o, n in zip(offsets.tolist(), sizes)]
+    assert got[:4] == [a.tolist() for a in want_plain[:4]] and got[6] == w_arr.tolist()
+    assert got[4] == order and got[5] == [3, 71, 7]
+    for gi, g in enumerate(cache.groups):
+        table = words[offsets[7 + gi]:offsets[7 + gi] + 3 * width].reshape(3, width)
+        assert table.tolist() == g.pool.gather(order, width).tolist()
+    assert native.lib().ri_cache_plan_step(cache.core.handle, s_arr.ctypes.data, c_arr.ctypes.data, 3, t_arr.ctypes.data,
+                                           w_arr.ctypes.data, len(w_arr), 7, width, words.ctypes.data, len(words),
+                                           offsets.ctypes.data) == -1            # token 9 in a vocabulary of 7
+    assert "outside the vocabulary" in native.lib().ri_last_error().decode()
+
+
 # ------------------------------------------------------------------------------------------------ the command line
 def test_runner_options_are_the_references():
     """Names, short forms and defaults of src/bin/runner.rs:24-123 for the options this build has."""
