@@ -18,7 +18,7 @@ class _Core:
     def __init__(self, pools, num_slots: int, max_seq_len: int):
         if num_slots < 1:
             raise CacheError("a cache needs at least one slot")
-        lib = native.lib()
+        lib = self._lib = native.lib()
         handles = (native.c_void_p * max(1, len(pools)))(*[p.handle for p in pools])
         self.pools = list(pools)                       # the core points into them: keep them alive
         self.handle = lib.ri_cache_new(handles, len(pools), num_slots, max_seq_len)
@@ -27,7 +27,7 @@ class _Core:
 
     def __del__(self):
         if getattr(self, "handle", None):
-            native.lib().ri_cache_delete(self.handle)
+            self._lib.ri_cache_delete(self.handle)
             self.handle = None
 
 
