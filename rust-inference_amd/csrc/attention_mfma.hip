@@ -222,12 +222,14 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][DH * LdsPage<DH>::VS];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int b = blockIdx.y, kvh = blockIdx.z;
+    // The kv head is the fastest grid index: consecutive workgroups go to consecutive XCDs, so the
+    // workgroups that walk the same keys and values (one kv head of one sequence) meet in one XCD's L2.
+    const int kvh = blockIdx.x, b = blockIdx.z;
     const int group = heads / kv_heads;
     const int tile_tokens = (16 * NT) / group;               // tokens per wavefront
     const int t_end = cu_seqlens[b + 1];
     // the last tokens of a sequence see the most keys: their workgroups are launched first
-    const int t_wg = cu_seqlens[b] + (int)(gridDim.x - 1 - blockIdx.x) * 4 * tile_tokens;
+    const int t_wg = cu_seqlens[b] + (int)(gridDim.y - 1 - blockIdx.y) * 4 * tile_tokens;
     if (t_wg >= t_end) return;                               // the whole workgroup leaves
     const int t0 = t_wg + wave * tile_tokens;
     const int nt = max(0, min(tile_tokens, t_end - t0));     // a wavefront without tokens still helps to fetch
@@ -617,7 +619,9 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
     RI_REQUIRE(group <= 16 * nt_tiles, "attention_prefill_bf16: %d query heads per kv head (at most %d)", group,
                16 * nt_tiles);
     const int tile_tokens = (16 * nt_tiles) / group;
-    dim3 grid((max_new + 4 * tile_tokens - 1) / (4 * tile_tokens), seqs, kv_heads);
+    const int tiles = (max_new + 4 * tile_tokens - 1) / (4 * tile_tokens);
+    RI_REQUIRE(tiles <= 65535, "attention_prefill_bf16: %d tiles of tokens exceed one launch", tiles);
+    dim3 grid(kv_heads, tiles, seqs);
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
 #define RI_PREFILL_CASE(DH, NT)                                                                                  \
