@@ -17,8 +17,9 @@
 // The mask is positional: the query at position p sees keys lo..p, lo = 0 or p - window + 1
 // (the reference: src/attention.rs:73, :117-118).  Scores are scaled after the dot product
 // (src/attention.rs:28, :121-127); statistics and accumulators are float32; the weights enter the
-// second product rounded to bfloat16 and the running sum is taken of the rounded weights, so they
-// still sum to one.
+// second product rounded to bfloat16, the running sum is taken of them before the rounding.  (Letting
+// the reference point of the exponents lag behind the running maximum, so that the accumulators are
+// rescaled only rarely, was tried and changed no timing: the rescaling is not what the kernel waits for.)
 //
 // Prefill: one wavefront per tile of tokens, walking the sequence's pages in order; the four
 // wavefronts of a workgroup share the pages through LDS.  Decode (one new
