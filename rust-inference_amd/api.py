@@ -34,7 +34,6 @@ class Model:
                  use_graphs: bool = True):
         self.decoder = decoder
         self.config = getattr(decoder, "config", None)
-        max_seq_len = min(max_seq_len, decoder.spec.max_positions)
         page = 32
         per_seq = -(-max_seq_len // page) * page
         self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)

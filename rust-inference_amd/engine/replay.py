@@ -53,7 +53,7 @@ def engine_for_trace(model, max_tokens: int) -> Engine:
     page = 32
     max_tokens = max(max_tokens, page)
     cache = model.new_cache(max_tokens=max_tokens, num_slots=max(1, -(-max_tokens // 64)),
-                            max_seq_len=min(max_tokens, model.spec.max_positions))
+                            max_seq_len=max_tokens)
     return Engine(model, cache)
 
 

@@ -121,7 +121,9 @@ class DecoderModel:
         return needs
 
     def new_cache(self, max_tokens: int, num_slots: int, max_seq_len: int | None = None, **kw) -> Cache:
-        max_seq_len = min(max_seq_len or self.spec.max_positions, self.spec.max_positions)
+        # the configuration's max_position_embeddings is the default length only: nothing in this
+        # architecture depends on it (the reference reads it and never uses it, src/models/config.rs:30)
+        max_seq_len = max_seq_len or self.spec.max_positions
         return Cache(self.cache_needs(), num_slots, max_tokens, max_seq_len, dtype=self.rt.dtype,
                      device=self.rt.device, **kw)
 

@@ -244,3 +244,13 @@ def test_configurations_drawn_at_random(tmp_path, seed):
                             ("batch", plans.unequal_batches([{k: (v, max(1, len(v) - 7)) for k, v in reqs.items()}]))):
             got = replay_in_process(model, steps)
             check_against_plain(folder, got, reqs, dtype_name, f"{cfg}, {what}")
+
+
+def test_a_sequence_may_pass_max_position_embeddings(model_dirs, loaded):
+    """The key is read and, as in the reference, bounds nothing (src/models/config.rs:30): configuration A
+    says 128 positions, the request has 150 tokens, the last 20 decoded one by one."""
+    cfg, _ = read_model_f64(model_dirs["A"])
+    assert cfg["max_position_embeddings"] == 128
+    reqs = requests_for("A", cfg, [150], 99)
+    got = replay_in_process(loaded("A", "float32"), plans.tail_one_by_one(reqs, 20))
+    check_against_plain(model_dirs["A"], got, reqs, "float32", "past max_position_embeddings")
