@@ -2,8 +2,7 @@
 its binding.  Nothing here touches the GPU, so the library loads and works on a machine without one."""
 from __future__ import annotations
 
-import ctypes
-from ctypes import POINTER, c_int, c_int32, c_int64, c_long, c_void_p
+from ctypes import POINTER, c_int, c_int32, c_long, c_void_p
 
 from ..errors import CacheError
 

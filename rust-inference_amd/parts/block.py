@@ -1,7 +1,8 @@
 """Arrangements: how a layer wires its norms, mixer and feed-forward around the residual stream."""
 from __future__ import annotations
 
-from ..kernels.ops import NormedLater
+import torch
+
 from .registry import build_part, register_part
 
 # A decode step of at most this many tokens leaves its norms to the products around them (the
@@ -33,7 +34,6 @@ class ResidualStream:
     def link(self, norm, act_dtype):
         """A ``NormLink`` for the branch that is about to run, if ``norm`` is the next reader of the
         stream and can be left to a product."""
-        import torch
         if (norm is None or not getattr(norm, "linkable", False) or self.pending is not None or self.later is not None
                 or act_dtype != torch.bfloat16 or self.sum.shape[0] > LINK_MAX_TOKENS
                 or norm.dim != self.sum.shape[1]):

@@ -3,7 +3,6 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part

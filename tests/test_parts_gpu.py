@@ -4,7 +4,6 @@ weights shared, a cache entry per run), a toy mixer that keeps a state of its ow
 no position encoding in one layer, a position encoding of another kind (a learned table added to q and
 k) and a feed-forward that routes every token to two of four experts in another; built and stepped
 through the unchanged engine."""
-import json
 import os
 from dataclasses import dataclass
 from typing import ClassVar
