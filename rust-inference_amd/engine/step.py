@@ -121,16 +121,16 @@ class Engine:
     """A model, its cache, and the step function over them.
 
     With ``use_graphs`` a step in which every sequence brings one token and wants its logits runs
-    as a HIP graph captured once per batch size: the launches of a decode step cost more than its
-    kernels otherwise.  Page tables then have the cache's full width and the attention grid is
-    sized for the longest sequence the cache allows; the results are the same."""
+    as a HIP graph captured once per batch size and bound on the sequence length: the launches of
+    a decode step cost more than its kernels otherwise.  Page tables then have the cache's full
+    width and the attention grid is sized for the bound; the results are the same."""
 
     def __init__(self, model, cache, use_graphs: bool = False):
         self.model, self.cache = model, cache
         self.device = model.rt.device
         self.use_graphs = use_graphs
         self._staging = None
-        self._graphs: dict[int, _DecodeGraph] = {}
+        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
 
     def _stage(self, n: int) -> _Staging:
         if self._staging is None or self._staging.capacity < n:
@@ -139,7 +139,7 @@ class Engine:
         return self._staging
 
     def build_context(self, entries: Sequence[StepEntry], staging: _Staging | None = None,
-                      full_width: bool = False) -> StepContext:
+                      full_width: bool = False, grid_len: int | None = None) -> StepContext:
         """Reserve the step's pages and send its layout to the device: one block of int32 words
         (tokens, sequence and position of each, sequence starts, slots, lengths after the step,
         wanted rows, a page table per key/value group), laid out by the cache's native side
@@ -188,7 +188,7 @@ class Engine:
                           tokens=piece(0, T), tok_seq=piece(1, T), tok_pos=piece(2, T), cu_seqlens=piece(3, B + 1),
                           slots=piece(4, B), len_after=piece(5, B), want_rows=piece(6, len(want)),
                           n_want=len(want), max_new=max(counts),
-                          max_len=cache.max_seq_len if full_width else max_len)
+                          max_len=grid_len or (cache.max_seq_len if full_width else max_len))
         ctx.page_tables = [piece(7 + gi, B * width).view(B, width) for gi in range(G)]
         return ctx
 
@@ -206,15 +206,21 @@ class Engine:
 
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         batch = len(entries)
-        dg = self._graphs.get(batch)
+        # A graph's launches are sized for sequences up to a power of two of tokens (1,024 at least, the
+        # cache's limit at most): the attention kernels launch a workgroup per chunk of keys that might be
+        # there, and a cache that allows long sequences must not make short ones pay for that.  A batch
+        # gets the next graph when its longest sequence grows past the bound.
+        longest = max(self.cache.length(e.slot) for e in entries) + 1
+        bound = min(self.cache.max_seq_len, max(1024, 1 << (longest - 1).bit_length()))
+        dg = self._graphs.get((batch, bound))
         if dg is None:
-            dg = self._graphs[batch] = _DecodeGraph(batch, self.device)
+            dg = self._graphs[(batch, bound)] = _DecodeGraph(batch, self.device)
             width = self.cache.max_pages_per_slot
             need = 7 * (batch + 5) + len(self.cache.groups) * (batch * width + 4)
             dg.staging = _Staging(need, self.device)
         # the layout of a decode step depends on the batch size alone, so the buffers a captured
         # graph reads are refilled in place
-        ctx = self.build_context(entries, staging=dg.staging, full_width=True)
+        ctx = self.build_context(entries, staging=dg.staging, full_width=True, grid_len=bound)
         if dg.graph is None:
             # once eagerly (libraries set themselves up outside the capture), then capture; writing
             # the same keys and values to the same places twice changes nothing, and per-sequence
