@@ -209,7 +209,9 @@ class Engine:
         # A graph's launches are sized for sequences up to a power of two of tokens (1,024 at least, the
         # cache's limit at most): the attention kernels launch a workgroup per chunk of keys that might be
         # there, and a cache that allows long sequences must not make short ones pay for that.  A batch
-        # gets the next graph when its longest sequence grows past the bound.
+        # gets the next graph when its longest sequence grows past the bound (capturing one costs about
+        # as much as two or three steps).  Finer bounds were tried and gained nothing: the workgroups of
+        # the empty chunks come last in the grid and cost little there.
         longest = max(self.cache.length(e.slot) for e in entries) + 1
         bound = min(self.cache.max_seq_len, max(1024, 1 << (longest - 1).bit_length()))
         dg = self._graphs.get((batch, bound))
