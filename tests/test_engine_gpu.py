@@ -254,3 +254,41 @@ def test_a_sequence_may_pass_max_position_embeddings(model_dirs, loaded):
     reqs = requests_for("A", cfg, [150], 99)
     got = replay_in_process(loaded("A", "float32"), plans.tail_one_by_one(reqs, 20))
     check_against_plain(model_dirs["A"], got, reqs, "float32", "past max_position_embeddings")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_any_cut_of_the_work_gives_the_same_logits(model_dirs, loaded, name, dtype_name):
+    """Steps of any shape: requests join at different times, and a step gives each live request between one
+    token and a few dozen, some of them one token (a decode step for them) beside others' long pieces; a
+    request that is finished leaves, and its slot serves the next one.  Every position's logits against the
+    plain implementation."""
+    from rust_inference_amd.engine import Engine, StepEntry
+    cfg, _ = read_model_f64(model_dirs[name])
+    rng = np.random.default_rng(7)
+    reqs = requests_for(name, cfg, [int(n) for n in rng.integers(1, 160, 9)], 123)
+    model = loaded(name, dtype_name)
+    engine = Engine(model, model.new_cache(max_tokens=4 * 192, num_slots=4, max_seq_len=192))
+    waiting, live, fed, got = list(reqs), {}, {}, {rid: [] for rid in reqs}
+    while waiting or live:
+        while waiting and len(live) < 4 and (not live or rng.random() < 0.5):
+            rid = waiting.pop(0)
+            live[rid], fed[rid] = engine.cache.acquire(), 0
+        entries, order = [], []
+        for rid, slot in live.items():
+            left = len(reqs[rid]) - fed[rid]
+            n = min(left, int(rng.choice([1, 1, 2, 7, 33, 64])))
+            entries.append(StepEntry(slot, reqs[rid][fed[rid]:fed[rid] + n], "all"))
+            order.append((rid, n))
+        logits = engine.step(entries).cpu().numpy()
+        at = 0
+        for rid, n in order:
+            got[rid].append(logits[at:at + n])
+            at += n
+            fed[rid] += n
+            if fed[rid] == len(reqs[rid]):
+                engine.cache.release(live.pop(rid))
+    engine.cache.check_consistent()
+    assert engine.cache.slots.free_count == 4
+    check_against_plain(model_dirs[name], {rid: np.concatenate(rows) for rid, rows in got.items()}, reqs, dtype_name,
+                        "any cut")
