@@ -292,3 +292,43 @@ def test_any_cut_of_the_work_gives_the_same_logits(model_dirs, loaded, name, dty
     assert engine.cache.slots.free_count == 4
     check_against_plain(model_dirs[name], {rid: np.concatenate(rows) for rid, rows in got.items()}, reqs, dtype_name,
                         "any cut")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_one_layer_of_the_large_model(tmp_path_factory, dtype_name):
+    """The layer sizes of Qwen3-8B (one layer, a small vocabulary): the sizes at which the decode kernels
+    choose their forms (rows shared by four wavefronts, packed weights, norms left to the products, the
+    attention kernel that also norms and rotates) run here end to end, eagerly and as graphs."""
+    from rust_inference_amd.engine import Engine
+    from rust_inference_amd.engine.replay import Replayer
+    from rust_inference_amd.parts import load_model
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 1000, "hidden_size": 4096,
+           "intermediate_size": 12288, "num_hidden_layers": 1, "num_attention_heads": 32, "num_key_value_heads": 8,
+           "head_dim": 128, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "tie_word_embeddings": False}
+    folder = _large_layer_folder(tmp_path_factory, cfg)
+    rng = np.random.default_rng(5)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, 1000, n)] for i, n in enumerate([290, 41, 130])}
+    model = load_model(folder, DTYPES[dtype_name])
+    for graphs in (False, True):
+        for what, steps in (("tail", plans.tail_one_by_one(reqs, 32)),
+                            ("batch", plans.unequal_batches([{k: (v, max(1, len(v) - 9)) for k, v in reqs.items()}]))):
+            cache = model.new_cache(max_tokens=plans.max_live_tokens(steps), num_slots=3, max_seq_len=320)
+            player, outs = Replayer(Engine(model, cache, use_graphs=graphs)), {}
+            for s in steps:
+                logits = player.feed(s)
+                if logits is not None:
+                    outs[s["step"]] = logits.cpu().numpy().copy()
+            got = plans.collect(steps, lambda i: outs[i], 1000)
+            check_against_plain(folder, got, reqs, dtype_name, f"large layer, {what}, graphs {graphs}")
+
+
+_large = {}
+
+
+def _large_layer_folder(tmp_path_factory, cfg):
+    """Written once for both dtypes (0.4 GB)."""
+    if "folder" not in _large:
+        from rust_inference_amd.weights import write_random_model
+        _large["folder"] = write_random_model(str(tmp_path_factory.mktemp("large") / "m"), cfg, seed=3,
+                                              dtype=torch.bfloat16, matrix_std=0.02, gain_std=0.1)
+    return _large["folder"]
