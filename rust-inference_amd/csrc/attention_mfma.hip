@@ -173,13 +173,16 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
 // A workgroup of four wavefronts takes 4 * (16 NT / group) consecutive tokens of one sequence and one kv
 // head.  The pages of keys and values go through LDS, fetched once for all four wavefronts and
 // double-buffered: while a page is in work the next one is on its way from global memory.  In LDS a key
-// row is padded to head_dim + 8 elements and a value row (one channel, 32 tokens) to 40, which spreads
-// the 16-byte fragment reads over all banks; the key rows of a page are stored in the order the two
-// MFMA tiles take them (rows {0-3, 8-11, 16-19, 24-27}, then the rest).
+// row is padded to head_dim + 16 elements and a value row (one channel, 32 tokens) to 48.  A fragment
+// read takes 16 bytes per lane with lanes 0-15 on 16 consecutive rows; timed alone, such reads run at the
+// full LDS rate (2.0 ns per wavefront read per CU) exactly when the row stride is 32 bytes modulo 64
+// (96, 160, 288 here), at 3.4-3.5 ns for every other stride that is not a multiple of 128 (a pad of 8
+// elements among them), and at 6.8 and 13.5 ns for multiples of 128 and 256.  The key rows of a page are
+// stored in the order the two MFMA tiles take them (rows {0-3, 8-11, 16-19, 24-27}, then the rest).
 template <int DH>
 struct LdsPage {
-    static constexpr int KS = DH + 8;                        // key row stride, elements
-    static constexpr int VS = PAGE + 8;                      // value row stride, elements
+    static constexpr int KS = DH + 16;                       // key row stride, elements
+    static constexpr int VS = PAGE + 16;                     // value row stride, elements
     static constexpr int CHUNKS = 4 * DH;                    // 16-byte pieces of a key page (and of a value page)
     static constexpr int PER_THREAD = (CHUNKS + 255) / 256;
 };
