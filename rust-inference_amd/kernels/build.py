@@ -29,6 +29,12 @@ CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-Wno-unused-command-line-argument",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
+# Flags of single files.  The attention kernels take maxima of matrix-core results; unless the compiler may
+# take them for numbers, it first passes every operand through an instruction that quiets signalling NaNs
+# (IEEE mode), which is a fifth of the softmax's vector instructions.  The kernels produce no NaN from
+# numbers: a masked score is -inf, and a column without a key uses 0 as its reference point.
+FILE_FLAGS = {"attention_mfma.hip": ["-fno-honor-nans"]}
+
 _lib = None
 
 
@@ -47,6 +53,7 @@ def source_hash() -> str:
         with open(path, "rb") as f:
             h.update(f.read())
     h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
 
@@ -66,7 +73,8 @@ def _is_current(lib_path: str) -> bool:
 
 
 def _compile_one(hipcc: str, src: str, obj: str, env: dict) -> None:
-    proc = subprocess.run([hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj], capture_output=True, text=True, env=env)
+    flags = HIPCC_FLAGS + FILE_FLAGS.get(os.path.basename(src), [])
+    proc = subprocess.run([hipcc, *flags, "-c", src, "-o", obj], capture_output=True, text=True, env=env)
     if proc.returncode != 0:
         raise KernelError(f"hipcc failed on {os.path.basename(src)}:\n{proc.stderr[-4000:]}")
 
