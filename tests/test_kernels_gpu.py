@@ -248,6 +248,23 @@ def test_mfma_decode_attention(ops, heads, kv_heads, dh):
     close(out, want, 1e-2, "decode attention on the matrix cores")
 
 
+@pytest.mark.parametrize("window", [None, 4500])
+def test_mfma_decode_attention_over_thousands_of_keys(ops, window):
+    """Past 16 chunks of 256 keys the chunks are joined in runs: sequences on both sides of that edge in one
+    call, and in the longest a key that stands out, placed in the first run, in a middle one and in the last."""
+    heads, kv_heads, dh = 4, 2, 64
+    lens = [4096, 4097, 6000, 700]
+    for far in (0, 2500, 5999):
+        rng = np.random.default_rng(31 + far)
+
+        def boost(qkv, k, kp, table, far=far):
+            kf = f64(kp[table[2, far // 32].item(), 0, far % 32])          # sequence 2, kv head 0: query head 1
+            qkv[2, dh:2 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16,
+                                   window=window, boost=boost, kernel="decode")
+        close(out, want, 1e-2, f"far key {far}, window {window}")
+
+
 @pytest.mark.parametrize("kernel", ["prefill", "decode"])
 def test_mfma_attention_finds_one_far_key(ops, kernel):
     rng = np.random.default_rng(19)
