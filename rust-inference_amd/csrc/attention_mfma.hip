@@ -20,6 +20,9 @@
 // second product rounded to bfloat16, the running sum is taken of them before the rounding.  (Letting
 // the reference point of the exponents lag behind the running maximum, so that the accumulators are
 // rescaled only rarely, was tried and changed no timing: the rescaling is not what the kernel waits for.)
+// (Also tried with two tiles a wavefront: all scores first, then one tile's value product interleaved with
+// the other tile's exponentials by scheduling hints.  The instructions came out in that order and the
+// kernel gained 1%: the two wavefronts of a SIMD already fill each other's gaps.)
 //
 // Prefill: one wavefront per tile of tokens, walking the sequence's pages in order; the four
 // wavefronts of a workgroup share the pages through LDS.  Decode (one new
