@@ -65,10 +65,6 @@ class KVGroup:
         self.k_pages = torch.zeros(k_shape, dtype=dtype, device=device) if allocate else None
         self.v_pages = torch.zeros(v_shape, dtype=dtype, device=device) if allocate else None
 
-    def table_rows(self, slots: Sequence[int], width: int):
-        """``[len(slots), width]`` int32 (numpy): the page tables of these slots."""
-        return self.pool.gather(slots, width)
-
 
 @dataclass
 class KVView:

@@ -46,15 +46,9 @@ class SlotAllocator:
     def release(self, slot: int) -> None:
         native.check(self._lib.ri_cache_release(self._core.handle, int(slot)))
 
-    def check_held(self, slot: int) -> None:
-        native.check(self._lib.ri_cache_check_held(self._core.handle, int(slot)))
-
     def is_held(self, slot: int) -> bool:
         return bool(self._lib.ri_cache_is_held(self._core.handle, int(slot)))
 
     @property
     def free_count(self) -> int:
         return self._lib.ri_cache_free_slots(self._core.handle)
-
-    def held_slots(self) -> list[int]:
-        return [s for s in range(self.num_slots) if self.is_held(s)]
