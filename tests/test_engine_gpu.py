@@ -138,6 +138,16 @@ def test_long_decoding(model_dirs, loaded, dtype_name):
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_decoding_over_thousands_of_keys(model_dirs, loaded, dtype_name):
+    """4,200 tokens, the last 8 one by one, beside a request of 300: past 4,096 keys the decode attention
+    joins its chunks in runs, and one batch holds a sequence on either side of that."""
+    cfg, _ = read_model_f64(model_dirs["D"])
+    reqs = requests_for("D", cfg, [4200, 300], 66)
+    got = replay_in_process(loaded("D", dtype_name), plans.tail_one_by_one(reqs, 8))
+    check_against_plain(model_dirs["D"], got, reqs, dtype_name, "thousands of keys")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_first_tokens_of_a_sequence(model_dirs, loaded, dtype_name):
     """Every token from the first one on its own step: position 0 sees one key only."""
     cfg, _ = read_model_f64(model_dirs["A"])
