@@ -452,3 +452,140 @@ def test_toy_model_decodes_the_same_through_graphs(toy_dir):
         outs.append(rows)
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------------------ another arrangement
+SIDE = {"architectures": ["ToySideBySideForCausalLM"], "vocab_size": 90, "hidden_size": 64, "inter": 112, "heads": 4,
+        "kv_heads": 1, "head_dim": 32, "eps": 1e-6, "theta": 5000.0}
+
+
+def register_side_by_side():
+    """An arrangement of its own, registered from here: one norm feeds the mixer and the feed-forward side by
+    side, ``h' = h + mixer(n(h)) + ff(n(h))``, so two branch outputs wait for the stream at once."""
+    from rust_inference_amd.config import ModelConfig, register_architecture
+    from rust_inference_amd.parts import LayerSpec, ModelSpec, PartSpec, Run, register_part
+    from rust_inference_amd.parts.registry import build_part
+
+    @register_part("arrangement", "toy_side_by_side")
+    class SideBySide:
+        def __init__(self, layer_spec):
+            self.norm = build_part("norm", layer_spec.mixer_norm)
+            self.mixer = build_part("mixer", layer_spec.mixer)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward)
+
+        def parts(self):
+            return (self.norm, self.mixer, self.feed_forward)
+
+        def forward(self, stream, ctx, store, page_table, act_dtype):
+            h = stream.normed(self.norm, act_dtype)
+            stream.push(self.mixer.forward(h, ctx, store, page_table))
+            stream.push(self.feed_forward.forward(h, ctx))
+
+    @dataclass(frozen=True)
+    class SideConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        inter: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        eps: float = 1e-6
+        theta: float = 1e4
+        ARCHITECTURE: ClassVar[str] = "ToySideBySideForCausalLM"
+        MODEL_TYPE: ClassVar[str] = "toy_side_by_side"
+
+        @classmethod
+        def from_dict(cls, raw):
+            import dataclasses
+            return cls(**{f.name: raw[f.name] for f in dataclasses.fields(cls)})
+
+    def spec(c):
+        d = c.hidden_size
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"dim": d, "eps": c.eps, "name": name})
+
+        def layer(p, arrangement):
+            return LayerSpec(
+                arrangement=arrangement, mixer_norm=norm(p + "n1"), feed_forward_norm=norm(p + "n2"),
+                feed_forward=PartSpec("swiglu", {"hidden": d, "inter": c.inter, "prefix": p + "ff."}),
+                mixer=PartSpec("attention", {"hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                             "prefix": p + "attn.", "qk_norm": True, "eps": c.eps, "window": None,
+                                             "position": PartSpec("rotate_half", {"head_dim": c.head_dim, "theta": c.theta})}))
+        return ModelSpec(
+            architecture="ToySideBySideForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
+            embedding=PartSpec("table", {"vocab": c.vocab_size, "dim": d, "name": "embed.weight"}),
+            layers=(layer("l0.", "toy_side_by_side"), layer("l1.", "prenorm"), layer("l2.", "toy_side_by_side")),
+            schedule=(Run(0, 0), Run(1, 1), Run(2, 2)),
+            final_norm=norm("final.weight"),
+            head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": True}),
+            max_positions=256)
+
+    register_architecture("ToySideBySideForCausalLM", SideConfig, spec, model_types=("toy_side_by_side",))
+
+
+def side_plain(w, ids):
+    c = SIDE
+    h = P.embedding(w["embed.weight"], ids)
+    ang = P.rope_angles(np.arange(len(ids)), c["head_dim"], c["theta"])
+
+    def attn(x, p):
+        s = x.shape[0]
+        q = P.rms_norm((x @ w[p + "attn.q_proj.weight"].T).reshape(s, c["heads"], c["head_dim"]),
+                       w[p + "attn.q_norm.weight"], c["eps"])
+        k = P.rms_norm((x @ w[p + "attn.k_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"]),
+                       w[p + "attn.k_norm.weight"], c["eps"])
+        v = (x @ w[p + "attn.v_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        return P.attention(P.apply_rope(q, ang), P.apply_rope(k, ang), v).reshape(s, -1) @ w[p + "attn.o_proj.weight"].T
+
+    def ff(x, p):
+        return P.swiglu_mlp(x, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+
+    def side_by_side(h, p):
+        x = P.rms_norm(h, w[p + "n1"], c["eps"])
+        return h + attn(x, p) + ff(x, p)
+
+    h = side_by_side(h, "l0.")
+    r = h + attn(P.rms_norm(h, w["l1.n1"], c["eps"]), "l1.")
+    h = r + ff(P.rms_norm(r, w["l1.n2"], c["eps"]), "l1.")
+    h = side_by_side(h, "l2.")
+    return P.rms_norm(h, w["final.weight"], c["eps"]) @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_an_arrangement_of_its_own(tmp_path, dtype_name):
+    """Layers whose two branches read one norm and are added together, around a pre-norm layer: registered
+    here, built by the unchanged model class, stepped whole, token by token and through graphs."""
+    register_side_by_side()
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    from safetensors import safe_open
+    folder = write_random_model(str(tmp_path / "m"), SIDE, seed=11, dtype=torch.float32, matrix_std=0.12)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
+    assert "l0.n2" not in w and "l1.n2" in w          # the arrangement says which tensors a layer has
+    model = load_model(folder, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
+    rng = np.random.default_rng(12)
+    reqs = {f"r{i}": [int(x) for x in rng.integers(0, SIDE["vocab_size"], n)] for i, n in enumerate([50, 7, 33])}
+    for what, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 20))):
+        engine = engine_for_trace(model, plans.max_live_tokens(steps))
+        player, outs = Replayer(engine), {}
+        for s in steps:
+            logits = player.feed(s)
+            if logits is not None:
+                outs[s["step"]] = logits.cpu().numpy()
+        got = plans.collect(steps, lambda i: outs[i], SIDE["vocab_size"])
+        for rid, toks in reqs.items():
+            assert_logits_close(got[rid], side_plain(w, toks), dtype_name, f"side by side, {what}, {rid}")
+    if dtype_name == "bfloat16":                       # decode steps as graphs give what eager steps give
+        rows = []
+        for graphs in (False, True):
+            eng = Engine(model, model.new_cache(max_tokens=2 * 64, num_slots=2, max_seq_len=64), use_graphs=graphs)
+            slots = [eng.cache.acquire() for _ in range(2)]
+            eng.step([StepEntry(s, p[:9], "last") for s, p in zip(slots, reqs.values())])
+            rows.append([eng.step([StepEntry(s, [(3 * i + s) % SIDE["vocab_size"]], "last") for s in slots]).clone()
+                         for i in range(6)])
+        for a, b in zip(*rows):
+            assert torch.equal(a, b)
