@@ -589,3 +589,140 @@ def test_an_arrangement_of_its_own(tmp_path, dtype_name):
                          for i in range(6)])
         for a, b in zip(*rows):
             assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------------------ a layer that reads another's cache
+SHARED = {"architectures": ["ToySharedCacheForCausalLM"], "vocab_size": 77, "hidden_size": 40, "inter": 72, "heads": 4,
+          "kv_heads": 2, "head_dim": 16, "eps": 1e-5, "theta": 10000.0}
+
+
+def register_shared_cache():
+    """Two layers on one cache entry: an attention layer writes keys and values, and a mixer defined here
+    reads that entry's values after it and writes nothing."""
+    from rust_inference_amd.cache import KVNeed
+    from rust_inference_amd.config import ModelConfig, register_architecture
+    from rust_inference_amd.parts import LayerSpec, Mixer, ModelSpec, PartSpec, Run, register_part
+    from rust_inference_amd.weights import MATRIX, TensorSpec
+
+    @register_part("mixer", "toy_value_mean")
+    class ValueMean(Mixer):
+        """y_t = W . mean(v_0 .. v_t), v_j the values of all kv heads at position j as they lie in the cache."""
+        def __init__(self, hidden, kv_heads, head_dim, name):
+            self.hidden, self.kv_heads, self.head_dim, self.name = hidden, kv_heads, head_dim, name
+
+        def tensors(self):
+            return {self.name: TensorSpec((self.hidden, self.kv_heads * self.head_dim), MATRIX)}
+
+        def bind(self, weights, rt):
+            self.w = weights[self.name].to(rt.device, torch.float32)
+
+        def cache_need(self):
+            return KVNeed(self.kv_heads, self.head_dim, None)          # the writer's need: one entry serves both
+
+        def forward(self, x, ctx, store, page_table):
+            out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            begin = 0
+            for b, (start, n) in enumerate(zip(ctx.starts, ctx.new_counts)):
+                length = start + n
+                pages = page_table[b, :-(-length // store.page_size)].long()
+                v = store.v_pages[pages]                                # [pages, kv heads, head_dim, page]
+                v = v.permute(0, 3, 1, 2).reshape(-1, self.kv_heads * self.head_dim)[:length].float()
+                count = torch.arange(start + 1, length + 1, device=x.device, dtype=torch.float32)
+                out[begin:begin + n] = (torch.cumsum(v, 0)[start:] / count[:, None]) @ self.w.T
+                begin += n
+            return out
+
+    @dataclass(frozen=True)
+    class SharedConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        inter: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        eps: float = 1e-5
+        theta: float = 1e4
+        ARCHITECTURE: ClassVar[str] = "ToySharedCacheForCausalLM"
+        MODEL_TYPE: ClassVar[str] = "toy_shared_cache"
+
+        @classmethod
+        def from_dict(cls, raw):
+            import dataclasses
+            return cls(**{f.name: raw[f.name] for f in dataclasses.fields(cls)})
+
+    def spec(c):
+        d = c.hidden_size
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"dim": d, "eps": c.eps, "name": name})
+
+        def ff(p):
+            return PartSpec("swiglu", {"hidden": d, "inter": c.inter, "prefix": p})
+        writer = LayerSpec(
+            mixer_norm=norm("l0.n1"), feed_forward_norm=norm("l0.n2"), feed_forward=ff("l0.ff."),
+            mixer=PartSpec("attention", {"hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                         "prefix": "l0.attn.", "qk_norm": False, "eps": c.eps, "window": None,
+                                         "position": PartSpec("rotate_half", {"head_dim": c.head_dim, "theta": c.theta})}))
+        reader = LayerSpec(
+            mixer_norm=norm("l1.n1"), feed_forward_norm=norm("l1.n2"), feed_forward=ff("l1.ff."),
+            mixer=PartSpec("toy_value_mean", {"hidden": d, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                              "name": "l1.mean.weight"}))
+        return ModelSpec(
+            architecture="ToySharedCacheForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
+            embedding=PartSpec("table", {"vocab": c.vocab_size, "dim": d, "name": "embed.weight"}),
+            layers=(writer, reader), schedule=(Run(0, 0), Run(1, 0)),       # both runs name cache entry 0
+            final_norm=norm("final.weight"),
+            head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": False}),
+            max_positions=256)
+
+    register_architecture("ToySharedCacheForCausalLM", SharedConfig, spec, model_types=("toy_shared_cache",))
+
+
+def shared_plain(w, ids):
+    c = SHARED
+    s = len(ids)
+    h = P.embedding(w["embed.weight"], ids)
+    ang = P.rope_angles(np.arange(s), c["head_dim"], c["theta"])
+    x = P.rms_norm(h, w["l0.n1"], c["eps"])
+    q = (x @ w["l0.attn.q_proj.weight"].T).reshape(s, c["heads"], c["head_dim"])
+    k = (x @ w["l0.attn.k_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+    v = (x @ w["l0.attn.v_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+    r = h + P.attention(P.apply_rope(q, ang), P.apply_rope(k, ang), v).reshape(s, -1) @ w["l0.attn.o_proj.weight"].T
+    h = r + P.swiglu_mlp(P.rms_norm(r, w["l0.n2"], c["eps"]), w["l0.ff.gate_proj.weight"], w["l0.ff.up_proj.weight"],
+                         w["l0.ff.down_proj.weight"])
+    mean = np.cumsum(v.reshape(s, -1), 0) / np.arange(1, s + 1)[:, None]
+    r = h + mean @ w["l1.mean.weight"].T                     # the reader ignores its own input: only the cache counts
+    h = r + P.swiglu_mlp(P.rms_norm(r, w["l1.n2"], c["eps"]), w["l1.ff.gate_proj.weight"], w["l1.ff.up_proj.weight"],
+                         w["l1.ff.down_proj.weight"])
+    return P.rms_norm(h, w["final.weight"], c["eps"]) @ w["head.weight"].T
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_a_layer_reads_the_cache_another_layer_wrote(tmp_path, dtype_name):
+    register_shared_cache()
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    from safetensors import safe_open
+    folder = write_random_model(str(tmp_path / "m"), SHARED, seed=21, dtype=torch.float32, matrix_std=0.12)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
+    model = load_model(folder, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
+    assert len(model.cache_needs()) == 1                      # two runs, one entry
+    rng = np.random.default_rng(22)
+    reqs = {f"r{i}": [int(x) for x in rng.integers(0, SHARED["vocab_size"], n)] for i, n in enumerate([45, 6, 70, 33])}
+    for what, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 32)),
+                        ("batches", plans.unequal_batches([
+                            {k: (v, max(1, len(v) - 20)) for k, v in list(reqs.items())[:2]},
+                            {k: (v, max(1, len(v) - 33)) for k, v in list(reqs.items())[2:]}]))):
+        engine = engine_for_trace(model, plans.max_live_tokens(steps))
+        assert len(engine.cache.groups) == 1 and engine.cache.groups[0].entries == [0]
+        player, outs = Replayer(engine), {}
+        for s in steps:
+            logits = player.feed(s)
+            if logits is not None:
+                outs[s["step"]] = logits.cpu().numpy()
+        engine.cache.check_consistent()
+        got = plans.collect(steps, lambda i: outs[i], SHARED["vocab_size"])
+        for rid, toks in reqs.items():
+            assert_logits_close(got[rid], shared_plain(w, toks), dtype_name, f"shared cache, {what}, {rid}")
