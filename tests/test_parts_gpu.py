@@ -726,3 +726,131 @@ def test_a_layer_reads_the_cache_another_layer_wrote(tmp_path, dtype_name):
         got = plans.collect(steps, lambda i: outs[i], SHARED["vocab_size"])
         for rid, toks in reqs.items():
             assert_logits_close(got[rid], shared_plain(w, toks), dtype_name, f"shared cache, {what}, {rid}")
+
+
+# ------------------------------------------------------------------------------------------------ another norm
+CENTRED = {"architectures": ["ToyCentredNormForCausalLM"], "vocab_size": 61, "hidden_size": 56, "inter": 88, "heads": 2,
+           "kv_heads": 2, "head_dim": 32, "eps": 1e-4, "theta": 20000.0}
+
+
+def register_centred_norm():
+    """A norm with a mean, a gain and a bias, registered from here and used at every norm of a model."""
+    from rust_inference_amd.config import ModelConfig, register_architecture
+    from rust_inference_amd.parts import LayerSpec, ModelSpec, Norm, PartSpec, Run, register_part
+    from rust_inference_amd.weights import GAIN, TensorSpec
+
+    @register_part("norm", "toy_centred")
+    class CentredNorm(Norm):
+        def __init__(self, dim, eps, name):
+            self.dim, self.eps, self.name = dim, eps, name
+
+        def tensors(self):
+            return {self.name + ".weight": TensorSpec((self.dim,), GAIN), self.name + ".bias": TensorSpec((self.dim,), GAIN)}
+
+        def bind(self, weights, rt):
+            self.w = rt.place_gain(weights[self.name + ".weight"])
+            self.b = rt.place_gain(weights[self.name + ".bias"])
+
+        def apply(self, residual, pending, out_dtype, rows=None):
+            total = residual if pending is None else residual + pending.float()
+            if rows is None:
+                if pending is not None:
+                    residual.copy_(total)                    # the stream takes the sum
+                x = residual
+            else:
+                x = total[rows.long()]
+            x = x - x.mean(-1, keepdim=True)
+            y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.w + self.b
+            return y.to(out_dtype)
+
+    @dataclass(frozen=True)
+    class CentredConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        inter: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        eps: float = 1e-5
+        theta: float = 1e4
+        ARCHITECTURE: ClassVar[str] = "ToyCentredNormForCausalLM"
+        MODEL_TYPE: ClassVar[str] = "toy_centred_norm"
+
+        @classmethod
+        def from_dict(cls, raw):
+            import dataclasses
+            return cls(**{f.name: raw[f.name] for f in dataclasses.fields(cls)})
+
+    def spec(c):
+        d = c.hidden_size
+
+        def norm(name):
+            return PartSpec("toy_centred", {"dim": d, "eps": c.eps, "name": name})
+
+        def layer(p):
+            return LayerSpec(
+                mixer_norm=norm(p + "n1"), feed_forward_norm=norm(p + "n2"),
+                feed_forward=PartSpec("swiglu", {"hidden": d, "inter": c.inter, "prefix": p + "ff."}),
+                mixer=PartSpec("attention", {"hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                             "prefix": p + "attn.", "qk_norm": True, "eps": c.eps, "window": None,
+                                             "position": PartSpec("rotate_half", {"head_dim": c.head_dim, "theta": c.theta})}))
+        return ModelSpec(
+            architecture="ToyCentredNormForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
+            embedding=PartSpec("table", {"vocab": c.vocab_size, "dim": d, "name": "embed.weight"}),
+            layers=(layer("l0."), layer("l1.")), schedule=(Run(0, 0), Run(1, 1)),
+            final_norm=norm("final"),
+            head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": False}),
+            max_positions=256)
+
+    register_architecture("ToyCentredNormForCausalLM", CentredConfig, spec, model_types=("toy_centred_norm",))
+
+
+def centred_plain(w, ids):
+    c = CENTRED
+    s = len(ids)
+    ang = P.rope_angles(np.arange(s), c["head_dim"], c["theta"])
+
+    def norm(x, name):
+        x = x - x.mean(-1, keepdims=True)
+        return x / np.sqrt((x * x).mean(-1, keepdims=True) + c["eps"]) * w[name + ".weight"] + w[name + ".bias"]
+
+    h = P.embedding(w["embed.weight"], ids)
+    for p in ("l0.", "l1."):
+        x = norm(h, p + "n1")
+        q = P.rms_norm((x @ w[p + "attn.q_proj.weight"].T).reshape(s, c["heads"], c["head_dim"]),
+                       w[p + "attn.q_norm.weight"], c["eps"])
+        k = P.rms_norm((x @ w[p + "attn.k_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"]),
+                       w[p + "attn.k_norm.weight"], c["eps"])
+        v = (x @ w[p + "attn.v_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        r = h + P.attention(P.apply_rope(q, ang), P.apply_rope(k, ang), v).reshape(s, -1) @ w[p + "attn.o_proj.weight"].T
+        h = r + P.swiglu_mlp(norm(r, p + "n2"), w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"],
+                             w[p + "ff.down_proj.weight"])
+    return norm(h, "final") @ w["head.weight"].T
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_a_norm_of_its_own(tmp_path, dtype_name):
+    """Every norm of the model is one registered here (mean, gain, bias): prompts whole, their tails token by
+    token (steps small enough that the products would take over an RMSNorm: here they must not)."""
+    register_centred_norm()
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    from safetensors import safe_open
+    folder = write_random_model(str(tmp_path / "m"), CENTRED, seed=31, dtype=torch.float32, matrix_std=0.12)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
+    assert "l0.n1.bias" in w
+    model = load_model(folder, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
+    rng = np.random.default_rng(32)
+    reqs = {f"r{i}": [int(x) for x in rng.integers(0, CENTRED["vocab_size"], n)] for i, n in enumerate([40, 5, 66])}
+    for what, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 24))):
+        engine = engine_for_trace(model, plans.max_live_tokens(steps))
+        player, outs = Replayer(engine), {}
+        for s in steps:
+            logits = player.feed(s)
+            if logits is not None:
+                outs[s["step"]] = logits.cpu().numpy()
+        got = plans.collect(steps, lambda i: outs[i], CENTRED["vocab_size"])
+        for rid, toks in reqs.items():
+            assert_logits_close(got[rid], centred_plain(w, toks), dtype_name, f"centred norm, {what}, {rid}")
