@@ -94,11 +94,11 @@ __device__ __forceinline__ void load_page(PageFrags<DH>& f, const bf16_t* __rest
         const int row = (i >> 2) * 8 + kt * 4 + (i & 3);
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks)
-            f.k[kt][ks].u = *reinterpret_cast<const uint4*>(kbase + row * DH + ks * 32 + jg * 8);
+            f.k[kt][ks].u = load_stream16(kbase + row * DH + ks * 32 + jg * 8);
     }
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt)
-        f.v[dt].u = *reinterpret_cast<const uint4*>(vbase + (dt * 16 + i) * PAGE + jg * 8);
+        f.v[dt].u = load_stream16(vbase + (dt * 16 + i) * PAGE + jg * 8);
 }
 
 // The state of NT tiles of 16 columns.  Lane l belongs to column l % 16 of every tile.

@@ -28,6 +28,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return *reinterpret_cast<const uint32_t*>(&v);
 }
 
+// A 16-byte load of data that is read once (a weight matrix streaming through): marked non-temporal, so
+// that it does not displace what the caches hold to be used again.
+__device__ __forceinline__ uint4 load_stream16(const void* p) {
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
 __device__ __forceinline__ void from_f32(float* p, float v) { *p = v; }

@@ -44,8 +44,8 @@ gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
         for (int c = 0; c < SK_CHUNK; ++c) {
             const int kk = k + c * 32;
             const bool ok = kk + jg * 8 < k_end;          // K and the slices are multiples of 8: all eight or none
-            wf[c].u = (ok && row_ok) ? *reinterpret_cast<const uint4*>(wp + kk) : zero;
-            if (SWIGLU) uf[c].u = (ok && row_ok) ? *reinterpret_cast<const uint4*>(up + kk) : zero;
+            wf[c].u = (ok && row_ok) ? load_stream16(wp + kk) : zero;
+            if (SWIGLU) uf[c].u = (ok && row_ok) ? load_stream16(up + kk) : zero;
             xf[c].u = (ok && x_ok) ? *reinterpret_cast<const uint4*>(xp + kk) : zero;
         }
 #pragma unroll
@@ -134,8 +134,8 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
 #pragma unroll
         for (int c = 0; c < SK_CHUNK; ++c) {
             const bool live = kt + c < kt_end;
-            wf[c].u = live ? *reinterpret_cast<const uint4*>(wp + (size_t)(kt + c) * 512) : zero;
-            if (SWIGLU) uf[c].u = live ? *reinterpret_cast<const uint4*>(up + (size_t)(kt + c) * 512) : zero;
+            wf[c].u = live ? load_stream16(wp + (size_t)(kt + c) * 512) : zero;
+            if (SWIGLU) uf[c].u = live ? load_stream16(up + (size_t)(kt + c) * 512) : zero;
             // the packed matrix is zero beyond K; x is not padded
             xf[c].u = (live && x_ok && (kt + c) * 32 + jg * 8 < K) ? *reinterpret_cast<const uint4*>(xp + (kt + c) * 32)
                                                                  : zero;

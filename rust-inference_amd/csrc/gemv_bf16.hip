@@ -66,8 +66,8 @@ gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_
     if (row_ok) {
         for (int k = k_begin + lane * 8; k < k_end; k += RI_WAVE * 8) {
             float wv[8], uv[8];
-            unpack8(*reinterpret_cast<const uint4*>(wr + k), wv);
-            if (SWIGLU) unpack8(*reinterpret_cast<const uint4*>(wu + k), uv);
+            unpack8(load_stream16(wr + k), wv);
+            if (SWIGLU) unpack8(load_stream16(wu + k), uv);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 if (m < M) {
