@@ -28,14 +28,28 @@ GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
 SPLIT_K = 4096
 # Which matrices get a packed copy for 3 to 16 rows (the gate|up matrix always does: its activation
-# rides in the kernel).  Measured at 4, 8 and 16 rows, packed kernel against library, in us:
-#   4096 x 1024 (8 MB) 4.5 : 7.5     1024 x 3072 (6 MB) 7.4 : 12.0    2048 x 2048 (8 MB) 5.9 : 11.1
-#   4096 x 4096 (34 MB) 10.8 : 15.4  6144 x 4096 (50 MB) 16.2 : 15.3  2560 x 9728 (50 MB) 19.7 : 18.3
-#   4096 x 12288 (101 MB) 27 : 22    10240 x 5120 (105 MB) 32 : 24    5120 x 8192 (84 MB) 29 : 20
-#   5120 x 25600 (262 MB) 90 : 136, and 74 with K cut into parts
-# so: the small ones, and the very long rows.
-PACKED_MAX_BYTES = 40_000_000
+# rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
+#   4096 x 1024 (8 MB) 4.1 : 7.5     1024 x 3072 (6 MB) 7.0 : 11.9    2048 x 2048 (8 MB) 5.3 : 11.0
+#   4096 x 4096 (34 MB) 9.2 : 15.3   6144 x 4096 (50 MB) 15.4 : 15.5  2560 x 9728 (50 MB) 19.2 : 18.3
+#   4096 x 12288 (101 MB) 22.5 : 21.3   5120 x 8192 (84 MB) 27.3 : 19.5   10240 x 5120 (105 MB) 29.7 : 24.3
+#   5120 x 25600 (262 MB) 85 : 135, and 65 with K cut into four parts
+# A product of this library's own also does the norms next to it (about 6 us each at these sizes) when its
+# neighbours are its own too, so a draw goes to the packed kernel: with q|k|v and down on it a decode step
+# of 8 sequences at Qwen3-8B sizes has no norm kernel left and is 3% shorter.  The kernel is a workgroup per
+# 16 rows of the matrix, and what it loses by is a last round of workgroups that leaves most compute units
+# idle (5120 rows: 320 workgroups on 256 compute units); cutting K into parts fills the round, but the parts
+# cannot add themselves into the residual stream, so only rows of 16,384 elements and more are cut.
+PACKED_MAX_BYTES = 101_000_000
 PACKED_LONG_K = 16384
+COMPUTE_UNITS = 256
+
+
+def _packed_pays(n: int, k: int) -> bool:
+    if k >= PACKED_LONG_K or n * k * 2 <= 40_000_000:
+        return True
+    tiles = -(-n // 16)
+    last_round = tiles % COMPUTE_UNITS
+    return n * k * 2 <= PACKED_MAX_BYTES and not (tiles > COMPUTE_UNITS and 0 < last_round < COMPUTE_UNITS // 2)
 
 
 class PackedWeight:
@@ -48,7 +62,7 @@ class PackedWeight:
         self.k = w.shape[1]
         # a long K is cut into pieces of 4096 whose float32 sums the next norm adds up: more workgroups
         # stream the weights (768 instead of 256 for 4096 x 12288), and the sum is never rounded to 16 bits
-        self.parts = self.k // SPLIT_K if (not swiglu and self.k >= 2 * SPLIT_K) else 1
+        self.parts = self.k // SPLIT_K if (not swiglu and self.k >= PACKED_LONG_K) else 1
 
 
 class Runtime:
@@ -108,7 +122,7 @@ class Runtime:
         """A placed weight, with a packed copy where the packed kernel is the faster one for 3 to 16
         rows (bfloat16 compute only)."""
         n, k = w.shape
-        pays = swiglu or n * k * 2 <= PACKED_MAX_BYTES or k >= PACKED_LONG_K
+        pays = swiglu or _packed_pays(n, k)
         if self.dtype != torch.bfloat16 or k % 8 or not pays:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
