@@ -94,8 +94,16 @@ int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, 
 // ceil(n/16) row tiles follow the gate's.
 // parts > 1 cuts K into that many pieces whose float32 sums go to out[part][m][n] (the consumer adds them in
 // order); it needs out_dtype float32 and no swiglu.
+// tiled: bit 0, the rows of x lie in the matrix cores' operand order (tiles of 32 columns, each 64 lanes x 8
+// elements, lane l holding row l % 16 and the columns 8 * (l / 16) ..+8 of the tile); bit 1, the bfloat16
+// result is to lie so (a product writes it for the next one, which then loads a tile as one kilobyte).
 int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
-                               int swiglu, int parts, void* stream);
+                               int swiglu, int parts, int tiled, void* stream);
+
+// The same product for 17 to 64 rows of x (it takes fewer too): every weight fragment meets two or four
+// tiles of 16 rows of x.  No parts, no links.
+int ri_gemm_mid_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
+                            int swiglu, void* stream);
 
 // The two decode-size products linked to the RMSNorms around them, so that those need no kernels of their
 // own.  W . norm(r) with norm(r) = r * inv * g equals inv * (W . (r * g)), inv = 1 / sqrt(mean(r^2) + eps):
@@ -113,7 +121,7 @@ int ri_gemm_skinny_packed_bf16_partials(int n);
 int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
                                       int k, int swiglu, const float* ssq_in, int n_in, float eps, int dim,
                                       float* residual, const float* next_gain, void* xg_out, float* ssq_out,
-                                      void* stream);
+                                      int tiled, void* stream);
 
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);

@@ -24,6 +24,17 @@ union Frag {
 
 __device__ __forceinline__ float silu_sk(float z) { return z / (1.0f + expf(-z)); }
 
+// Up to 16 rows of activations in the order the matrix cores take them as a B operand: tiles of 32 columns,
+// each 64 lanes x 8 elements, lane l holding row l % 16 and the columns 8 * (l / 16) ..+8 of the tile.  A
+// product that writes its result this way spares the next one loads that touch sixteen cache lines for
+// half of each: the tile is one kilobyte in a row.  TILED_X: x lies so; TILED_OUT: the bfloat16 result
+// (out, or a link's xg_out) is to lie so.
+#define TILED_X 1
+#define TILED_OUT 2
+__device__ __forceinline__ size_t tiled_at(int m, int n) {
+    return ((size_t)(n >> 5) * 64 + (m & 15) + 16 * ((n & 31) >> 3)) * 8 + (n & 7);
+}
+
 template <int SK_WAVES, bool SWIGLU, typename TO>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N,
@@ -88,7 +99,7 @@ gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
 template <int SK_WAVES, bool SWIGLU, typename TO>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked,
-                          int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset, NormLink link) {
+                          int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset, NormLink link, int tiled) {
     __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][4][64];
     __shared__ float inv_lds[16];
     __shared__ float sq_lds[16][17];
@@ -104,7 +115,9 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     out += (size_t)blockIdx.y * M * N;
     const bf16_t* wp = wpacked + ((size_t)nt * k_tiles * 64 + lane) * 8;
     const bf16_t* up = SWIGLU ? wpacked + ((size_t)(up_tile_offset + nt) * k_tiles * 64 + lane) * 8 : nullptr;
-    const bf16_t* xp = x + (size_t)(x_ok ? i : 0) * K + jg * 8;
+    const bool x_tiled = tiled & TILED_X;
+    const bf16_t* xp = x_tiled ? x + (size_t)lane * 8 : x + (size_t)(x_ok ? i : 0) * K + jg * 8;
+    const int x_step = x_tiled ? 512 : 32;                   // elements from one step's fragment to the next
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
     // Loads whose values are wanted only after the weights have streamed are issued here, so that their
@@ -140,8 +153,8 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
             wf[c].u = live ? load_stream16(wp + (size_t)(kt + c) * 512) : zero;
             if (SWIGLU) uf[c].u = live ? load_stream16(up + (size_t)(kt + c) * 512) : zero;
             // the packed matrix is zero beyond K; x is not padded
-            xf[c].u = (live && x_ok && (kt + c) * 32 + jg * 8 < K) ? *reinterpret_cast<const uint4*>(xp + (kt + c) * 32)
-                                                                 : zero;
+            xf[c].u = (live && x_ok && (kt + c) * 32 + jg * 8 < K)
+                          ? *reinterpret_cast<const uint4*>(xp + (size_t)(kt + c) * x_step) : zero;
         }
 #pragma unroll
         for (int c = 0; c < SK_CHUNK; ++c) {
@@ -188,11 +201,11 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
                 const size_t at = (size_t)m * N + n;
                 v += res_pre;
                 link.residual[at] = v;                   // this element belongs to this thread alone
-                link.xg_out[at] = f32_to_bf16(v * gain_pre);
+                link.xg_out[(tiled & TILED_OUT) ? tiled_at(m, n) : at] = f32_to_bf16(v * gain_pre);
             }
             sq_lds[m][nl] = ok ? v * v : 0.f;
         } else if (ok) {
-            from_f32(out + (size_t)m * N + n, v);
+            from_f32(out + ((tiled & TILED_OUT) ? tiled_at(m, n) : (size_t)m * N + n), v);
         }
     }
     if (link.residual) {                                 // the workgroup's share of every row's sum of squares
@@ -211,44 +224,46 @@ static int skinny_waves(int n, int k) { return k >= 8192 ? 8 : 4; }
 
 template <int WAVES, bool SWIGLU>
 static void launch_packed(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts,
-                          const NormLink& link, hipStream_t s) {
+                          const NormLink& link, int tiled, hipStream_t s) {
     const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
     const int part_tiles = (k_tiles + parts - 1) / parts;
     const int tiles_per_wave = (part_tiles + WAVES - 1) / WAVES;
     dim3 grid(row_tiles, parts);
     if (out_dtype == RI_F32)
         gemm_skinny_packed_kernel<WAVES, SWIGLU, float><<<grid, WAVES * 64, 0, s>>>(
-            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link);
+            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link, tiled);
     else
         gemm_skinny_packed_kernel<WAVES, SWIGLU, bf16_t><<<grid, WAVES * 64, 0, s>>>(
-            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link);
+            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link, tiled);
 }
 
 static int packed_run(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k, int swiglu,
-                      int parts, const NormLink& link, hipStream_t s) {
+                      int parts, const NormLink& link, int tiled, hipStream_t s) {
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)wpacked;
     const bool eight = skinny_waves(n, (k + parts - 1) / parts) == 8;
     if (swiglu) {
-        if (eight) launch_packed<8, true>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
-        else       launch_packed<4, true>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
+        if (eight) launch_packed<8, true>(out, out_dtype, xb, wb, m, n, k, parts, link, tiled, s);
+        else       launch_packed<4, true>(out, out_dtype, xb, wb, m, n, k, parts, link, tiled, s);
     } else {
-        if (eight) launch_packed<8, false>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
-        else       launch_packed<4, false>(out, out_dtype, xb, wb, m, n, k, parts, link, s);
+        if (eight) launch_packed<8, false>(out, out_dtype, xb, wb, m, n, k, parts, link, tiled, s);
+        else       launch_packed<4, false>(out, out_dtype, xb, wb, m, n, k, parts, link, tiled, s);
     }
     RI_LAUNCH_CHECK("gemm_skinny_packed_bf16");
     return 0;
 }
 
 extern "C" int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
-                                          int k, int swiglu, int parts, void* stream) {
+                                          int k, int swiglu, int parts, int tiled, void* stream) {
     RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_packed_bf16: %d rows of x, this kernel takes 1 to 16", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_packed_bf16: out dtype %d", out_dtype);
     RI_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || (!swiglu && out_dtype == RI_F32)),
                "gemm_skinny_packed_bf16: %d parts of K (more than one needs float32 sums and no activation)", parts);
+    RI_REQUIRE(!(tiled & ~(TILED_X | TILED_OUT)) && (!(tiled & TILED_OUT) || (out_dtype == RI_BF16 && parts == 1)),
+               "gemm_skinny_packed_bf16: layout flags %d (a tiled result is bfloat16 and whole)", tiled);
     NormLink link = {};
-    return packed_run(out, out_dtype, x, wpacked, m, n, k, swiglu, parts, link, (hipStream_t)stream);
+    return packed_run(out, out_dtype, x, wpacked, m, n, k, swiglu, parts, link, tiled, (hipStream_t)stream);
 }
 
 // Number of workgroups (and so of partial sums of squares per row) of a linked product with n output columns.
@@ -257,7 +272,7 @@ extern "C" int ri_gemm_skinny_packed_bf16_partials(int n) { return (n + 15) / 16
 extern "C" int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, const void* wpacked, int m,
                                                  int n, int k, int swiglu, const float* ssq_in, int n_in, float eps,
                                                  int dim, float* residual, const float* next_gain, void* xg_out,
-                                                 float* ssq_out, void* stream) {
+                                                 float* ssq_out, int tiled, void* stream) {
     RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_packed_bf16_linked: %d rows of x, this kernel takes 1 to 16", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_packed_bf16_linked: n %d, k %d (k must be a multiple of 8)", n,
                k);
@@ -268,8 +283,116 @@ extern "C" int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const
                "gemm_skinny_packed_bf16_linked: a product that feeds the residual stream needs the next gain and both "
                "outputs");
     RI_REQUIRE(residual || out, "gemm_skinny_packed_bf16_linked: no output");
+    RI_REQUIRE(!(tiled & ~(TILED_X | TILED_OUT)) && (!(tiled & TILED_OUT) || residual || out_dtype == RI_BF16),
+               "gemm_skinny_packed_bf16_linked: layout flags %d (a tiled result is bfloat16)", tiled);
     NormLink link = {ssq_in, n_in, eps, dim, residual, next_gain, (bf16_t*)xg_out, ssq_out};
-    return packed_run(out, out_dtype, x, wpacked, m, n, k, swiglu, 1, link, (hipStream_t)stream);
+    return packed_run(out, out_dtype, x, wpacked, m, n, k, swiglu, 1, link, tiled, (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------ 17 to 64 rows of x
+// The packed matrix against RT tiles of 16 rows of x: every weight fragment, read once from memory, meets
+// RT fragments of x from the L2 cache (the weights stream past that cache without settling in it, so the
+// few hundred kilobytes of x stay there).  Otherwise as the kernel above, without the norm links: steps of
+// this size keep their norm kernels.  A row's result does not depend on the number of rows: rows beyond M
+// are zero columns, and every row tile has accumulators of its own.
+template <int SK_WAVES, bool SWIGLU, typename TO, int RT>
+__global__ void __launch_bounds__(SK_WAVES * 64)
+gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked, int M,
+                       int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset) {
+    constexpr int CH = RT <= 2 ? 8 : 4;                      // MFMA steps whose loads are in flight together
+    __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][RT * 4][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, jg = lane >> 4;
+    const int nt = blockIdx.x;
+    const int kt_begin = wave * tiles_per_wave, kt_end = min(k_tiles, kt_begin + tiles_per_wave);
+    const bf16_t* wp = wpacked + ((size_t)nt * k_tiles * 64 + lane) * 8;
+    const bf16_t* up = SWIGLU ? wpacked + ((size_t)(up_tile_offset + nt) * k_tiles * 64 + lane) * 8 : nullptr;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    const bf16_t* xp[RT];
+    bool x_ok[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        x_ok[rt] = rt * 16 + i < M;
+        xp[rt] = x + (size_t)(x_ok[rt] ? rt * 16 + i : 0) * K + jg * 8;
+    }
+    floatx4 acc[RT], accu[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = accu[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int kt = kt_begin; kt < kt_end; kt += CH) {
+        Frag wf[CH], uf[CH], xf[RT][CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const bool live = kt + c < kt_end;
+            wf[c].u = live ? load_stream16(wp + (size_t)(kt + c) * 512) : zero;
+            if (SWIGLU) uf[c].u = live ? load_stream16(up + (size_t)(kt + c) * 512) : zero;
+            const bool k_ok = live && (kt + c) * 32 + jg * 8 < K;            // the packed matrix is zero beyond K; x is not padded
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                xf[rt][c].u = (k_ok && x_ok[rt]) ? *reinterpret_cast<const uint4*>(xp[rt] + (kt + c) * 32) : zero;
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt], 0, 0, 0);
+                if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt], 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            red[0][wave][rt * 4 + e][lane] = acc[rt][e];
+            if (SWIGLU) red[1][wave][rt * 4 + e][lane] = accu[rt][e];
+        }
+    __syncthreads();
+    // D[row n, column m] of a tile: lane ln of register r holds n = 4 * (ln / 16) + r, m = ln % 16
+    for (int t = threadIdx.x; t < RT * 256; t += SK_WAVES * 64) {
+        const int rt = t >> 8, ln = t & 63, r = (t >> 6) & 3;
+        const int n = nt * 16 + 4 * (ln >> 4) + r, m = rt * 16 + (ln & 15);
+        float g = 0.f, u = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < SK_WAVES; ++wv) {
+            g += red[0][wv][rt * 4 + r][ln];
+            if (SWIGLU) u += red[1][wv][rt * 4 + r][ln];
+        }
+        if (m < M && n < N) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_sk(g) * u : g);
+    }
+}
+
+template <int WAVES, bool SWIGLU, int RT>
+static void launch_mid(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, hipStream_t s) {
+    const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
+    const int tiles_per_wave = (k_tiles + WAVES - 1) / WAVES;
+    if (out_dtype == RI_F32)
+        gemm_mid_packed_kernel<WAVES, SWIGLU, float, RT><<<row_tiles, WAVES * 64, 0, s>>>(
+            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+    else
+        gemm_mid_packed_kernel<WAVES, SWIGLU, bf16_t, RT><<<row_tiles, WAVES * 64, 0, s>>>(
+            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+}
+
+extern "C" int ri_gemm_mid_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
+                                       int swiglu, void* stream) {
+    RI_REQUIRE(m > 0 && m <= 64, "gemm_mid_packed_bf16: %d rows of x, this kernel takes 1 to 64", m);
+    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_mid_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_mid_packed_bf16: out dtype %d", out_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)wpacked;
+    const bool eight = skinny_waves(n, k) == 8;
+#define RI_MID_CASE(W, SG, RT) launch_mid<W, SG, RT>(out, out_dtype, xb, wb, m, n, k, s)
+    if (m <= 32) {
+        if (swiglu) { if (eight) RI_MID_CASE(8, true, 2); else RI_MID_CASE(4, true, 2); }
+        else        { if (eight) RI_MID_CASE(8, false, 2); else RI_MID_CASE(4, false, 2); }
+    } else {
+        if (swiglu) { if (eight) RI_MID_CASE(8, true, 4); else RI_MID_CASE(4, true, 4); }
+        else        { if (eight) RI_MID_CASE(8, false, 4); else RI_MID_CASE(4, false, 4); }
+    }
+#undef RI_MID_CASE
+    RI_LAUNCH_CHECK("gemm_mid_packed_bf16");
+    return 0;
 }
 
 template <int WAVES, bool SWIGLU>

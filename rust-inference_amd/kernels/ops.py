@@ -43,14 +43,15 @@ _SIGNATURES = {
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "ri_sample_split": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                         c_float, c_float, c_void_p],
-    "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemm_mid_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
     "ri_gemm_skinny_packed_bf16_partials": [c_int],
     "ri_gemv_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
                             c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "ri_gemm_skinny_packed_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
-                                          c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+                                          c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -362,44 +363,104 @@ def pack_for_mfma(w: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
     return tiles.reshape(n16 // 16, k32 // 32, 64, 8).contiguous()
 
 
-def gemm_skinny_packed_bf16(x: torch.Tensor, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16,
-                            swiglu: bool = False, parts: int = 1) -> torch.Tensor:
-    """``x @ w.T`` for up to 16 bfloat16 rows with ``w`` packed by ``pack_for_mfma``; ``n`` is the number of
-    output columns (rows of w; of its gate half with ``swiglu``).  With ``parts > 1`` K is cut into that many
-    pieces and the result is their float32 sums ``[parts, M, n]``, for a consumer that adds them."""
+TILED_X, TILED_OUT = 1, 2
+
+
+class TiledRows:
+    """Up to 16 bfloat16 rows of ``k`` columns in the order the matrix cores take them as an operand:
+    ``data[ceil(k / 32), 64, 8]``, lane ``l`` of a tile holding row ``l % 16`` and the columns
+    ``8 * (l // 16) ..+8`` of the tile's 32.  The packed product writes its result this way for the
+    next packed product, which then loads a tile as one kilobyte in a row; rows beyond ``m`` and columns
+    beyond ``k`` are never read."""
+
+    def __init__(self, data: torch.Tensor, m: int, k: int):
+        self.data, self.shape = data, (m, k)
+        self.dtype, self.device = data.dtype, data.device
+
+    @staticmethod
+    def empty(m: int, k: int, device) -> "TiledRows":
+        if not 1 <= m <= 16:
+            raise ShapeError(f"tiled rows hold 1 to 16 rows, not {m}")
+        return TiledRows(torch.empty((-(-k // 32), 64, 8), dtype=torch.bfloat16, device=device), m, k)
+
+    def rows(self) -> torch.Tensor:
+        """The same values row-major, ``[m, k]``."""
+        m, k = self.shape
+        tiles = self.data.shape[0]
+        return self.data.view(tiles, 4, 16, 8).permute(2, 0, 1, 3).reshape(16, tiles * 32)[:m, :k].contiguous()
+
+
+def as_rows(x):
+    """A tensor for code that wants plain rows."""
+    return x.rows() if isinstance(x, TiledRows) else x
+
+
+def gemm_skinny_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16,
+                            swiglu: bool = False, parts: int = 1, tiled_out: bool = False):
+    """``x @ w.T`` for up to 16 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by
+    ``pack_for_mfma``; ``n`` is the number of output columns (rows of w; of its gate half with ``swiglu``).
+    With ``parts > 1`` K is cut into that many pieces and the result is their float32 sums ``[parts, M, n]``,
+    for a consumer that adds them.  With ``tiled_out`` the bfloat16 result comes as ``TiledRows``."""
     m, k = x.shape
     row_tiles = -(-n // 16)
     want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
     if tuple(wpacked.shape) != want:
         raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
-    out = torch.empty((m, n) if parts == 1 else (parts, m, n), dtype=out_dtype, device=x.device)
-    _call("ri_gemm_skinny_packed_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
-          _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), int(parts), _stream())
+    if tiled_out and (parts != 1 or out_dtype != torch.bfloat16):
+        raise ShapeError("a tiled result is bfloat16 and whole")
+    flags = (TILED_X if isinstance(x, TiledRows) else 0) | (TILED_OUT if tiled_out else 0)
+    xd = _dev(x.data, "x", torch.bfloat16) if isinstance(x, TiledRows) else _dev(x, "x", torch.bfloat16)
+    if tiled_out:
+        out = TiledRows.empty(m, n, x.device)
+        od = _dev(out.data, "out")
+    else:
+        out = torch.empty((m, n) if parts == 1 else (parts, m, n), dtype=out_dtype, device=x.device)
+        od = _dev(out, "out")
+    _call("ri_gemm_skinny_packed_bf16", od, code(out_dtype), xd, _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
+          int(swiglu), int(parts), flags, _stream())
     return out
 
 
 class NormedLater:
     """Rows of a residual stream whose RMSNorm is left to the product that reads them:
     ``xg = bfloat16(r * gain)`` and partial sums of ``r^2`` per row, ``[M, partials]``; the
-    normed rows are ``xg / sqrt(ssq.sum(1) / dim + eps)``."""
+    normed rows are ``xg / sqrt(ssq.sum(1) / dim + eps)``.  ``xg`` is a tensor or ``TiledRows``."""
 
-    def __init__(self, xg: torch.Tensor, ssq: torch.Tensor, eps: float, dim: int):
+    def __init__(self, xg, ssq: torch.Tensor, eps: float, dim: int):
         self.xg, self.ssq, self.eps, self.dim = xg, ssq, float(eps), int(dim)
         self.shape, self.dtype, self.device = xg.shape, xg.dtype, xg.device
 
 
+def gemm_mid_packed_bf16(x: torch.Tensor, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16,
+                         swiglu: bool = False) -> torch.Tensor:
+    """``x @ w.T`` for up to 64 bfloat16 rows with ``w`` packed by ``pack_for_mfma``: the packed product for
+    the steps of 17 to 64 tokens."""
+    m, k = x.shape
+    row_tiles = -(-n // 16)
+    want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
+    if tuple(wpacked.shape) != want:
+        raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _call("ri_gemm_mid_packed_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
+          _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), _stream())
+    return out
+
+
 def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfloat16, swiglu: bool = False,
                    residual: torch.Tensor | None = None, next_gain: torch.Tensor | None = None,
-                   next_eps: float = 0.0):
+                   next_eps: float = 0.0, tiled_out: bool = False):
     """A decode-size product that does the RMSNorm before it, the residual add and the RMSNorm's
     preparation after it, or both, in the same kernel.
 
-    ``x`` is bfloat16 rows or a ``NormedLater``; ``w`` the row-major weight (``packed`` false: up to 8
-    rows, one wavefront per weight row) or its MFMA tiles (``packed`` true: up to 16 rows).  With
-    ``residual`` (float32 ``[M, n]``, updated in place to ``residual + x @ w.T``) the result is the
-    ``NormedLater`` of the new residual for a norm with ``next_gain`` and ``next_eps``; else the product."""
+    ``x`` is bfloat16 rows (a tensor or ``TiledRows``) or a ``NormedLater``; ``w`` the row-major weight
+    (``packed`` false: up to 8 rows, one wavefront per weight row) or its MFMA tiles (``packed`` true: up to
+    16 rows).  With ``residual`` (float32 ``[M, n]``, updated in place to ``residual + x @ w.T``) the result
+    is the ``NormedLater`` of the new residual for a norm with ``next_gain`` and ``next_eps``; else the
+    product.  ``tiled_out`` (packed only) asks for the bfloat16 rows of the result as ``TiledRows``."""
     later = x if isinstance(x, NormedLater) else None
     xr = later.xg if later else x
+    if not packed:
+        xr, tiled_out = as_rows(xr), False
     m, k = xr.shape
     name = "ri_gemm_skinny_packed_bf16" if packed else "ri_gemv_bf16"
     if packed:
@@ -409,6 +470,10 @@ def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfl
         wd = _dev(w, "wpacked", torch.bfloat16)
     else:
         wd = _dev(w, "w", torch.bfloat16, (n * (2 if swiglu else 1), k))
+    x_tiled = isinstance(xr, TiledRows)
+    xd = _dev(xr.data, "x", torch.bfloat16) if x_tiled else _dev(xr, "x", torch.bfloat16, (m, k))
+    # the packed kernel takes the layouts of x and of its result as one more argument
+    layout = ((TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0),) if packed else ()
     if later is not None:
         ssq_in = _dev(later.ssq, "ssq", torch.float32, (m, later.ssq.shape[1]))
         n_in, eps, dim = later.ssq.shape[1], later.eps, later.dim
@@ -417,16 +482,19 @@ def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfl
     else:
         ssq_in, n_in, eps, dim = None, 0, 0.0, 0
     if residual is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=xr.device)
-        _call(name + "_linked", _dev(out, "out"), code(out_dtype), _dev(xr, "x", torch.bfloat16, (m, k)), wd, m, n, k,
-              int(swiglu), ssq_in, n_in, eps, dim, None, None, None, None, _stream())
+        if tiled_out and out_dtype != torch.bfloat16:
+            raise ShapeError("a tiled result is bfloat16")
+        out = TiledRows.empty(m, n, xr.device) if tiled_out else torch.empty((m, n), dtype=out_dtype, device=xr.device)
+        _call(name + "_linked", _dev(out.data if tiled_out else out, "out"), code(out_dtype), xd, wd, m, n, k,
+              int(swiglu), ssq_in, n_in, eps, dim, None, None, None, None, *layout, _stream())
         return out
     if swiglu:
         raise ShapeError("a gate|up product does not feed the residual stream")
     partials = _get("ri_gemm_skinny_packed_bf16_partials")(n) if packed else _get("ri_gemv_bf16_partials")(n, k)
-    xg = torch.empty((m, n), dtype=torch.bfloat16, device=xr.device)
+    xg = TiledRows.empty(m, n, xr.device) if tiled_out else torch.empty((m, n), dtype=torch.bfloat16, device=xr.device)
     ssq = torch.empty((m, partials), dtype=torch.float32, device=xr.device)
-    _call(name + "_linked", None, code(torch.bfloat16), _dev(xr, "x", torch.bfloat16, (m, k)), wd, m, n, k, 0,
+    _call(name + "_linked", None, code(torch.bfloat16), xd, wd, m, n, k, 0,
           ssq_in, n_in, eps, dim, _dev(residual, "residual", torch.float32, (m, n)),
-          _dev(next_gain, "next_gain", torch.float32, (n,)), _dev(xg, "xg"), _dev(ssq, "ssq"), _stream())
+          _dev(next_gain, "next_gain", torch.float32, (n,)), _dev(xg.data if tiled_out else xg, "xg"), _dev(ssq, "ssq"),
+          *layout, _stream())
     return NormedLater(xg, ssq, next_eps, n)

@@ -69,6 +69,7 @@ class GroupedQueryAttention(Mixer):
         qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
         self.w_qkv = rt.pack(rt.place_matrix(qkv))
         self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]))
+        self.takes_tiled = self.w_qkv.packed is not None       # prepared rows may come in the matrix cores' order
         self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
         self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
         self.position.bind(weights, rt)

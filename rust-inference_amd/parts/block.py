@@ -14,9 +14,10 @@ class NormLink:
     """An offer to a branch's last product: add your result into ``residual`` yourself and prepare
     the rows for ``norm``, which then needs no kernel of its own."""
 
-    def __init__(self, residual, norm):
+    def __init__(self, residual, norm, tiled: bool = False):
         self.residual, self.norm = residual, norm
         self.gain, self.eps = norm.gain, norm.eps
+        self.tiled = tiled           # the reader of the prepared rows takes them in the matrix cores' order
 
 
 class ResidualStream:
@@ -30,15 +31,16 @@ class ResidualStream:
         self.pending = None
         self.later = None            # (NormedLater, the norm it was prepared for)
         self.next_entry_norm = None  # the norm that reads the stream after the current layer, if known
+        self.next_entry_tiled = False  # and whether the part behind it reads tiled rows
 
-    def link(self, norm, act_dtype):
+    def link(self, norm, act_dtype, tiled: bool = False):
         """A ``NormLink`` for the branch that is about to run, if ``norm`` is the next reader of the
-        stream and can be left to a product."""
+        stream and can be left to a product.  ``tiled``: the part behind that norm reads tiled rows."""
         if (norm is None or not getattr(norm, "linkable", False) or self.pending is not None or self.later is not None
                 or act_dtype != torch.bfloat16 or self.sum.shape[0] > LINK_MAX_TOKENS
                 or norm.dim != self.sum.shape[1]):
             return None
-        return NormLink(self.sum, norm)
+        return NormLink(self.sum, norm, tiled)
 
     def push(self, branch) -> None:
         if self.pending is not None or self.later is not None:
@@ -91,18 +93,22 @@ class PreNormBlock:
         """The norm through which this layer first reads the stream."""
         return self.mixer_norm
 
+    def entry_takes_tiled(self) -> bool:
+        """Whether the part behind that norm reads rows in the matrix cores' order."""
+        return bool(getattr(self.mixer, "takes_tiled", False))
+
     def forward(self, stream: ResidualStream, ctx, store, page_table, act_dtype) -> None:
         # a part with ``links_norms`` takes a NormedLater as input and a NormLink for its output
         if getattr(self.mixer, "links_norms", False):
             h = stream.normed(self.mixer_norm, act_dtype, later_ok=True)
-            link = stream.link(self.feed_forward_norm, act_dtype)
+            link = stream.link(self.feed_forward_norm, act_dtype, getattr(self.feed_forward, "takes_tiled", False))
             stream.push(self.mixer.forward(h, ctx, store, page_table, link=link))
         else:
             h = stream.normed(self.mixer_norm, act_dtype)
             stream.push(self.mixer.forward(h, ctx, store, page_table))
         if getattr(self.feed_forward, "links_norms", False):
             h = stream.normed(self.feed_forward_norm, act_dtype, later_ok=True)
-            link = stream.link(stream.next_entry_norm, act_dtype)
+            link = stream.link(stream.next_entry_norm, act_dtype, stream.next_entry_tiled)
             stream.push(self.feed_forward.forward(h, ctx, link=link))
         else:
             h = stream.normed(self.feed_forward_norm, act_dtype)

@@ -137,6 +137,8 @@ class DecoderModel:
             follower = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
             entry = getattr(follower, "entry_norm", None)
             stream.next_entry_norm = entry() if entry else None
+            tiled = getattr(follower, "entry_takes_tiled", None)
+            stream.next_entry_tiled = tiled() if tiled else False
             store, table = None, None
             if run.cache is not None:
                 need = cache.needs[run.cache]

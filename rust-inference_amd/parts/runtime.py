@@ -26,6 +26,12 @@ from ..kernels import ops
 #              takes the library's own design: x staged through LDS, persistent workgroups.
 GEMV_MAX_ROWS = 2
 SKINNY_MAX_ROWS = 16
+# 17 to 64 rows: the packed kernel with two or four tiles of x to every weight tile beats the library on small
+# matrices (at 32 rows, 4096 x 1024: 5.5 us against 9.8; gate|up of 2 x 3072 x 1024 with its activation: 6.5
+# against 14.0) and loses on large ones (6144 x 4096: 23.6 against 15.1), where the rows of x, fetched by
+# every workgroup from the L2 cache, weigh as much as the weights.
+MID_MAX_ROWS = 64
+MID_MAX_BYTES = 20_000_000
 SPLIT_K = 4096
 # Which matrices get a packed copy for 3 to 16 rows (the gate|up matrix always does: its activation
 # rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
@@ -114,9 +120,10 @@ class Runtime:
         """The rows of a ``NormedLater`` for a product that cannot do the norm itself (``xg`` was
         rounded once already, so this differs from the plain norm by one more rounding)."""
         if not isinstance(x, ops.NormedLater):
-            return x
+            return ops.as_rows(x)
+        xg = ops.as_rows(x.xg)
         inv = torch.rsqrt(x.ssq.sum(1, keepdim=True) / x.dim + x.eps)
-        return (x.xg.float() * inv).to(x.xg.dtype)
+        return (xg.float() * inv).to(xg.dtype)
 
     def pack(self, w: torch.Tensor, swiglu: bool = False) -> PackedWeight:
         """A placed weight, with a packed copy where the packed kernel is the faster one for 3 to 16
@@ -127,12 +134,15 @@ class Runtime:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
 
-    def linear_packed(self, x, pw: PackedWeight, out_dtype=None, parts_ok: bool = False, link=None):
+    def linear_packed(self, x, pw: PackedWeight, out_dtype=None, parts_ok: bool = False, link=None,
+                      tiled_out: bool = False):
         """``x @ w.T`` (or ``silu(x @ gate.T) * (x @ up.T)`` for a fused gate|up weight) with the kernel
         that fits the number of rows.  With ``parts_ok`` the result may be ``[parts, M, N]`` float32, the
         sums over pieces of K, for a consumer that adds them (the residual stream's next norm).
 
-        ``x`` may be a ``NormedLater``.  With ``link`` (the residual stream's offer to the last product of
+        ``x`` may be a ``NormedLater`` or ``TiledRows``.  With ``tiled_out`` the caller takes the result as
+        ``TiledRows`` where the packed kernel makes it (3 to 16 rows): the layout the next packed product
+        reads fastest.  With ``link`` (the residual stream's offer to the last product of
         a branch) a kernel that can adds the result into the stream and prepares the next norm; the
         return value is then ``(NormedLater, norm)`` for the stream instead of a tensor."""
         out_dtype = out_dtype or self.dtype
@@ -147,18 +157,23 @@ class Runtime:
                 mine = (pw.packed, True)
             if mine is not None:
                 in_parts = mine[1] and parts_ok and pw.parts > 1        # very long rows: parts beat the link
+                tiles = mine[1] and tiled_out and out_dtype == torch.bfloat16
                 if link is not None and not pw.swiglu and not in_parts and link.residual.shape == (m, pw.n):
                     made = ops.linked_product(x, mine[0], pw.n, mine[1], residual=link.residual,
-                                              next_gain=link.gain, next_eps=link.eps)
+                                              next_gain=link.gain, next_eps=link.eps,
+                                              tiled_out=mine[1] and link.tiled)
                     return (made, link.norm)
                 if in_parts:
-                    return ops.gemm_skinny_packed_bf16(self.normed_now(x), pw.packed, pw.n, torch.float32,
-                                                       parts=pw.parts)
+                    x = self.normed_now(x) if later else x
+                    return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=pw.parts)
                 if later:
-                    return ops.linked_product(x, mine[0], pw.n, mine[1], out_dtype, swiglu=pw.swiglu)
+                    return ops.linked_product(x, mine[0], pw.n, mine[1], out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
                 if not mine[1]:
-                    return ops.gemv_bf16(x, pw.w, out_dtype, swiglu=pw.swiglu)
-                return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
+                    return ops.gemv_bf16(ops.as_rows(x), pw.w, out_dtype, swiglu=pw.swiglu)
+                return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
+            if (SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and pw.packed is not None
+                    and pw.w.shape[0] * pw.k * 2 <= MID_MAX_BYTES):
+                return ops.gemm_mid_packed_bf16(self.normed_now(x), pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
         y = self.linear(x, pw.w, None if pw.swiglu else out_dtype)
         return ops.swiglu(y) if pw.swiglu else y
 

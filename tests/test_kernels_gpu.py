@@ -454,6 +454,69 @@ def test_products_linked_to_norms(ops, packed, m, hidden, k, inter):
     close(chained.ssq.sum(1), (f64(residual) ** 2).sum(1), 1e-5, "sums of squares, second link")
 
 
+@pytest.mark.parametrize("m", [1, 17, 32, 33, 50, 64])
+@pytest.mark.parametrize("n, k", [(37, 72), (1000, 1024), (584, 12288)])
+def test_packed_product_of_17_to_64_rows(ops, m, n, k):
+    rng = np.random.default_rng(m + n)
+    x = t(rng.normal(size=(m, k)), torch.bfloat16)
+    w = t(rng.normal(size=(n, k)) / np.sqrt(k), torch.bfloat16)
+    gu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
+    pw, pgu = ops.pack_for_mfma(w), ops.pack_for_mfma(gu, swiglu=True)
+    out = ops.gemm_mid_packed_bf16(x, pw, n, torch.float32)
+    close(out, f64(x) @ f64(w).T, 2e-5, "packed product, 17 to 64 rows")
+    y = f64(x) @ f64(gu).T
+    close(ops.gemm_mid_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 1e-2,
+          "the same with swiglu")
+    # a row's result is the same whatever the number of rows, and the same as the kernel for up to 16 rows gives
+    first = min(m, 16)
+    assert torch.equal(out[:first], ops.gemm_skinny_packed_bf16(x[:first].contiguous(), pw, n, torch.float32))
+    with pytest.raises(Exception, match="1 to 64"):
+        ops.gemm_mid_packed_bf16(t(rng.normal(size=(65, k)), torch.bfloat16), pw, n)
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 13, 16])
+@pytest.mark.parametrize("hidden, k, inter", [(104, 72, 56), (4096, 4096, 1000), (584, 12288, 40)])
+def test_rows_in_the_matrix_cores_order(ops, m, hidden, k, inter):
+    """A packed product can leave its result in the order the next packed product loads as an operand, and take
+    its input in it: every such chain gives, bit for bit, what the same chain gives through plain rows."""
+    rng = np.random.default_rng(3 * m + hidden)
+    eps = 1e-5
+    x = t(rng.normal(size=(m, k)), torch.bfloat16)
+    pw_a = ops.pack_for_mfma(t(rng.normal(size=(hidden, k)) / np.sqrt(k), torch.bfloat16))
+    pw_gu = ops.pack_for_mfma(t(rng.normal(size=(2 * inter, hidden)) * (4.0 / np.sqrt(hidden)), torch.bfloat16), swiglu=True)
+    pw_b = ops.pack_for_mfma(t(rng.normal(size=(hidden, inter)) / np.sqrt(inter), torch.bfloat16))
+    gain = t(1 + 0.3 * rng.normal(size=hidden))
+    r0 = t(rng.normal(size=(m, hidden)) * 3)
+
+    # the layout itself: rows() undoes it
+    plain = ops.gemm_skinny_packed_bf16(x, pw_a, hidden)
+    tiled = ops.gemm_skinny_packed_bf16(x, pw_a, hidden, tiled_out=True)
+    assert isinstance(tiled, ops.TiledRows) and tiled.shape == (m, hidden)
+    assert torch.equal(tiled.rows(), plain)
+    # read back as an operand: with the activation, plain, and with K cut into parts
+    pw_c = ops.pack_for_mfma(t(rng.normal(size=(inter, hidden)) / np.sqrt(hidden), torch.bfloat16))
+    assert torch.equal(ops.gemm_skinny_packed_bf16(tiled, pw_gu, inter, torch.bfloat16, swiglu=True),
+                       ops.gemm_skinny_packed_bf16(plain, pw_gu, inter, torch.bfloat16, swiglu=True))
+    assert torch.equal(ops.gemm_skinny_packed_bf16(tiled, pw_c, inter), ops.gemm_skinny_packed_bf16(plain, pw_c, inter))
+    assert torch.equal(ops.gemm_skinny_packed_bf16(tiled, pw_c, inter, torch.float32, parts=2),
+                       ops.gemm_skinny_packed_bf16(plain, pw_c, inter, torch.float32, parts=2))
+    # a layer's chain of links: norm left to the products, rows handed on in either layout
+    outs = []
+    for tiles in (False, True):
+        residual = r0.clone()
+        later = ops.linked_product(x, pw_a, hidden, True, residual=residual, next_gain=gain, next_eps=eps,
+                                   tiled_out=tiles)
+        assert isinstance(later.xg, ops.TiledRows) == tiles
+        act = ops.linked_product(later, pw_gu, inter, True, torch.bfloat16, swiglu=True, tiled_out=tiles)
+        later2 = ops.linked_product(act, pw_b, hidden, True, residual=residual, next_gain=gain, next_eps=eps,
+                                    tiled_out=tiles)
+        outs.append((residual, ops.as_rows(later.xg), ops.as_rows(act), ops.as_rows(later2.xg), later.ssq, later2.ssq))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    with pytest.raises(Exception, match="tiled"):
+        ops.gemm_skinny_packed_bf16(x, pw_a, hidden, torch.float32, tiled_out=True)
+
+
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 1e-6), (torch.bfloat16, 5e-3)])
 def test_swiglu(ops, dtype, rel):
     assert f64(ops.swiglu(t([[0.0, 2.0, 3.0, 3.0]])))[0, 0] == 0.0                 # src/ops/elementwise.rs:59-70
