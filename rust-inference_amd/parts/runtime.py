@@ -8,23 +8,21 @@ from ..errors import KernelError, ShapeError
 from ..kernels import ops
 
 # Which product kernel runs, by the number of rows of x (measured on MI355X at Qwen3-8B sizes with the
-# weights streamed from HBM, every variant replayed as a graph):
-#   1-2 rows   one wavefront per weight row (gemv_bf16): 5.1 to 5.5 TB/s on the large matrices;
-#              from three rows on it is bound by its vector arithmetic.
-#   3-16 rows  the matrix-core kernel on weights packed into MFMA tiles ahead of time, where a part
-#              asked for the packed copy (the attention output matrix and the fused gate|up matrix:
-#              4.5 TB/s with the activation in the epilogue against 4.2 TB/s for the library's product
-#              plus an activation kernel; 3.0 against 2.2 TB/s on the 4096 x 4096 matrix).  Elsewhere
-#              the vendor library's product is as fast or faster (4.5 to 4.9 TB/s) and is used.
+# weights streamed from HBM through non-temporal loads, every variant replayed as a graph):
+#   1 row      one wavefront per weight row (gemv_bf16): 5.6 to 5.7 TB/s on the large matrices, 7.0 on the
+#              output head.  (At two rows the packed kernel is ahead: 471 against 438 tok/s for the model.)
+#   2-16 rows  the matrix-core kernel on weights packed into MFMA tiles ahead of time, where a part asked for
+#              the packed copy; it hands its rows to the next packed product in the operand's order
+#              (ops.TiledRows) and does the norms around it.  Where there is no packed copy the vendor
+#              library's product is used (the rule is at PACKED_MAX_BYTES below).
+#   17-64      the same kernel with two or four tiles of x, on small matrices only (MID_MAX_BYTES below).
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
-#              A form of the packed kernel for up to 64 rows (every weight tile used for four tiles of x
-#              taken from the L2 cache) was tried and lost to the library from 24 rows on at every one of
-#              these matrices (q|k|v at 32 rows: 23 us against 16 us).  So did one whose workgroups own
-#              four row tiles and all tiles of x, with K cut into parts for the narrow matrices (at 64
-#              rows: down 36 us against 39 us, o 20 against 15, gate|up 80 against 52): one workgroup a
-#              compute unit, its stream and its reduction one after the other.  Beating the library here
-#              takes the library's own design: x staged through LDS, persistent workgroups.
-GEMV_MAX_ROWS = 2
+#              Beating it on large matrices at 17 rows and more takes its own design: x staged through LDS,
+#              persistent workgroups.  Tried and dropped here: workgroups that own four row tiles and all
+#              tiles of x, with K cut into parts for the narrow matrices (at 64 rows: down 36 us against 39
+#              us, o 20 against 15, gate|up 80 against 52); x through a piece of LDS of each wavefront's
+#              own, fetched in whole cache lines (faster at 16 rows, slower at 4 and 8 and on short K).
+GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
 # 17 to 64 rows: the packed kernel with two or four tiles of x to every weight tile beats the library on small
 # matrices (at 32 rows, 4096 x 1024: 5.5 us against 9.8; gate|up of 2 x 3072 x 1024 with its activation: 6.5
@@ -112,7 +110,7 @@ class Runtime:
         if m <= GEMV_MAX_ROWS and k % 8 == 0:
             if isinstance(x, ops.NormedLater):
                 return ops.linked_product(x, w, w.shape[0], False, out_dtype)
-            return ops.gemv_bf16(x, w, out_dtype)
+            return ops.gemv_bf16(ops.as_rows(x), w, out_dtype)
         return self._library_mm(self.normed_now(x), w, out_dtype)
 
     @staticmethod
@@ -150,8 +148,7 @@ class Runtime:
         if self.dtype == torch.bfloat16 and pw.k % 8 == 0:
             later = isinstance(x, ops.NormedLater)
             mine = None
-            # two rows of the gate|up matrix: the matrix-core kernel is already ahead (40 us against 47 us)
-            if m == 1 or (m <= GEMV_MAX_ROWS and not (pw.swiglu and pw.packed is not None)):
+            if m <= GEMV_MAX_ROWS or (m <= 2 and pw.packed is None):
                 mine = (pw.w, False)
             elif m <= SKINNY_MAX_ROWS and pw.packed is not None:
                 mine = (pw.packed, True)
