@@ -128,6 +128,14 @@ class Cache:
             raise native.fail()
         return n
 
+    def longest(self, slots) -> int:
+        """The length of the longest of these sequences."""
+        s = np.asarray(slots, dtype=np.int32)
+        n = self._lib.ri_cache_longest(self.core.handle, s.ctypes.data, len(s))
+        if n < 0:
+            raise native.fail()
+        return n
+
     # ---- steps
     def reserve(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         """Map pages for the tokens a step is about to write.  Either every sequence

@@ -26,6 +26,7 @@ _SIGNATURES = {
     "ri_cache_check_held": ([c_void_p, c_int], c_int),
     "ri_cache_free_slots": ([c_void_p], c_int),
     "ri_cache_length": ([c_void_p, c_int], c_long),
+    "ri_cache_longest": ([c_void_p, c_void_p, c_int], c_long),
     "ri_cache_reserve": ([c_void_p, c_void_p, c_void_p, c_int], c_int),
     "ri_cache_commit": ([c_void_p, c_void_p, c_void_p, c_int], c_int),
     "ri_cache_check": ([c_void_p], c_int),

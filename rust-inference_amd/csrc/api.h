@@ -171,6 +171,7 @@ int ri_cache_is_held(void* cache, int slot);                             // 0 or
 int ri_cache_check_held(void* cache, int slot);
 int ri_cache_free_slots(void* cache);                                    // the count
 long ri_cache_length(void* cache, int slot);                             // the length, or -1
+long ri_cache_longest(void* cache, const int32_t* slots, int n);        // the longest of them, or -1
 int ri_cache_reserve(void* cache, const int32_t* slots, const int32_t* counts, int n);     // all or nothing
 int ri_cache_commit(void* cache, const int32_t* slots, const int32_t* counts, int n);
 int ri_cache_check(void* cache);

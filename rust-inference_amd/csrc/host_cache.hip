@@ -208,6 +208,17 @@ extern "C" long ri_cache_length(void* cache, int slot) {
     return (long)c->lengths[slot];
 }
 
+// The longest of these sequences, or -1 (one call for a whole batch instead of one per sequence).
+extern "C" long ri_cache_longest(void* cache, const int32_t* slots, int n) {
+    CacheCore* c = (CacheCore*)cache;
+    long longest = 0;
+    for (int i = 0; i < n; ++i) {
+        if (c->check_held(slots[i])) return -1;
+        longest = std::max(longest, (long)c->lengths[slots[i]]);
+    }
+    return longest;
+}
+
 // Maps pages for the tokens a step is about to write: either every sequence gets its pages in every
 // pool, or the cache is left as it was.
 extern "C" int ri_cache_reserve(void* cache, const int32_t* slots, const int32_t* counts, int n) {

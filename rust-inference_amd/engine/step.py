@@ -48,6 +48,13 @@ def wanted_indices(n: int, want: Want) -> list[int]:
     return out
 
 
+def _one_token_wanted(e: StepEntry) -> bool:
+    """One token whose logits are wanted: the entry of a decode step."""
+    if len(e.tokens) != 1:
+        return False
+    return e.want == "last" or e.want == "all" or (not isinstance(e.want, str) and wanted_indices(1, e.want) == [0])
+
+
 def plan_step(entries: Sequence[StepEntry], lengths: Sequence[int], vocab_size: int):
     """The host-side layout of a step: flat tokens, each token's sequence and position, where
     each sequence starts among them, and the wanted rows, as int32 arrays.  ``lengths[i]`` is
@@ -197,7 +204,7 @@ class Engine:
         the entries and of each entry's wanted places.  (With graphs the logits of a decode step
         live in the graph's own buffer and are overwritten by the next decode step of that size.)"""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
-        if self.use_graphs and all(len(e.tokens) == 1 and wanted_indices(1, e.want) == [0] for e in entries):
+        if self.use_graphs and entries and all(_one_token_wanted(e) for e in entries):
             return self._graph_step(entries)
         ctx = self.build_context(entries)
         logits = self.model.forward(ctx, self.cache)
@@ -212,7 +219,8 @@ class Engine:
         # gets the next graph when its longest sequence grows past the bound (capturing one costs about
         # as much as two or three steps).  Finer bounds were tried and gained nothing: the workgroups of
         # the empty chunks come last in the grid and cost little there.
-        longest = max(self.cache.length(e.slot) for e in entries) + 1
+        slots = np.fromiter((e.slot for e in entries), dtype=np.int32, count=batch)
+        longest = self.cache.longest(slots) + 1
         bound = min(self.cache.max_seq_len, max(1024, 1 << (longest - 1).bit_length()))
         dg = self._graphs.get((batch, bound))
         if dg is None:
@@ -220,21 +228,50 @@ class Engine:
             width = self.cache.max_pages_per_slot
             need = 7 * (batch + 5) + len(self.cache.groups) * (batch * width + 4)
             dg.staging = _Staging(need, self.device)
+        if dg.graph is not None:
+            return self._replay(dg, entries, slots)
         # the layout of a decode step depends on the batch size alone, so the buffers a captured
         # graph reads are refilled in place
         ctx = self.build_context(entries, staging=dg.staging, full_width=True, grid_len=bound)
-        if dg.graph is None:
-            # once eagerly (libraries set themselves up outside the capture), then capture; writing
-            # the same keys and values to the same places twice changes nothing, and per-sequence
-            # state is put back to where it was before the rehearsal
-            saved = self.cache.snapshot_state()
-            self.model.forward(ctx, self.cache)
-            self.cache.restore_state(saved)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                dg.logits = self.model.forward(ctx, self.cache)
-            dg.graph, dg.ctx = graph, ctx
+        # once eagerly (libraries set themselves up outside the capture), then capture; writing
+        # the same keys and values to the same places twice changes nothing, and per-sequence
+        # state is put back to where it was before the rehearsal
+        saved = self.cache.snapshot_state()
+        self.model.forward(ctx, self.cache)
+        self.cache.restore_state(saved)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            dg.logits = self.model.forward(ctx, self.cache)
+        dg.graph, dg.ctx = graph, ctx
         dg.graph.replay()
         self.cache.commit(ctx.slot_list, ctx.new_counts)
+        return dg.logits
+
+    def _replay(self, dg: _DecodeGraph, entries: Sequence[StepEntry], slots: np.ndarray) -> torch.Tensor:
+        """A decode step whose graph exists: reserve the pages, write the step's layout into the buffers the
+        graph reads, replay.  The same layout as ``build_context`` makes, without the objects a first run
+        needs (at 64 sequences the host's share of a step is a few per cent of it)."""
+        cache, batch = self.cache, dg.batch
+        tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=batch)
+        vocab = self.model.spec.vocab_size
+        if tokens.min() < 0 or tokens.max() >= vocab:
+            bad = int(tokens[(tokens < 0) | (tokens >= vocab)][0])
+            raise ShapeError(f"token id {bad} is outside the vocabulary of {vocab}")
+        tokens = tokens.astype(np.int32)
+        ones = np.ones(batch, dtype=np.int32)
+        want = np.arange(batch, dtype=np.int32)
+        cache.reserve(slots, ones)
+        width, groups = cache.max_pages_per_slot, len(cache.groups)
+        capacity = 3 * (batch + 4) + (batch + 5) + 2 * (batch + 4) + (batch + 4) + groups * (batch * width + 4)
+        words = dg.staging.begin(capacity)
+        offsets = np.empty(7 + groups, dtype=np.int64)
+        used = cache_native.lib().ri_cache_plan_step(
+            cache.core.handle, slots.ctypes.data, ones.ctypes.data, batch, tokens.ctypes.data, want.ctypes.data, batch,
+            vocab, width, words.ctypes.data, capacity, offsets.ctypes.data)
+        if used < 0:
+            raise ShapeError(cache_native.lib().ri_last_error().decode())
+        dg.staging.upload(used)
+        dg.graph.replay()
+        cache.commit(slots, ones)
         return dg.logits
