@@ -31,7 +31,7 @@ SKINNY_MAX_ROWS = 16
 MID_MAX_ROWS = 64
 MID_MAX_BYTES = 20_000_000
 SPLIT_K = 4096
-# Which matrices get a packed copy for 3 to 16 rows (the gate|up matrix always does: its activation
+# Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation
 # rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
 #   4096 x 1024 (8 MB) 4.1 : 7.5     1024 x 3072 (6 MB) 7.0 : 11.9    2048 x 2048 (8 MB) 5.3 : 11.0
 #   4096 x 4096 (34 MB) 9.2 : 15.3   6144 x 4096 (50 MB) 15.4 : 15.5  2560 x 9728 (50 MB) 19.2 : 18.3
@@ -124,7 +124,7 @@ class Runtime:
         return (xg.float() * inv).to(xg.dtype)
 
     def pack(self, w: torch.Tensor, swiglu: bool = False) -> PackedWeight:
-        """A placed weight, with a packed copy where the packed kernel is the faster one for 3 to 16
+        """A placed weight, with a packed copy where the packed kernel is the faster one for 2 to 16
         rows (bfloat16 compute only)."""
         n, k = w.shape
         pays = swiglu or _packed_pays(n, k)
@@ -139,7 +139,7 @@ class Runtime:
         sums over pieces of K, for a consumer that adds them (the residual stream's next norm).
 
         ``x`` may be a ``NormedLater`` or ``TiledRows``.  With ``tiled_out`` the caller takes the result as
-        ``TiledRows`` where the packed kernel makes it (3 to 16 rows): the layout the next packed product
+        ``TiledRows`` where the packed kernel makes it (2 to 16 rows): the layout the next packed product
         reads fastest.  With ``link`` (the residual stream's offer to the last product of
         a branch) a kernel that can adds the result into the stream and prepares the next norm; the
         return value is then ``(NormedLater, norm)`` for the stream instead of a tensor."""

@@ -149,7 +149,7 @@ def test_prenorm_block_leaves_norms_to_the_products(rows):
     stream.push(ff.forward(stream.normed(norms[0], torch.bfloat16), None, link=link))
     h1 = plain_branch(h0, "a")
     if rows <= 16:                                # the down product of such steps takes the link (a small matrix:
-        assert stream.later is not None and stream.pending is None      # it has a packed copy for 3 to 16 rows)
+        assert stream.later is not None and stream.pending is None      # it has a packed copy for 2 to 16 rows)
         assert rel_to_max(f64(stream.sum), h1) < 5e-3
     assert stream.link(norms[2], torch.bfloat16) is None          # something waits: no second offer
     x = stream.normed(norms[1], torch.bfloat16, later_ok=True)
