@@ -172,6 +172,36 @@ def test_prenorm_block_leaves_norms_to_the_products(rows):
     assert rel_to_max(f64(x), P.rms_norm(h1[-1:], w64["b"], eps)) < 1e-2
 
 
+def test_tiled_rows_reach_every_kind_of_product():
+    """Rows in the matrix cores' order may meet a product that has no packed kernel for them (a matrix
+    without a packed copy, the one-row kernel, the library): it gets plain rows and gives the same result."""
+    from rust_inference_amd.kernels import ops
+    from rust_inference_amd.parts.runtime import PackedWeight, Runtime
+    rt = Runtime(DEV, torch.bfloat16)
+    rng = np.random.default_rng(41)
+    n, k = 96, 160
+    w = t(rng.normal(size=(n, k)) / np.sqrt(k), torch.bfloat16)
+    plain_w, packed_w = PackedWeight(w, None, False), PackedWeight(w, ops.pack_for_mfma(w), False)
+    maker = ops.pack_for_mfma(t(np.eye(k), torch.bfloat16))            # x itself comes out of a product, tiled
+    for m in (1, 2, 5, 16):
+        x = t(rng.normal(size=(m, k)), torch.bfloat16)
+        xt = ops.gemm_skinny_packed_bf16(x, maker, k, tiled_out=True)
+        assert torch.equal(xt.rows(), x)
+        want = f64(x) @ f64(w).T
+        for pw in (plain_w, packed_w):
+            assert rel_to_max(f64(rt.linear_packed(xt, pw)), want) < 1e-2
+            assert torch.equal(rt.linear_packed(xt, pw), rt.linear_packed(x, pw))
+        # a prepared norm whose rows are tiled, read by a product that cannot take them so
+        gain = t(1 + 0.2 * rng.normal(size=k))
+        residual = t(rng.normal(size=(m, k)))
+        later = ops.linked_product(x, maker, k, True, residual=residual, next_gain=gain, next_eps=1e-5, tiled_out=True)
+        assert isinstance(later.xg, ops.TiledRows)
+        normed = P.rms_norm(f64(residual), f64(gain), 1e-5)
+        assert rel_to_max(f64(rt.linear_packed(later, plain_w, out_dtype=torch.float32)), normed @ f64(w).T) < 1e-2
+        assert rel_to_max(f64(rt.linear_packed(later, packed_w, out_dtype=torch.float32)), normed @ f64(w).T) < 1e-2
+        assert rel_to_max(f64(rt.normed_now(later)), normed) < 1e-2
+
+
 # ------------------------------------------------------------------------------------------------ the toy architecture
 TOY = {"architectures": ["ToyMixForCausalLM"], "vocab_size": 130, "hidden_size": 48, "inter": 80, "heads": 4,
        "kv_heads": 2, "head_dim": 16, "window": 24, "eps": 1e-5, "theta": 10000.0, "experts": 4, "period": 37}
