@@ -16,8 +16,9 @@ from .spec import PartSpec
 
 # Up to this many sequences a decode step norms and rotates q and k inside the attention kernel (one
 # launch less per layer); beyond it the many workgroups each repeating that work cost more than the
-# launch (measured at 64 sequences of 2,048 tokens: 140 us against 111 + 6 us).
-FUSED_DECODE_MAX_SEQS = 16
+# launch (measured at 64 sequences of 2,048 tokens: 140 us against 111 + 6 us; at 24 and 32 sequences the
+# one kernel is still ahead, by 1% of the step).
+FUSED_DECODE_MAX_SEQS = 32
 
 
 @register_part("mixer", "attention")
