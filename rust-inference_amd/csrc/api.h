@@ -22,7 +22,7 @@ int ri_embed_gather(float* out, const void* table, int table_dtype, const int32_
 // pending may be `parts` tensors [parts][total_rows][dim] that are added one after the other.
 int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype, int parts,
                    int total_rows, const float* gain, float eps, const int32_t* rows, int n_rows, int dim,
-                   void* stream);
+                   int tiled, void* stream);
 
 // Plain residual add on gathered rows, no norm: out[row] = residual[src] + pending[src], float32.
 int ri_add_rows(float* out, const float* residual, const void* pending, int pending_dtype,
@@ -65,8 +65,10 @@ int ri_attention_decode_chunks(int max_len);
 int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride, const void* k_pages,
                              const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
                              const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,
-                             int kv_heads, int head_dim, int page_size, int window, float scale, void* stream);
+                             int kv_heads, int head_dim, int page_size, int window, float scale, int tiled_out, void* stream);
 
+// tiled_out (both decode forms): the result [seqs, heads * head_dim] is written in the matrix cores' operand order
+// (see tiled_at in common.h) for the packed product that reads it.
 // The decode attention of a layer from the raw fused projection (which is not changed): per-head norm (gains
 // may be NULL) and rotation (inv_freq may be NULL) of the new token's q and k, its k and v into their pages
 // and attention in chunks of 256 keys in one kernel, the join in a second.
@@ -74,7 +76,7 @@ int ri_attention_decode_fused_bf16(void* out, float* workspace, const void* qkv,
                                    const float* k_gain, float eps, const float* inv_freq, void* k_pages,
                                    void* v_pages, const int32_t* tok_pos, const int32_t* page_table, int table_width,
                                    int seqs, int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
-                                   int window, float scale, void* stream);
+                                   int window, float scale, int tiled_out, void* stream);
 
 // out[M, N] (float32) = x[M, K] (float32) . w[N, K]^T, w float32 or bfloat16; true 32-bit arithmetic.
 int ri_gemm_f32(float* out, const float* x, const void* w, int w_dtype, int m, int n, int k, void* stream);
@@ -103,7 +105,7 @@ int ri_gemm_skinny_packed_bf16(void* out, int out_dtype, const void* x, const vo
 // The same product for 17 to 64 rows of x (it takes fewer too): every weight fragment meets two or four
 // tiles of 16 rows of x.  No parts, no links.
 int ri_gemm_mid_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
-                            int swiglu, void* stream);
+                            int swiglu, int tiled, void* stream);
 
 // The two decode-size products linked to the RMSNorms around them, so that those need no kernels of their
 // own.  W . norm(r) with norm(r) = r * inv * g equals inv * (W . (r * g)), inv = 1 / sqrt(mean(r^2) + eps):

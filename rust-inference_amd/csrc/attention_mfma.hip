@@ -453,7 +453,7 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 template <int DH, int PB>
 __global__ void __launch_bounds__(DH * PB)
 attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
-                        int heads, int window, int max_chunks) {
+                        int heads, int window, int max_chunks, int tiled) {
     __shared__ float part_o[JOIN_PARTS][DH];
     __shared__ float part_ml[JOIN_PARTS][2];
     const int b = blockIdx.x, h = blockIdx.y;                       // token b is sequence b's one new token
@@ -478,7 +478,7 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
             l += base[c * (DH + 2) + DH + 1] * f;
         }
         if (parts == 1) {                                           // the whole workgroup is here or nowhere
-            out[((long)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+            out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
             return;
         }
         part_o[p][d] = acc;
@@ -499,17 +499,17 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
         acc += part_o[p][d] * f;
         l += part_ml[p][1] * f;
     }
-    out[((long)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+    out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
 }
 
 template <int DH>
 static void launch_join(bf16_t* out, const float* ws, const int32_t* tok_pos, int seqs, int heads, int window,
-                        int max_chunks, hipStream_t s) {
+                        int max_chunks, int tiled, hipStream_t s) {
     if (max_chunks <= JOIN_SERIAL)
-        attn_decode_join_kernel<DH, 1><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window, max_chunks);
+        attn_decode_join_kernel<DH, 1><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window, max_chunks, tiled);
     else
         attn_decode_join_kernel<DH, JOIN_PARTS><<<dim3(seqs, heads), DH * JOIN_PARTS, 0, s>>>(out, ws, tok_pos, heads,
-                                                                                           window, max_chunks);
+                                                                                           window, max_chunks, tiled);
 }
 
 // ------------------------------------------------------------------ decode, everything in one kernel
@@ -740,8 +740,9 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
                                         const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
                                         const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
                                         int max_chunks, int heads, int kv_heads, int head_dim, int page_size,
-                                        int window, float scale, void* stream) {
+                                        int window, float scale, int tiled_out, void* stream) {
     if (check_common("attention_decode_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width)) return 1;
+    RI_REQUIRE(!tiled_out || (seqs <= 64 && head_dim % 32 == 0), "attention_decode_bf16: tiled rows are at most 64 (%d)", seqs);
     const int group = heads / kv_heads;
     RI_REQUIRE(group <= 16, "attention_decode_bf16: %d query heads per kv head (at most 16)", group);
     RI_REQUIRE(seqs > 0 && max_chunks > 0 && max_chunks <= 65535 && heads <= 65535,
@@ -754,7 +755,7 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
         attn_decode_mfma_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                           \
             workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
             tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks);                   \
-        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, max_chunks, s);                    \
+        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, max_chunks, tiled_out, s);                    \
         break;
     switch (head_dim) {
         RI_DECODE_CASE(32)
@@ -773,9 +774,10 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
                                               const float* inv_freq, void* k_pages, void* v_pages,
                                               const int32_t* tok_pos, const int32_t* page_table, int table_width,
                                               int seqs, int max_chunks, int heads, int kv_heads, int head_dim,
-                                              int page_size, int window, float scale, void* stream) {
+                                              int page_size, int window, float scale, int tiled_out, void* stream) {
     if (check_common("attention_decode_fused_bf16", heads, kv_heads, head_dim, page_size, q_stride, table_width))
         return 1;
+    RI_REQUIRE(!tiled_out || (seqs <= 64 && head_dim % 32 == 0), "attention_decode_fused_bf16: tiled rows are at most 64 (%d)", seqs);
     const int group = heads / kv_heads;
     RI_REQUIRE(group <= 16, "attention_decode_fused_bf16: %d query heads per kv head (at most 16)", group);
     RI_REQUIRE(seqs > 0 && max_chunks > 0 && max_chunks <= 65535 && heads <= 65535,
@@ -790,7 +792,7 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
         attn_decode_fused_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                          \
             workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq, (bf16_t*)k_pages,             \
             (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks); \
-        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, max_chunks, s);                    \
+        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, max_chunks, tiled_out, s);                    \
         break;
     switch (head_dim) {
         RI_FUSED_CASE(32)

@@ -28,6 +28,18 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return *reinterpret_cast<const uint32_t*>(&v);
 }
 
+// Rows of activations in the order the matrix cores take them as a B operand: tiles of 16 rows x 32 columns,
+// each 64 lanes x 8 elements (lane l: row l % 16, columns 8 * (l / 16) ..+8 of the tile), the tiles of a row
+// tile one after the other, row tile after row tile.  A product or a norm that writes its result this way
+// spares the product after it loads that touch sixteen cache lines for half of each: a tile is one kilobyte
+// in a row.  k_tiles is the number of column tiles, ceil(columns / 32).  TILED_X: x lies so; TILED_OUT: the
+// bfloat16 result is to lie so.
+#define TILED_X 1
+#define TILED_OUT 2
+__device__ __forceinline__ size_t tiled_at(int m, int n, int k_tiles) {
+    return (((size_t)(m >> 4) * k_tiles + (n >> 5)) * 64 + (m & 15) + 16 * ((n & 31) >> 3)) * 8 + (n & 7);
+}
+
 // A 16-byte load of data that is read once (a weight matrix streaming through): marked non-temporal, so
 // that it does not displace what the caches hold to be used again.
 __device__ __forceinline__ uint4 load_stream16(const void* p) {

@@ -24,17 +24,6 @@ union Frag {
 
 __device__ __forceinline__ float silu_sk(float z) { return z / (1.0f + expf(-z)); }
 
-// Up to 16 rows of activations in the order the matrix cores take them as a B operand: tiles of 32 columns,
-// each 64 lanes x 8 elements, lane l holding row l % 16 and the columns 8 * (l / 16) ..+8 of the tile.  A
-// product that writes its result this way spares the next one loads that touch sixteen cache lines for
-// half of each: the tile is one kilobyte in a row.  TILED_X: x lies so; TILED_OUT: the bfloat16 result
-// (out, or a link's xg_out) is to lie so.
-#define TILED_X 1
-#define TILED_OUT 2
-__device__ __forceinline__ size_t tiled_at(int m, int n) {
-    return ((size_t)(n >> 5) * 64 + (m & 15) + 16 * ((n & 31) >> 3)) * 8 + (n & 7);
-}
-
 template <int SK_WAVES, bool SWIGLU, typename TO>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N,
@@ -201,11 +190,11 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
                 const size_t at = (size_t)m * N + n;
                 v += res_pre;
                 link.residual[at] = v;                   // this element belongs to this thread alone
-                link.xg_out[(tiled & TILED_OUT) ? tiled_at(m, n) : at] = f32_to_bf16(v * gain_pre);
+                link.xg_out[(tiled & TILED_OUT) ? tiled_at(m, n, (N + 31) / 32) : at] = f32_to_bf16(v * gain_pre);
             }
             sq_lds[m][nl] = ok ? v * v : 0.f;
         } else if (ok) {
-            from_f32(out + ((tiled & TILED_OUT) ? tiled_at(m, n) : (size_t)m * N + n), v);
+            from_f32(out + ((tiled & TILED_OUT) ? tiled_at(m, n, (N + 31) / 32) : (size_t)m * N + n), v);
         }
     }
     if (link.residual) {                                 // the workgroup's share of every row's sum of squares
@@ -300,7 +289,7 @@ extern "C" int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const
 template <int SK_WAVES, bool SWIGLU, typename TO, int RT>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked, int M,
-                       int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset) {
+                       int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset, int tiled) {
     constexpr int CH = RT <= 2 ? 8 : 4;                      // MFMA steps whose loads are in flight together
     __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][RT * 4][64];
     const int lane = threadIdx.x & 63;
@@ -316,8 +305,10 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         x_ok[rt] = rt * 16 + i < M;
-        xp[rt] = x + (size_t)(x_ok[rt] ? rt * 16 + i : 0) * K + jg * 8;
+        xp[rt] = (tiled & TILED_X) ? x + ((size_t)rt * k_tiles * 64 + lane) * 8
+                                   : x + (size_t)(x_ok[rt] ? rt * 16 + i : 0) * K + jg * 8;
     }
+    const int x_step = (tiled & TILED_X) ? 512 : 32;         // elements from one step's fragment to the next
     floatx4 acc[RT], accu[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = accu[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -331,7 +322,7 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
             const bool k_ok = live && (kt + c) * 32 + jg * 8 < K;            // the packed matrix is zero beyond K; x is not padded
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
-                xf[rt][c].u = (k_ok && x_ok[rt]) ? *reinterpret_cast<const uint4*>(xp[rt] + (kt + c) * 32) : zero;
+                xf[rt][c].u = (k_ok && x_ok[rt]) ? *reinterpret_cast<const uint4*>(xp[rt] + (size_t)(kt + c) * x_step) : zero;
         }
 #pragma unroll
         for (int c = 0; c < CH; ++c)
@@ -359,32 +350,36 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
             g += red[0][wv][rt * 4 + r][ln];
             if (SWIGLU) u += red[1][wv][rt * 4 + r][ln];
         }
-        if (m < M && n < N) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_sk(g) * u : g);
+        if (m < M && n < N)
+            from_f32(out + ((tiled & TILED_OUT) ? tiled_at(m, n, (N + 31) / 32) : (size_t)m * N + n), SWIGLU ? silu_sk(g) * u : g);
     }
 }
 
 template <int WAVES, bool SWIGLU, int RT>
-static void launch_mid(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, hipStream_t s) {
+static void launch_mid(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, int tiled,
+                       hipStream_t s) {
     const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
     const int tiles_per_wave = (k_tiles + WAVES - 1) / WAVES;
     if (out_dtype == RI_F32)
         gemm_mid_packed_kernel<WAVES, SWIGLU, float, RT><<<row_tiles, WAVES * 64, 0, s>>>(
-            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, tiled);
     else
         gemm_mid_packed_kernel<WAVES, SWIGLU, bf16_t, RT><<<row_tiles, WAVES * 64, 0, s>>>(
-            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles);
+            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, tiled);
 }
 
 extern "C" int ri_gemm_mid_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
-                                       int swiglu, void* stream) {
+                                       int swiglu, int tiled, void* stream) {
     RI_REQUIRE(m > 0 && m <= 64, "gemm_mid_packed_bf16: %d rows of x, this kernel takes 1 to 64", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_mid_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_mid_packed_bf16: out dtype %d", out_dtype);
+    RI_REQUIRE(!(tiled & ~(TILED_X | TILED_OUT)) && (!(tiled & TILED_OUT) || out_dtype == RI_BF16),
+               "gemm_mid_packed_bf16: layout flags %d (a tiled result is bfloat16)", tiled);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)wpacked;
     const bool eight = skinny_waves(n, k) == 8;
-#define RI_MID_CASE(W, SG, RT) launch_mid<W, SG, RT>(out, out_dtype, xb, wb, m, n, k, s)
+#define RI_MID_CASE(W, SG, RT) launch_mid<W, SG, RT>(out, out_dtype, xb, wb, m, n, k, tiled, s)
     if (m <= 32) {
         if (swiglu) { if (eight) RI_MID_CASE(8, true, 2); else RI_MID_CASE(4, true, 2); }
         else        { if (eight) RI_MID_CASE(8, false, 2); else RI_MID_CASE(4, false, 2); }

@@ -80,7 +80,7 @@ template <typename TP, typename TO, int VPT>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const TP* __restrict__ pending,
                        int parts, size_t part_stride, const float* __restrict__ gain, float eps,
-                       const int32_t* __restrict__ rows, int dim) {
+                       const int32_t* __restrict__ rows, int dim, int tiled) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[row] : row) * dim;
@@ -115,8 +115,8 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
         const int d = (i * 256 + threadIdx.x) * 4;
-        if (d < dim)
-            store4(o + d, make_float4(v[i].x * inv * g[i].x, v[i].y * inv * g[i].y, v[i].z * inv * g[i].z,
+        if (d < dim)                                         // four columns of one chunk of eight either way
+            store4(tiled ? out + tiled_at(row, d, (dim + 31) / 32) : o + d, make_float4(v[i].x * inv * g[i].x, v[i].y * inv * g[i].y, v[i].z * inv * g[i].z,
                                       v[i].w * inv * g[i].w));
     }
 }
@@ -124,44 +124,48 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
 template <typename TP, typename TO>
 static void launch_add_rmsnorm_typed(TO* out, float* residual, const TP* pending, int parts, size_t ps,
                                      const float* gain, float eps, const int32_t* rows, int n_rows, int dim,
-                                     hipStream_t s) {
+                                     int tiled, hipStream_t s) {
     if (dim % 4 == 0 && dim <= 1024)
-        add_rmsnorm_vec_kernel<TP, TO, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
     else if (dim % 4 == 0 && dim <= 2048)
-        add_rmsnorm_vec_kernel<TP, TO, 2><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 2><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
     else if (dim % 4 == 0 && dim <= 4096)
-        add_rmsnorm_vec_kernel<TP, TO, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
     else if (dim % 4 == 0 && dim <= 8192)
-        add_rmsnorm_vec_kernel<TP, TO, 8><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
+        add_rmsnorm_vec_kernel<TP, TO, 8><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
     else
         add_rmsnorm_kernel<TP, TO><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
 }
 
 template <typename TP>
 static void launch_add_rmsnorm(void* out, int out_dtype, float* residual, const TP* pending, int parts, size_t ps,
-                               const float* gain, float eps, const int32_t* rows, int n_rows, int dim, hipStream_t s) {
+                               const float* gain, float eps, const int32_t* rows, int n_rows, int dim, int tiled,
+                               hipStream_t s) {
     if (out_dtype == RI_F32)
-        launch_add_rmsnorm_typed<TP, float>((float*)out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, s);
+        launch_add_rmsnorm_typed<TP, float>((float*)out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, 0, s);
     else
         launch_add_rmsnorm_typed<TP, bf16_t>((bf16_t*)out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim,
-                                             s);
+                                             tiled, s);
 }
 
 extern "C" int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pending, int pending_dtype,
                               int parts, int total_rows, const float* gain, float eps, const int32_t* rows, int n_rows,
-                              int dim, void* stream) {
+                              int dim, int tiled, void* stream) {
     RI_REQUIRE(n_rows > 0 && dim > 0, "add_rmsnorm: rows %d, dim %d", n_rows, dim);
     RI_REQUIRE(parts >= 1 && parts <= 64 && total_rows >= 1, "add_rmsnorm: %d parts of %d rows", parts, total_rows);
     const size_t ps = (size_t)total_rows * dim;
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "add_rmsnorm: out dtype %d", out_dtype);
     RI_REQUIRE(pending_dtype == RI_F32 || pending_dtype == RI_BF16, "add_rmsnorm: pending dtype %d", pending_dtype);
+    RI_REQUIRE(!tiled || (out_dtype == RI_BF16 && dim % 4 == 0 && dim <= 8192 && n_rows <= 64),
+               "add_rmsnorm: tiled rows are bfloat16, at most 64, of a multiple of 4 up to 8192 elements (%d of %d)",
+               n_rows, dim);
     hipStream_t s = (hipStream_t)stream;
     if (pending_dtype == RI_F32)
         launch_add_rmsnorm<float>(out, out_dtype, residual, (const float*)pending, parts, ps, gain, eps, rows, n_rows,
-                                  dim, s);
+                                  dim, tiled, s);
     else
         launch_add_rmsnorm<bf16_t>(out, out_dtype, residual, (const bf16_t*)pending, parts, ps, gain, eps, rows, n_rows,
-                                   dim, s);
+                                   dim, tiled, s);
     RI_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }

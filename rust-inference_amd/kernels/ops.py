@@ -21,7 +21,7 @@ _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 _SIGNATURES = {
     "ri_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_add_rmsnorm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_int,
-                       c_int, c_void_p],
+                       c_int, c_int, c_void_p],
     "ri_add_rows": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_qk_norm_rope_kv_write": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p,
                                  c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -31,10 +31,10 @@ _SIGNATURES = {
     "ri_attention_prefill_bf16": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "ri_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "ri_attention_decode_fused_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float,
                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                       c_int, c_int, c_int, c_int, c_float, c_void_p],
+                                       c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_skinny_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -44,7 +44,7 @@ _SIGNATURES = {
     "ri_sample_split": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                         c_float, c_float, c_void_p],
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "ri_gemm_mid_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemm_mid_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
     "ri_gemm_skinny_packed_bf16_partials": [c_int],
@@ -121,10 +121,11 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
 
 
 def add_rmsnorm(residual: torch.Tensor, pending, gain: torch.Tensor, eps: float, out_dtype,
-                rows: torch.Tensor | None = None) -> torch.Tensor:
+                rows: torch.Tensor | None = None, tiled: bool = False):
     """``residual += pending`` (in place, when ``rows`` is None) and the RMSNorm of the sum.
     With ``rows`` the sum and norm are taken of those rows only and nothing is written back.
-    ``pending`` may be ``[parts, T, dim]``: the parts of a product split along K, added in order."""
+    ``pending`` may be ``[parts, T, dim]``: the parts of a product split along K, added in order.
+    With ``tiled`` the normed rows (bfloat16, at most 64) come as ``TiledRows``."""
     t, dim = residual.shape
     n = t if rows is None else rows.shape[0]
     parts = 1
@@ -134,10 +135,13 @@ def add_rmsnorm(residual: torch.Tensor, pending, gain: torch.Tensor, eps: float,
             raise ShapeError(f"pending parts are {list(pending.shape)}, the stream is {[t, dim]}")
     elif pending is not None and tuple(pending.shape) != (t, dim):
         raise ShapeError(f"pending is {list(pending.shape)}, the stream is {[t, dim]}")
-    out = torch.empty((n, dim), dtype=out_dtype, device=residual.device)
-    _call("ri_add_rmsnorm", _dev(out, "out"), code(out_dtype), _dev(residual, "residual", torch.float32),
+    out = TiledRows.empty(n, dim, residual.device) if tiled else torch.empty((n, dim), dtype=out_dtype,
+                                                                             device=residual.device)
+    _call("ri_add_rmsnorm", _dev(out.data if tiled else out, "out"), code(out_dtype),
+          _dev(residual, "residual", torch.float32),
           _opt(pending, "pending"), code(pending.dtype) if pending is not None else F32, parts, t,
-          _dev(gain, "gain", torch.float32, (dim,)), float(eps), _opt(rows, "rows", torch.int32), n, dim, _stream())
+          _dev(gain, "gain", torch.float32, (dim,)), float(eps), _opt(rows, "rows", torch.int32), n, dim, int(tiled),
+          _stream())
     return out
 
 
@@ -270,28 +274,32 @@ def attention_prefill_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_tabl
 
 
 def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_len: int,
-                          heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float) -> torch.Tensor:
+                          heads: int, kv_heads: int, head_dim: int, window: int | None, scale: float,
+                          tiled_out: bool = False):
     """Matrix-core attention for one new token per sequence; ``max_len`` bounds every sequence's length
-    after this step (it sizes the grid and the workspace, not the result)."""
+    after this step (it sizes the grid and the workspace, not the result).  ``tiled_out``: the result as
+    ``TiledRows`` (at most 64 sequences)."""
     tokens, stride = qkv.shape
     if tokens != seqs:
         raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
     chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
-    out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    out = (TiledRows.empty(tokens, heads * head_dim, qkv.device) if tiled_out else
+           torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device))
     ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
-    _call("ri_attention_decode_bf16", _dev(out, "out"), _dev(ws, "workspace"), _dev(qkv, "qkv", torch.bfloat16), stride,
+    _call("ri_attention_decode_bf16", _dev(out.data if tiled_out else out, "out"), _dev(ws, "workspace"), _dev(qkv, "qkv", torch.bfloat16), stride,
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
-          k_pages.shape[2], int(window or 0), float(scale), _stream())
+          k_pages.shape[2], int(window or 0), float(scale), int(tiled_out), _stream())
     return out
 
 
 def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_pages, tok_pos, page_table, seqs: int,
                                 max_len: int, heads: int, kv_heads: int, head_dim: int, window: int | None,
-                                scale: float) -> torch.Tensor:
+                                scale: float, tiled_out: bool = False):
     """A layer's decode attention from the raw ``qkv: [seqs, (H + 2 Hkv) dh]``: q/k norm, rotation, the new
-    token's k and v into their pages and attention in one kernel, then the join."""
+    token's k and v into their pages and attention in one kernel, then the join.  ``tiled_out``: the result
+    as ``TiledRows``."""
     tokens, stride = qkv.shape
     if tokens != seqs:
         raise ShapeError(f"decode attention takes one token per sequence, got {tokens} tokens for {seqs} sequences")
@@ -300,16 +308,17 @@ def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_p
         raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv heads "
                          f"of {head_dim}")
     chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
-    out = torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    out = (TiledRows.empty(tokens, heads * head_dim, qkv.device) if tiled_out else
+           torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device))
     ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
     half = head_dim // 2
-    _call("ri_attention_decode_fused_bf16", _dev(out, "out"), _dev(ws, "workspace"),
+    _call("ri_attention_decode_fused_bf16", _dev(out.data if tiled_out else out, "out"), _dev(ws, "workspace"),
           _dev(qkv, "qkv", torch.bfloat16), stride, _opt(q_gain, "q_gain", torch.float32, (head_dim,)),
           _opt(k_gain, "k_gain", torch.float32, (head_dim,)), float(eps),
           _opt(inv_freq, "inv_freq", torch.float32, (half,)), _dev(k_pages, "k_pages", torch.bfloat16),
           _dev(v_pages, "v_pages", torch.bfloat16), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, chunks, heads, kv_heads, head_dim,
-          page_size, int(window or 0), float(scale), _stream())
+          page_size, int(window or 0), float(scale), int(tiled_out), _stream())
     return out
 
 
@@ -367,11 +376,11 @@ TILED_X, TILED_OUT = 1, 2
 
 
 class TiledRows:
-    """Up to 16 bfloat16 rows of ``k`` columns in the order the matrix cores take them as an operand:
-    ``data[ceil(k / 32), 64, 8]``, lane ``l`` of a tile holding row ``l % 16`` and the columns
-    ``8 * (l // 16) ..+8`` of the tile's 32.  The packed product writes its result this way for the
-    next packed product, which then loads a tile as one kilobyte in a row; rows beyond ``m`` and columns
-    beyond ``k`` are never read."""
+    """Up to 64 bfloat16 rows of ``k`` columns in the order the matrix cores take them as an operand:
+    ``data[ceil(m / 16), ceil(k / 32), 64, 8]``, lane ``l`` of a tile holding row ``l % 16`` of its 16 rows and
+    the columns ``8 * (l // 16) ..+8`` of its 32.  A packed product, a norm or the decode attention writes its
+    result this way for the packed product after it, which then loads a tile as one kilobyte in a row; rows
+    beyond ``m`` and columns beyond ``k`` are never read."""
 
     def __init__(self, data: torch.Tensor, m: int, k: int):
         self.data, self.shape = data, (m, k)
@@ -379,15 +388,16 @@ class TiledRows:
 
     @staticmethod
     def empty(m: int, k: int, device) -> "TiledRows":
-        if not 1 <= m <= 16:
-            raise ShapeError(f"tiled rows hold 1 to 16 rows, not {m}")
-        return TiledRows(torch.empty((-(-k // 32), 64, 8), dtype=torch.bfloat16, device=device), m, k)
+        if not 1 <= m <= 64:
+            raise ShapeError(f"tiled rows hold 1 to 64 rows, not {m}")
+        return TiledRows(torch.empty((-(-m // 16), -(-k // 32), 64, 8), dtype=torch.bfloat16, device=device), m, k)
 
     def rows(self) -> torch.Tensor:
         """The same values row-major, ``[m, k]``."""
         m, k = self.shape
-        tiles = self.data.shape[0]
-        return self.data.view(tiles, 4, 16, 8).permute(2, 0, 1, 3).reshape(16, tiles * 32)[:m, :k].contiguous()
+        row_tiles, tiles = self.data.shape[:2]
+        return (self.data.view(row_tiles, tiles, 4, 16, 8).permute(0, 3, 1, 2, 4)
+                .reshape(row_tiles * 16, tiles * 32)[:m, :k].contiguous())
 
 
 def as_rows(x):
@@ -431,18 +441,23 @@ class NormedLater:
         self.shape, self.dtype, self.device = xg.shape, xg.dtype, xg.device
 
 
-def gemm_mid_packed_bf16(x: torch.Tensor, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16,
-                         swiglu: bool = False) -> torch.Tensor:
-    """``x @ w.T`` for up to 64 bfloat16 rows with ``w`` packed by ``pack_for_mfma``: the packed product for
-    the steps of 17 to 64 tokens."""
+def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16, swiglu: bool = False,
+                         tiled_out: bool = False):
+    """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by
+    ``pack_for_mfma``: the packed product for the steps of 17 to 64 tokens.  ``tiled_out``: the bfloat16
+    result as ``TiledRows``."""
     m, k = x.shape
     row_tiles = -(-n // 16)
     want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
     if tuple(wpacked.shape) != want:
         raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
-    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    _call("ri_gemm_mid_packed_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
-          _dev(wpacked, "wpacked", torch.bfloat16), m, n, k, int(swiglu), _stream())
+    if tiled_out and out_dtype != torch.bfloat16:
+        raise ShapeError("a tiled result is bfloat16")
+    x_tiled = isinstance(x, TiledRows)
+    out = TiledRows.empty(m, n, x.device) if tiled_out else torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _call("ri_gemm_mid_packed_bf16", _dev(out.data if tiled_out else out, "out"), code(out_dtype),
+          _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
+          int(swiglu), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), _stream())
     return out
 
 

@@ -70,10 +70,13 @@ class GroupedQueryAttention(Mixer):
         qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
         self.w_qkv = rt.pack(rt.place_matrix(qkv))
         self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]))
-        self.takes_tiled = self.w_qkv.packed is not None       # prepared rows may come in the matrix cores' order
         self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
         self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
         self.position.bind(weights, rt)
+
+    def takes_tiled_at(self, m: int) -> bool:
+        """Whether this part's first product reads ``m`` rows in the matrix cores' order."""
+        return self.rt.takes_tiled(self.w_qkv, m)
 
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window)
@@ -89,7 +92,8 @@ class GroupedQueryAttention(Mixer):
             o = ops.attention_decode_fused_bf16(qkv, self.q_gain, self.k_gain, self.eps,
                                                 self.position.rotation_table(), store.k_pages, store.v_pages,
                                                 ctx.tok_pos, page_table, ctx.B, ctx.max_len, self.heads,
-                                                self.kv_heads, self.head_dim, self.window, self.scale)
+                                                self.kv_heads, self.head_dim, self.window, self.scale,
+                                                tiled_out=rt.takes_tiled(self.w_o, ctx.B))
             return rt.linear_packed(o, self.w_o, link=link)
         ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
                                   ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
@@ -104,7 +108,8 @@ class GroupedQueryAttention(Mixer):
         if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
             if ctx.is_decode:
                 return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
-                                                 page_table, ctx.B, ctx.max_len, *args)
+                                                 page_table, ctx.B, ctx.max_len, *args,
+                                                 tiled_out=self.rt.takes_tiled(self.w_o, ctx.B))
             return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                               page_table, ctx.B, ctx.max_new, *args)
         return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args)

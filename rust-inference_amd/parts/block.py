@@ -8,6 +8,8 @@ from .registry import build_part, register_part
 # A decode step of at most this many tokens leaves its norms to the products around them (the
 # products that can do it take no more rows).
 LINK_MAX_TOKENS = 16
+# Up to this many rows a norm hands its rows on in the matrix cores' order when the reader asks.
+TILED_MAX_ROWS = 64
 
 
 class NormLink:
@@ -50,8 +52,9 @@ class ResidualStream:
         else:
             self.pending = branch
 
-    def normed(self, norm, out_dtype, rows=None, later_ok: bool = False):
-        """The stream through ``norm``.  With ``later_ok`` the caller takes a ``NormedLater`` too."""
+    def normed(self, norm, out_dtype, rows=None, later_ok: bool = False, tiled: bool = False):
+        """The stream through ``norm``.  With ``later_ok`` the caller takes a ``NormedLater`` too, with
+        ``tiled`` (a norm that can, up to 64 rows) ``ops.TiledRows``."""
         if self.later is not None:
             later, for_norm = self.later
             self.later = None
@@ -60,7 +63,11 @@ class ResidualStream:
             # prepared for another reader: the sum is complete, norm it the plain way
         if self.pending is not None and self.pending.dim() == 3 and not getattr(norm, "accepts_parts", False):
             self.pending = self.pending.sum(0)       # a norm that does not know about parts
-        out = norm.apply(self.sum, self.pending, out_dtype, rows)
+        if (tiled and rows is None and getattr(norm, "can_tile", False) and out_dtype == torch.bfloat16
+                and self.sum.shape[0] <= TILED_MAX_ROWS):
+            out = norm.apply(self.sum, self.pending, out_dtype, rows, tiled=True)
+        else:
+            out = norm.apply(self.sum, self.pending, out_dtype, rows)
         if rows is None:
             self.pending = None      # the kernel wrote sum + pending back
         return out
@@ -72,6 +79,11 @@ class ResidualStream:
             pending = self.pending.sum(0) if self.pending.dim() == 3 else self.pending
             self.sum.add_(pending.to(self.sum.dtype))
             self.pending = None
+
+
+def _takes_tiled(part, rows: int) -> bool:
+    asks = getattr(part, "takes_tiled_at", None)
+    return bool(asks(rows)) if asks else False
 
 
 @register_part("arrangement", "prenorm")
@@ -93,21 +105,23 @@ class PreNormBlock:
         """The norm through which this layer first reads the stream."""
         return self.mixer_norm
 
-    def entry_takes_tiled(self) -> bool:
-        """Whether the part behind that norm reads rows in the matrix cores' order."""
-        return bool(getattr(self.mixer, "takes_tiled", False))
+    def entry_takes_tiled(self, rows: int) -> bool:
+        """Whether the part behind that norm reads ``rows`` rows in the matrix cores' order."""
+        return _takes_tiled(self.mixer, rows)
 
     def forward(self, stream: ResidualStream, ctx, store, page_table, act_dtype) -> None:
         # a part with ``links_norms`` takes a NormedLater as input and a NormLink for its output
+        rows = stream.sum.shape[0]
         if getattr(self.mixer, "links_norms", False):
-            h = stream.normed(self.mixer_norm, act_dtype, later_ok=True)
-            link = stream.link(self.feed_forward_norm, act_dtype, getattr(self.feed_forward, "takes_tiled", False))
+            h = stream.normed(self.mixer_norm, act_dtype, later_ok=True, tiled=_takes_tiled(self.mixer, rows))
+            link = stream.link(self.feed_forward_norm, act_dtype, _takes_tiled(self.feed_forward, rows))
             stream.push(self.mixer.forward(h, ctx, store, page_table, link=link))
         else:
             h = stream.normed(self.mixer_norm, act_dtype)
             stream.push(self.mixer.forward(h, ctx, store, page_table))
         if getattr(self.feed_forward, "links_norms", False):
-            h = stream.normed(self.feed_forward_norm, act_dtype, later_ok=True)
+            h = stream.normed(self.feed_forward_norm, act_dtype, later_ok=True,
+                              tiled=_takes_tiled(self.feed_forward, rows))
             link = stream.link(stream.next_entry_norm, act_dtype, stream.next_entry_tiled)
             stream.push(self.feed_forward.forward(h, ctx, link=link))
         else:

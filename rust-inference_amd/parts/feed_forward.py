@@ -33,13 +33,15 @@ class SwiGLU(FeedForward):
         gate_up = rt.place_matrix(torch.cat([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], 0))
         self.w_gate_up = rt.pack(gate_up, swiglu=True)
         self.w_down = rt.pack(rt.place_matrix(weights[p + "down_proj.weight"]))
-        # rows prepared for this part may come in the matrix cores' order when its first product takes them so
-        self.takes_tiled = self.w_gate_up.packed is not None
+
+    def takes_tiled_at(self, m: int) -> bool:
+        """Whether this part's first product reads ``m`` rows in the matrix cores' order."""
+        return self.rt.takes_tiled(self.w_gate_up, m)
 
     def forward(self, x, ctx, link=None):
         rt = self.rt
         # the activation is in the epilogue of the decode-size kernels, which hand the down product its rows
         # in the order it loads fastest when that product is a packed one too
-        a = rt.linear_packed(x, self.w_gate_up, tiled_out=self.w_down.packed is not None)
+        a = rt.linear_packed(x, self.w_gate_up, tiled_out=rt.takes_tiled(self.w_down, x.shape[0]))
         # may come in parts: the stream's next norm adds them
         return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)

@@ -138,7 +138,7 @@ class DecoderModel:
             entry = getattr(follower, "entry_norm", None)
             stream.next_entry_norm = entry() if entry else None
             tiled = getattr(follower, "entry_takes_tiled", None)
-            stream.next_entry_tiled = tiled() if tiled else False
+            stream.next_entry_tiled = tiled(stream.sum.shape[0]) if tiled else False
             store, table = None, None
             if run.cache is not None:
                 need = cache.needs[run.cache]

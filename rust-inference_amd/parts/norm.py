@@ -14,6 +14,7 @@ class RMSNorm(Norm):
 
     accepts_parts = True
     linkable = True          # gain, eps and dim are all a product needs to do this norm itself
+    can_tile = True          # hands its rows on in the matrix cores' order when asked (up to 64 rows)
 
     def __init__(self, dim: int, eps: float, name: str):
         self.dim, self.eps, self.name = dim, eps, name
@@ -25,5 +26,6 @@ class RMSNorm(Norm):
         self.rt = rt
         self.gain = rt.place_gain(weights[self.name])
 
-    def apply(self, residual, pending, out_dtype, rows=None):
-        return ops.add_rmsnorm(residual, pending, self.gain, self.eps, out_dtype, rows)
+    def apply(self, residual, pending, out_dtype, rows=None, tiled=False):
+        tiled = tiled and self.dim % 4 == 0 and self.dim <= 8192        # what the vectorised kernel takes
+        return ops.add_rmsnorm(residual, pending, self.gain, self.eps, out_dtype, rows, tiled=tiled)

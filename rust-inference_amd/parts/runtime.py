@@ -24,12 +24,17 @@ from ..kernels import ops
 #              own, fetched in whole cache lines (faster at 16 rows, slower at 4 and 8 and on short K).
 GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
-# 17 to 64 rows: the packed kernel with two or four tiles of x to every weight tile beats the library on small
-# matrices (at 32 rows, 4096 x 1024: 5.5 us against 9.8; gate|up of 2 x 3072 x 1024 with its activation: 6.5
-# against 14.0) and loses on large ones (6144 x 4096: 23.6 against 15.1), where the rows of x, fetched by
-# every workgroup from the L2 cache, weigh as much as the weights.
+# 17 to 64 rows: the packed kernel with two or four tiles of x to every weight tile.  With x in plain rows,
+# which every workgroup fetches from the L2 cache sixteen half cache lines a load, it beats the library on
+# small matrices only (at 32 rows, 4096 x 1024: 5.5 us against 9.8; 6144 x 4096: 23.6 against 15.1).  With
+# x in tiles (whoever makes the rows makes them so when the product asks) it is level or ahead on the large
+# ones too up to 32 rows (Qwen3-8B sizes at 32 rows, us: q|k|v 16.6 : 16.1, o 10.9 : 13.0, gate|up 40.2 : 51.0
+# + 5 for the activation, down 28.3 : 28.5; 5120 x 25600: 97 : 146; the model's decode step at 24 and 32
+# sequences is 5% and 7% shorter).  From 33 rows on it is not: q|k|v 23.2 : 18.0, and gate|up, level alone
+# with the activation counted (51.8 : 51.8 + 5), made the step at 48 sequences 1% longer.
 MID_MAX_ROWS = 64
 MID_MAX_BYTES = 20_000_000
+MID_TILED_ROWS = 32
 SPLIT_K = 4096
 # Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation
 # rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
@@ -132,6 +137,23 @@ class Runtime:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
 
+    @staticmethod
+    def _mid_pays(pw: PackedWeight, m: int, tiled: bool) -> bool:
+        """Whether the packed kernel for 17 to 64 rows beats the library's product (and, for gate|up, its
+        activation kernel) on this matrix."""
+        if pw.w.shape[0] * pw.k * 2 <= MID_MAX_BYTES:
+            return True
+        return tiled and m <= MID_TILED_ROWS
+
+    def takes_tiled(self, pw: PackedWeight, m: int) -> bool:
+        """Whether the product of ``m`` rows with this weight runs on a packed kernel: whoever makes its
+        rows then makes them as ``ops.TiledRows``."""
+        if self.dtype != torch.bfloat16 or pw.packed is None or pw.k % 8:
+            return False
+        if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
+            return True
+        return SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and self._mid_pays(pw, m, True)
+
     def linear_packed(self, x, pw: PackedWeight, out_dtype=None, parts_ok: bool = False, link=None,
                       tiled_out: bool = False):
         """``x @ w.T`` (or ``silu(x @ gate.T) * (x @ up.T)`` for a fused gate|up weight) with the kernel
@@ -169,8 +191,10 @@ class Runtime:
                     return ops.gemv_bf16(ops.as_rows(x), pw.w, out_dtype, swiglu=pw.swiglu)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
             if (SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and pw.packed is not None
-                    and pw.w.shape[0] * pw.k * 2 <= MID_MAX_BYTES):
-                return ops.gemm_mid_packed_bf16(self.normed_now(x), pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
+                    and self._mid_pays(pw, m, isinstance(x, ops.TiledRows))):
+                x = self.normed_now(x) if later else x
+                return ops.gemm_mid_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu,
+                                                tiled_out=tiled_out and out_dtype == torch.bfloat16)
         y = self.linear(x, pw.w, None if pw.swiglu else out_dtype)
         return ops.swiglu(y) if pw.swiglu else y
 

@@ -474,6 +474,60 @@ def test_packed_product_of_17_to_64_rows(ops, m, n, k):
         ops.gemm_mid_packed_bf16(t(rng.normal(size=(65, k)), torch.bfloat16), pw, n)
 
 
+@pytest.mark.parametrize("m", [1, 16, 17, 40, 64])
+@pytest.mark.parametrize("dim, n", [(104, 56), (4096, 1000), (584, 40)])
+def test_every_maker_of_rows_can_tile_them(ops, m, dim, n):
+    """The norm, the decode attention and the product for 17 to 64 rows write their rows in the matrix cores'
+    order on request, bit for bit the rows they write plainly; the products read them so."""
+    rng = np.random.default_rng(5 * m + dim)
+    residual = t(rng.normal(size=(m, dim)) * 2)
+    pending = t(rng.normal(size=(m, dim)), torch.bfloat16)
+    gain = t(1 + 0.2 * rng.normal(size=dim))
+    plain = ops.add_rmsnorm(residual.clone(), pending, gain, 1e-5, torch.bfloat16)
+    r2 = residual.clone()
+    tiled = ops.add_rmsnorm(r2, pending, gain, 1e-5, torch.bfloat16, tiled=True)
+    assert isinstance(tiled, ops.TiledRows) and tiled.shape == (m, dim) and torch.equal(tiled.rows(), plain)
+    close(r2, f64(residual) + f64(pending), 1e-6, "the sum is written back either way")
+    # into the products: the one for 17 to 64 rows takes fewer too
+    pw = ops.pack_for_mfma(t(rng.normal(size=(n, dim)) / np.sqrt(dim), torch.bfloat16))
+    pgu = ops.pack_for_mfma(t(rng.normal(size=(2 * n, dim)) * (4.0 / np.sqrt(dim)), torch.bfloat16), swiglu=True)
+    want = ops.gemm_mid_packed_bf16(plain, pw, n)
+    assert torch.equal(ops.gemm_mid_packed_bf16(tiled, pw, n), want)
+    out_tiled = ops.gemm_mid_packed_bf16(tiled, pw, n, tiled_out=True)
+    assert isinstance(out_tiled, ops.TiledRows) and torch.equal(out_tiled.rows(), want)
+    assert torch.equal(ops.gemm_mid_packed_bf16(tiled, pgu, n, swiglu=True, tiled_out=True).rows(),
+                       ops.gemm_mid_packed_bf16(plain, pgu, n, swiglu=True))
+    if m <= 16:
+        assert torch.equal(ops.gemm_skinny_packed_bf16(tiled, pw, n), want)
+    with pytest.raises(Exception, match="64"):
+        ops.add_rmsnorm(t(rng.normal(size=(65, dim))), None, gain, 1e-5, torch.bfloat16, tiled=True)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_decode_attention_writes_tiled_rows(ops, fused):
+    rng = np.random.default_rng(77)
+    heads, kv_heads, dh = 8, 2, 64
+    lens = [int(x) for x in rng.integers(1, 600, size=20)]
+    B = len(lens)
+    k, v, kp, vp, table = paged(rng, [n + 1 for n in lens], kv_heads, dh, dtype=torch.bfloat16, spare=12)
+    pos = t([n - 1 for n in lens], torch.int32)
+    outs = []
+    for tiles in (False, True):
+        if fused:
+            raw = t(np.random.default_rng(78).normal(size=(B, (heads + 2 * kv_heads) * dh)) * 2, torch.bfloat16)
+            gains = t(np.ones(dh))
+            out = ops.attention_decode_fused_bf16(raw, gains, gains, 1e-5, t(P.rope_inv_freq(dh, 1e4)), kp, vp, pos, table,
+                                                  B, max(lens) + 50, heads, kv_heads, dh, None, dh ** -0.5, tiled_out=tiles)
+        else:
+            qkv = t(np.random.default_rng(79).normal(size=(B, (heads + 2 * kv_heads) * dh)), torch.bfloat16)
+            cu = t(np.arange(B + 1), torch.int32)
+            out = ops.attention_decode_bf16(qkv, kp, vp, cu, pos, table, B, max(lens) + 50, heads, kv_heads, dh, None,
+                                            dh ** -0.5, tiled_out=tiles)
+        assert isinstance(out, ops.TiledRows) == tiles
+        outs.append(ops.as_rows(out))
+    assert torch.equal(outs[0], outs[1]) and outs[0].shape == (B, heads * dh)
+
+
 @pytest.mark.parametrize("m", [1, 3, 8, 13, 16])
 @pytest.mark.parametrize("hidden, k, inter", [(104, 72, 56), (4096, 4096, 1000), (584, 12288, 40)])
 def test_rows_in_the_matrix_cores_order(ops, m, hidden, k, inter):
