@@ -34,7 +34,11 @@ def assert_same_tokens(got, want, dtype_name):
                     f"request {i}, token {j}: {a} against {b} (margin {margins[j]:.3f}, {dtype_name})"
                 break
         else:
-            assert len(g) == len(toks), f"request {i}: {len(g)} tokens against {len(toks)}"
+            # one side may have ended on a stop token (which is not put out) where the other picked another token:
+            # the same parting of ways, seen as a difference in length
+            j = min(len(g), len(toks))
+            assert len(g) == len(toks) or (dtype_name == "bfloat16" and j < len(margins) and margins[j] < 0.08), \
+                f"request {i}: {len(g)} tokens against {len(toks)}"
 
 
 def prompts_for(cfg, lengths, seed):
@@ -59,6 +63,29 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name, lengths, st
     assert res.stats.prompt_tokens == sum(lengths) and res.stats.decode_tokens == len(prompts) * (steps - 1)
     model.cache.check_consistent()
     assert model.cache.slots.free_count == 4
+
+
+@pytest.mark.parametrize("requests", [20, 40])
+def test_batches_of_tens_of_sequences(model_dirs, requests):
+    """Twenty and forty sequences a batch (the decode steps of 17 to 32 rows and of 33 to 64 take other kernels
+    than the smaller ones), some stopping early so that the batch shrinks through those sizes: graphs and
+    eager steps give the same tokens, and those are the plain implementation's."""
+    from rust_inference_amd import Model
+    cfg, _ = read_model_f64(model_dirs["D"])
+    rng = np.random.default_rng(requests)
+    lengths = [int(n) for n in rng.integers(1, 50, size=requests)]
+    prompts = prompts_for(cfg, lengths, 13)
+    stop = [int(t) for t in rng.integers(0, cfg["vocab_size"], 12)]             # a few sequences end on them
+    outs = []
+    for graphs in (False, True):
+        model = Model.load(model_dirs["D"], dtype="bfloat16", max_batch=requests, max_seq_len=96, use_graphs=graphs)
+        res = model.generate(prompts, max_new_tokens=12, stop_token_ids=stop)
+        model.cache.check_consistent()
+        assert model.cache.slots.free_count == requests
+        outs.append(res)
+    assert outs[0].tokens == outs[1].tokens and outs[0].finish_reasons == outs[1].finish_reasons
+    assert "stop" in outs[0].finish_reasons
+    assert_same_tokens(outs[0].tokens, plain_greedy_with_margins(model_dirs["D"], prompts, 12, stop), "bfloat16")
 
 
 def test_stop_tokens_and_batches_one_after_another(model_dirs):
