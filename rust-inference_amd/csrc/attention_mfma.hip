@@ -383,14 +383,17 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     const int b = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;      // chunks last: the empty ones start last
     const int group = heads / kv_heads;
     const int tok = b;                                       // one new token per sequence: token b is sequence b's
+    // The position and this wavefront's entry of the page table are asked for together: neither address
+    // depends on the other's value, and each is a trip to memory that the page's loads would wait for in turn.
+    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;   // this wavefront's page
     const int qpos = tok_pos[tok];
+    const int phys = page_table[(long)b * table_width + min(page, table_width - 1)];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
 
-    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;   // this wavefront's page
     const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
     PageFrags<DH> f;
-    if (has) load_page<DH>(f, k_pages, v_pages, page_table[(long)b * table_width + page], kv_heads, kvh, lane);
+    if (has) load_page<DH>(f, k_pages, v_pages, phys, kv_heads, kvh, lane);
 
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
@@ -502,11 +505,53 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
     out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
 }
 
+// The join of up to JOIN_SERIAL chunks with every load asked for at once, before the position is known:
+// the chunks' results and markers lie at places that depend on the grid alone, so one trip to memory
+// fetches them all (those of chunks the sequence has not reached are fetched and not used), where the
+// loop above makes three trips in turn (the position, the maxima, the results).  The same operations in
+// the same order as that loop: the results are equal bit for bit.
+template <int DH>
+__global__ void __launch_bounds__(DH)
+attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
+                              int heads, int window, int max_chunks, int tiled) {
+    const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    const float* base = ws + ((long)b * heads + h) * max_chunks * (DH + 2);
+    float o[JOIN_SERIAL], mc[JOIN_SERIAL], lc[JOIN_SERIAL];
+#pragma unroll
+    for (int c = 0; c < JOIN_SERIAL; ++c) {
+        o[c] = 0.f;
+        mc[c] = -INFINITY;
+        lc[c] = 0.f;
+        if (c < max_chunks) {
+            o[c] = base[c * (DH + 2) + d];
+            mc[c] = base[c * (DH + 2) + DH];
+            lc[c] = base[c * (DH + 2) + DH + 1];
+        }
+    }
+    const int qpos = tok_pos[b];
+    const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
+    const int c_lo = lo / DECODE_CHUNK, c_hi = qpos / DECODE_CHUNK;
+    float m = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < JOIN_SERIAL; ++c)
+        if (c >= c_lo && c <= c_hi) m = fmaxf(m, mc[c]);
+    float acc = 0.f, l = 0.f;
+#pragma unroll
+    for (int c = 0; c < JOIN_SERIAL; ++c) {                          // always in chunk order
+        if (c >= c_lo && c <= c_hi) {
+            const float f = mc[c] == -INFINITY ? 0.f : exp2f(mc[c] - m);
+            acc += o[c] * f;
+            l += lc[c] * f;
+        }
+    }
+    out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+}
+
 template <int DH>
 static void launch_join(bf16_t* out, const float* ws, const int32_t* tok_pos, int seqs, int heads, int window,
                         int max_chunks, int tiled, hipStream_t s) {
     if (max_chunks <= JOIN_SERIAL)
-        attn_decode_join_kernel<DH, 1><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window, max_chunks, tiled);
+        attn_decode_join_small_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window, max_chunks, tiled);
     else
         attn_decode_join_kernel<DH, JOIN_PARTS><<<dim3(seqs, heads), DH * JOIN_PARTS, 0, s>>>(out, ws, tok_pos, heads,
                                                                                            window, max_chunks, tiled);
@@ -565,17 +610,19 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;      // chunks last: the empty ones start last
     const int group = heads / kv_heads;
+    // the position and this wavefront's entry of the page table are asked for together (see above)
+    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;
     const int qpos = tok_pos[b];                             // token b is sequence b's one new token
+    const int phys = page_table[(long)b * table_width + min(page, table_width - 1)];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
     const bool owner = chunk == qpos / DECODE_CHUNK;         // this chunk holds the new token's position
 
     // 1. this wavefront's page is on its way while the queries are made
-    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;
     const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
-    const long phys_new = page_table[(long)b * table_width + qpos / PAGE];
     PageFrags<DH> f;
-    if (has) load_page<DH>(f, k_pages, v_pages, page_table[(long)b * table_width + page], kv_heads, kvh, lane);
+    if (has) load_page<DH>(f, k_pages, v_pages, phys, kv_heads, kvh, lane);
+    const long phys_new = page_table[(long)b * table_width + qpos / PAGE];
 
     // 2. queries of the group; in the owner also the new key and value
     const bf16_t* row = qkv + (long)b * q_stride;

@@ -105,6 +105,9 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     const bf16_t* wp = wpacked + ((size_t)nt * k_tiles * 64 + lane) * 8;
     const bf16_t* up = SWIGLU ? wpacked + ((size_t)(up_tile_offset + nt) * k_tiles * 64 + lane) * 8 : nullptr;
     const bool x_tiled = tiled & TILED_X;
+    // the same in every wavefront of the launch
+    const bool ring = K % 32 == 0 && tiles_per_wave % SK_CHUNK == 0 && part_tiles == tiles_per_wave * SK_WAVES &&
+                      k_tiles % part_tiles == 0;
     const bf16_t* xp = x_tiled ? x + (size_t)lane * 8 : x + (size_t)(x_ok ? i : 0) * K + jg * 8;
     const int x_step = x_tiled ? 512 : 32;                   // elements from one step's fragment to the next
     const uint4 zero = make_uint4(0, 0, 0, 0);
@@ -134,6 +137,36 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     }
 
     floatx4 acc = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
+    if (ring) {
+        // Every wavefront's share is a whole number of rounds of SK_CHUNK steps and K a multiple of 32: the
+        // fragments are a ring, and a register asks for the step SK_CHUNK further on as soon as the matrix
+        // cores have taken the one it held, so that SK_CHUNK steps' loads stay in flight all the way instead
+        // of draining at the end of every round.  The sums are the same ones in the same order.
+        Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];
+#pragma unroll
+        for (int c = 0; c < SK_CHUNK; ++c) {
+            wf[c].u = load_stream16(wp + (size_t)(kt_begin + c) * 512);
+            if (SWIGLU) uf[c].u = load_stream16(up + (size_t)(kt_begin + c) * 512);
+            xf[c].u = x_ok ? *reinterpret_cast<const uint4*>(xp + (size_t)(kt_begin + c) * x_step) : zero;
+        }
+        int kt = kt_begin;
+        for (; kt + SK_CHUNK < kt_end; kt += SK_CHUNK) {
+#pragma unroll
+            for (int c = 0; c < SK_CHUNK; ++c) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
+                if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
+                const size_t next = (size_t)(kt + c + SK_CHUNK);
+                wf[c].u = load_stream16(wp + next * 512);
+                if (SWIGLU) uf[c].u = load_stream16(up + next * 512);
+                xf[c].u = x_ok ? *reinterpret_cast<const uint4*>(xp + next * x_step) : zero;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < SK_CHUNK; ++c) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
+            if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
+        }
+    } else
     for (int kt = kt_begin; kt < kt_end; kt += SK_CHUNK) {
         Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];
 #pragma unroll
