@@ -62,6 +62,10 @@ int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const vo
 // workspace: float32 [seqs, heads, max_chunks, head_dim + 2]; max_chunks >= ri_attention_decode_chunks(longest
 // sequence after this step); at most 16 query heads per kv head.
 int ri_attention_decode_chunks(int max_len);
+// Whether ri_attention_decode_bf16 takes a step of this size with its streaming kernel (a workgroup walks a
+// whole run of a sequence's pages; no join when a sequence is one run): the number of runs per sequence, or
+// 0 for one workgroup per chunk.
+int ri_attention_decode_streams(int seqs, int kv_heads, int max_chunks);
 int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride, const void* k_pages,
                              const void* v_pages, const int32_t* cu_seqlens, const int32_t* tok_pos,
                              const int32_t* page_table, int table_width, int seqs, int max_chunks, int heads,

@@ -530,7 +530,9 @@ attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict_
     }
     const int qpos = tok_pos[b];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    const int c_lo = lo / DECODE_CHUNK, c_hi = qpos / DECODE_CHUNK;
+    // window < 0: the entries are not chunks at fixed places but the runs of the streaming kernel, all of
+    // them written (an empty run as a maximum of -inf)
+    const int c_lo = window < 0 ? 0 : lo / DECODE_CHUNK, c_hi = window < 0 ? max_chunks - 1 : qpos / DECODE_CHUNK;
     float m = -INFINITY;
 #pragma unroll
     for (int c = 0; c < JOIN_SERIAL; ++c)
@@ -557,15 +559,7 @@ static void launch_join(bf16_t* out, const float* ws, const int32_t* tok_pos, in
                                                                                            window, max_chunks, tiled);
 }
 
-// ------------------------------------------------------------------ decode, everything in one kernel
-// The decode step's attention from the raw projection: per-head RMSNorm and rotation of the new token's q
-// and k, the write of its k and v into their page, and the attention over chunks of 256 keys, in one
-// kernel; the join of the chunks follows as a second one.  Every workgroup norms and rotates the group's
-// queries for itself (a few hundred elements); the workgroup whose chunk holds the new token's position
-// also makes the new key and value, stores them for later steps and patches them into the fragments it
-// has just read from the page (the page in memory does not have them yet).  (Joining inside the same
-// kernel, by the workgroup that finishes last, was tried: the device-wide fences it needs write the
-// whole L2 back and cost many times what the second launch costs.)
+// ------------------------------------------------------------------ decode: the new token's own q, k and v
 template <int DH>
 __device__ __forceinline__ void norm_rotate_head(bf16_t* dst_lds, const bf16_t* __restrict__ x,
                                                  const float* __restrict__ gain, float eps,
@@ -593,6 +587,209 @@ __device__ __forceinline__ void norm_rotate_head(bf16_t* dst_lds, const bf16_t* 
     }
 }
 
+// The new token's key and value, which its page in memory does not hold yet, put into the fragments that
+// were read from that page: key r of the page from knew, its value from vnew (both in LDS).
+template <int DH>
+__device__ __forceinline__ void patch_new_token(PageFrags<DH>& f, const bf16_t* knew, const bf16_t* vnew, int r,
+                                                int lane) {
+    const int jg = lane >> 4, col = lane & 15;
+    const int i_new = (r >> 3) * 4 + (r & 3);                // the fragment row that holds key r
+    if (col == i_new) {
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks) {
+            const uint4 kv = *reinterpret_cast<const uint4*>(&knew[ks * 32 + jg * 8]);
+            if ((r & 7) >= 4) f.k[1][ks].u = kv; else f.k[0][ks].u = kv;
+        }
+    }
+    if (jg == (r >> 3)) {                                    // lanes whose eight keys include key r
+        const int e = r & 7;
+#pragma unroll
+        for (int dt = 0; dt < DH / 16; ++dt) {
+            const uint32_t v = vnew[dt * 16 + col];
+            uint32_t w[4] = {f.v[dt].u.x, f.v[dt].u.y, f.v[dt].u.z, f.v[dt].u.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (k == (e >> 1)) w[k] = (e & 1) ? ((w[k] & 0x0000FFFFu) | (v << 16)) : ((w[k] & 0xFFFF0000u) | v);
+            f.v[dt].u = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ decode, streaming
+// When the step has keys enough to fill the machine without cutting every sequence into chunks of 256 (many
+// sequences, or very long ones), a workgroup walks a whole run of a sequence's pages instead: its four
+// wavefronts take every fourth page, each with the next page's loads in flight while it works on the one it
+// has, and keep their running maximum, sum and output across pages as the prefill kernel does.  The memory
+// system then sees one long stream per wavefront rather than a burst per workgroup with a start and an end
+// around it.  A sequence is cut into `splits` runs of whole chunks by its own length alone; with one run the
+// kernel writes the output itself and no join follows, with more the runs' results go to the workspace
+// [seqs, heads, splits, DH + 2] and the join adds them in run order.
+#define STREAM_WAVES 4
+
+// FUSED: qkv is the raw projection; the kernel norms and rotates the group's queries for itself, and the
+// workgroup whose run ends at the new token's position makes the new key and value and stores them into their
+// page before any page is read.
+template <int DH, bool FUSED>
+__global__ void __launch_bounds__(STREAM_WAVES * 64, 2)
+attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride,
+                          const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+                          const float* __restrict__ inv_freq, bf16_t* k_pages, bf16_t* v_pages,
+                          const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
+                          int heads, int kv_heads, int window, float scale_log2, int splits, int tiled) {
+    static_assert(!FUSED || DH <= 128, "one (d, d + DH/2) pair per lane");
+    __shared__ float o_lds[STREAM_WAVES][DH * 17];
+    __shared__ float ml_lds[STREAM_WAVES][2][16];
+    __shared__ __attribute__((aligned(16))) bf16_t q_lds[FUSED ? 16 : 1][DH];
+    __shared__ __attribute__((aligned(16))) bf16_t knew[DH];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+    const int group = heads / kv_heads;
+    const int qpos = tok_pos[b];                             // token b is sequence b's one new token
+    const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
+    const int c_lo = lo / DECODE_CHUNK, c_hi = qpos / DECODE_CHUNK;
+    const int per = (c_hi - c_lo + splits) / splits;         // chunks per run: by the sequence's own length
+    const int c0 = c_lo + split * per, c1 = min(c_hi, c0 + per - 1);
+    const int p_first = max(c0 * (DECODE_CHUNK / PAGE), lo / PAGE);
+    const int p_last = min(c1 * (DECODE_CHUNK / PAGE) + DECODE_CHUNK / PAGE - 1, qpos / PAGE);   // below p_first: an empty run
+    const int32_t* table = page_table + (long)b * table_width;
+
+    // This wavefront's pages are p_first + wave + STREAM_WAVES * j, j = 0, 1, ...; lane l holds the table's entry for
+    // j = base + l, fetched 64 at a time, so that a page's address never waits for a trip to memory of its own.
+    const int mine = p_first + wave;
+    int held = 0;
+    {
+        const int pg = mine + STREAM_WAVES * lane;
+        held = pg <= p_last ? table[pg] : 0;
+    }
+    auto phys_of = [&](int j) -> long { return (long)__builtin_amdgcn_readlane(held, j & 63); };
+    auto open_page = [&](int pg) -> bool { return pg * PAGE + PAGE - 1 <= qpos && pg * PAGE >= lo; };
+    // The group's queries and, where the run ends at the new token, its key and value.  These go into their
+    // page before the workgroup reads any page: the barrier makes them visible to the wavefront that will
+    // read that page, the last of the run, so nothing has to be patched into fragments afterwards.
+    Columns<DH, 1> c;
+    init_columns<DH, 1>(c);
+    const int jg = lane >> 4, col = lane & 15;
+    if (FUSED) {
+        const bf16_t* row = qkv + (long)b * q_stride;
+        const int page_new = qpos / PAGE;
+        for (int g = wave; g < group; g += STREAM_WAVES)
+            norm_rotate_head<DH>(q_lds[g], row + (kvh * group + g) * DH, q_gain, eps, inv_freq, qpos, lane);
+        if (p_first <= p_last && p_last == page_new) {       // this run holds the new token's position
+            const int slot = qpos % PAGE;
+            const long head_base = ((long)table[page_new] * kv_heads + kvh) * (long)(PAGE * DH);
+            if (wave == STREAM_WAVES - 1) {                  // the key: norm, rotation, into its page
+                norm_rotate_head<DH>(knew, row + (heads + kvh) * DH, k_gain, eps, inv_freq, qpos, lane);
+                __builtin_amdgcn_wave_barrier();
+                for (int d = lane; d < DH; d += 64) k_pages[head_base + (long)slot * DH + d] = knew[d];
+            } else if (wave == STREAM_WAVES - 2) {           // the value: a copy, transposed inside the page
+                for (int d = lane; d < DH; d += 64)
+                    v_pages[head_base + (long)d * PAGE + slot] = row[(heads + kv_heads + kvh) * DH + d];
+            }
+        }
+        __syncthreads();
+    }
+    if (col < group) {
+        c.qpos[0] = qpos;
+        c.lo[0] = lo;
+        if (FUSED) {
+#pragma unroll
+            for (int ks = 0; ks < DH / 32; ++ks)
+                c.q[0][ks].u = *reinterpret_cast<const uint4*>(&q_lds[col][ks * 32 + jg * 8]);
+        } else {
+            const bf16_t* qp = qkv + (long)b * q_stride + (kvh * group + col) * DH + jg * 8;
+#pragma unroll
+            for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
+        }
+    }
+    PageFrags<DH> fa, fb;
+    bool ha = mine <= p_last;
+    if (ha) load_page<DH>(fa, k_pages, v_pages, phys_of(0), kv_heads, kvh, lane);
+    for (int j = 0;; j += 2) {
+        const int pa = mine + STREAM_WAVES * j, pb = pa + STREAM_WAVES;
+        const bool hb = pb <= p_last;
+        if (hb) {
+            load_page<DH>(fb, k_pages, v_pages, phys_of(j + 1), kv_heads, kvh, lane);
+        }
+        if (ha) process_page<DH, 1>(c, fa, pa, lane, scale_log2, open_page(pa));
+        if (!hb) break;
+        const int pa2 = pb + STREAM_WAVES;
+        ha = pa2 <= p_last;
+        if (ha) {
+            if (((j + 2) & 63) == 0) {                       // the next 64 entries of the table
+                const int pg = pa2 + STREAM_WAVES * lane;
+                held = pg <= p_last ? table[pg] : 0;
+            }
+            load_page<DH>(fa, k_pages, v_pages, phys_of(j + 2), kv_heads, kvh, lane);
+        }
+        process_page<DH, 1>(c, fb, pb, lane, scale_log2, open_page(pb));
+        if (!ha) break;
+    }
+    finish_columns<DH, 1>(c);
+
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_lds[wave][(dt * 16 + jg * 4 + r) * 17 + col] = c.o[0][dt][r];
+    if (jg == 0) {
+        ml_lds[wave][0][col] = c.m[0];
+        ml_lds[wave][1][col] = c.l[0];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < group * DH; idx += STREAM_WAVES * 64) {
+        const int g = idx / DH, d = idx - g * DH;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < STREAM_WAVES; ++w) m = fmaxf(m, ml_lds[w][0][g]);
+        float acc = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < STREAM_WAVES; ++w) {              // always in wavefront order
+            const float mw = ml_lds[w][0][g];
+            const float f2 = mw == -INFINITY ? 0.f : exp2f(mw - m);
+            acc += o_lds[w][d * 17 + g] * f2;
+            l += ml_lds[w][1][g] * f2;
+        }
+        const int h = kvh * group + g;
+        if (splits == 1) {                                   // the new token sees itself at least: l > 0
+            out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
+        } else {
+            float* dst = ws + (((long)b * heads + h) * splits + split) * (DH + 2);
+            dst[d] = acc;
+            if (d == 0) {
+                dst[DH] = m;
+                dst[DH + 1] = l;
+            }
+        }
+    }
+}
+
+// Runs per sequence of the streaming kernel for a step of `seqs` sequences of up to `max_chunks` chunks, or 0
+// where the kernel of one workgroup per chunk is the faster one.  It depends on the step's size alone.
+// Measured at 8 kv heads of 128: with 64 sequences of 2,080 keys one run per sequence (512 workgroups, no
+// join) takes 94 us where the chunks and their join take 97 + 6; 8 sequences of 32,800 keys in 16 runs make
+// the step 2% shorter; with fewer workgroups than that the streams are too few to keep the memory busy (one
+// sequence of 131,000 keys in 16 runs: 12% longer), and at 32 or 48 sequences of 2,080 keys runs that still
+// need a join lose by 2%.
+static int stream_splits(int seqs, int kv_heads, int max_chunks) {
+    const long rows = (long)seqs * kv_heads;
+    if (rows >= 512) return 1;
+    if (rows >= 64 && max_chunks >= 64) return min(JOIN_SERIAL, max_chunks);
+    return 0;
+}
+
+extern "C" int ri_attention_decode_streams(int seqs, int kv_heads, int max_chunks) {
+    return stream_splits(seqs, kv_heads, max_chunks);
+}
+
+// ------------------------------------------------------------------ decode, everything in one kernel
+// The decode step's attention from the raw projection: per-head RMSNorm and rotation of the new token's q
+// and k, the write of its k and v into their page, and the attention over chunks of 256 keys, in one
+// kernel; the join of the chunks follows as a second one.  Every workgroup norms and rotates the group's
+// queries for itself (a few hundred elements); the workgroup whose chunk holds the new token's position
+// also makes the new key and value, stores them for later steps and patches them into the fragments it
+// has just read from the page (the page in memory does not have them yet).  (Joining inside the same
+// kernel, by the workgroup that finishes last, was tried: the device-wide fences it needs write the
+// whole L2 back and cost many times what the second launch costs.)
 template <int DH>
 __global__ void __launch_bounds__(DECODE_WAVES * 64)
 attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ q_gain,
@@ -656,29 +853,7 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
         for (int ks = 0; ks < DH / 32; ++ks)
             c.q[0][ks].u = *reinterpret_cast<const uint4*>(&q_lds[col][ks * 32 + jg * 8]);
     }
-    if (has && page == qpos / PAGE) {                        // the new token's key and value are not in memory yet
-        const int r = qpos % PAGE;
-        const int i_new = (r >> 3) * 4 + (r & 3);            // the fragment row that holds key r
-        if (col == i_new) {
-#pragma unroll
-            for (int ks = 0; ks < DH / 32; ++ks) {
-                const uint4 kv = *reinterpret_cast<const uint4*>(&knew[ks * 32 + jg * 8]);
-                if ((r & 7) >= 4) f.k[1][ks].u = kv; else f.k[0][ks].u = kv;
-            }
-        }
-        if (jg == (r >> 3)) {                                // lanes whose eight keys include key r
-            const int e = r & 7;
-#pragma unroll
-            for (int dt = 0; dt < DH / 16; ++dt) {
-                const uint32_t v = vnew[dt * 16 + col];
-                uint32_t w[4] = {f.v[dt].u.x, f.v[dt].u.y, f.v[dt].u.z, f.v[dt].u.w};
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (k == (e >> 1)) w[k] = (e & 1) ? ((w[k] & 0x0000FFFFu) | (v << 16)) : ((w[k] & 0xFFFF0000u) | v);
-                f.v[dt].u = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-        }
-    }
+    if (has && page == qpos / PAGE) patch_new_token<DH>(f, knew, vnew, qpos % PAGE, lane);
     if (has) process_page<DH, 1>(c, f, page, lane, scale_log2, false);
     finish_columns<DH, 1>(c);
 
@@ -797,6 +972,28 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
     dim3 grid(seqs, kv_heads, max_chunks);
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
+    const int splits = stream_splits(seqs, kv_heads, max_chunks);
+    if (splits > 0) {
+        dim3 sgrid(seqs, kv_heads, splits);
+#define RI_STREAM_CASE(DH)                                                                                        \
+    case DH:                                                                                                      \
+        attn_decode_stream_kernel<DH, false><<<sgrid, STREAM_WAVES * 64, 0, s>>>(                                 \
+            (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,                \
+            (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,        \
+            scale_log2, splits, tiled_out);                                                                       \
+        if (splits > 1)                                                                                           \
+            attn_decode_join_small_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos,  \
+                                                                               heads, -1, splits, tiled_out);     \
+        break;
+        switch (head_dim) {
+            RI_STREAM_CASE(32)
+            RI_STREAM_CASE(64)
+            RI_STREAM_CASE(128)
+        }
+#undef RI_STREAM_CASE
+        RI_LAUNCH_CHECK("attention_decode_bf16 (streaming)");
+        return 0;
+    }
 #define RI_DECODE_CASE(DH)                                                                                        \
     case DH:                                                                                                      \
         attn_decode_mfma_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                           \
@@ -834,6 +1031,28 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
     dim3 grid(seqs, kv_heads, max_chunks);
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
+    const int splits = stream_splits(seqs, kv_heads, max_chunks);
+    if (splits > 0) {
+        dim3 sgrid(seqs, kv_heads, splits);
+#define RI_STREAM_CASE(DH)                                                                                        \
+    case DH:                                                                                                      \
+        attn_decode_stream_kernel<DH, true><<<sgrid, STREAM_WAVES * 64, 0, s>>>(                                  \
+            (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,                 \
+            (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,        \
+            scale_log2, splits, tiled_out);                                                                       \
+        if (splits > 1)                                                                                           \
+            attn_decode_join_small_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos,  \
+                                                                               heads, -1, splits, tiled_out);     \
+        break;
+        switch (head_dim) {
+            RI_STREAM_CASE(32)
+            RI_STREAM_CASE(64)
+            RI_STREAM_CASE(128)
+        }
+#undef RI_STREAM_CASE
+        RI_LAUNCH_CHECK("attention_decode_fused_bf16 (streaming)");
+        return 0;
+    }
 #define RI_FUSED_CASE(DH)                                                                                         \
     case DH:                                                                                                      \
         attn_decode_fused_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                          \

@@ -46,6 +46,7 @@ _SIGNATURES = {
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_mid_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
+    "ri_attention_decode_streams": [c_int, c_int, c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
     "ri_gemm_skinny_packed_bf16_partials": [c_int],
     "ri_gemv_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
@@ -271,6 +272,13 @@ def attention_prefill_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_tabl
           _dev(page_table, "page_table", torch.int32), page_table.shape[1], seqs, max_new, heads, kv_heads, head_dim,
           k_pages.shape[2], int(window or 0), float(scale), _stream())
     return out
+
+
+def decode_attention_streams(seqs: int, kv_heads: int, max_len: int) -> bool:
+    """Whether ``attention_decode_bf16`` walks a step of this size with its streaming kernel (whole runs of a
+    sequence's pages per workgroup) rather than with one workgroup per chunk of 256 keys."""
+    chunks = _get("ri_attention_decode_chunks")(int(max_len))
+    return _get("ri_attention_decode_streams")(int(seqs), int(kv_heads), chunks) > 0
 
 
 def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_len: int,

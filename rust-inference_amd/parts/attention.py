@@ -17,7 +17,9 @@ from .spec import PartSpec
 # Up to this many sequences a decode step norms and rotates q and k inside the attention kernel (one
 # launch less per layer); beyond it the many workgroups each repeating that work cost more than the
 # launch (measured at 64 sequences of 2,048 tokens: 140 us against 111 + 6 us; at 24 and 32 sequences the
-# one kernel is still ahead, by 1% of the step).
+# one kernel is still ahead, by 1% of the step).  Steps that the attention takes with its streaming kernel
+# (a workgroup per run of a sequence's pages: ops.decode_attention_streams) repeat little of it and are
+# fused at any size.
 FUSED_DECODE_MAX_SEQS = 32
 
 
@@ -86,8 +88,9 @@ class GroupedQueryAttention(Mixer):
         qkv = rt.linear_packed(x, self.w_qkv)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
         group = self.heads // self.kv_heads
-        if (ctx.is_decode and ctx.B <= FUSED_DECODE_MAX_SEQS
-                and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, True)):
+        if (ctx.is_decode and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, True)
+                and (ctx.B <= FUSED_DECODE_MAX_SEQS
+                     or ops.decode_attention_streams(ctx.B, self.kv_heads, ctx.max_len))):
             # one token per sequence: norm, rotation, cache write and attention are one kernel
             o = ops.attention_decode_fused_bf16(qkv, self.q_gain, self.k_gain, self.eps,
                                                 self.position.rotation_table(), store.k_pages, store.v_pages,

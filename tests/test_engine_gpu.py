@@ -256,6 +256,36 @@ def test_configurations_drawn_at_random(tmp_path, seed):
             check_against_plain(folder, got, reqs, dtype_name, f"{cfg}, {what}")
 
 
+@pytest.mark.parametrize("graphs", [False, True])
+def test_a_batch_of_seventy_sequences_with_eight_kv_heads(tmp_path, graphs):
+    """512 (sequence, kv head) pairs and more: the decode attention walks each sequence's pages in one run
+    per workgroup, and the step's products go to the vendor library.  Seventy requests of unequal lengths
+    start together and decode their last tokens one by one; the shorter ones end earlier, so the batch
+    shrinks through the sizes at which the kernels change."""
+    from rust_inference_amd.engine import Engine
+    from rust_inference_amd.engine.replay import Replayer
+    from rust_inference_amd.kernels import ops
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 300, "hidden_size": 72,
+           "intermediate_size": 88, "num_hidden_layers": 2, "num_attention_heads": 16, "num_key_value_heads": 8,
+           "head_dim": 32, "rope_theta": 1e4, "rms_norm_eps": 1e-6, "tie_word_embeddings": True}
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=11, dtype=torch.bfloat16, matrix_std=0.12, gain_std=0.1)
+    rng = np.random.default_rng(70)
+    reqs = {f"r{i}": [int(t) for t in rng.integers(0, 300, n)] for i, n in enumerate(rng.integers(4, 90, 70))}
+    assert ops.decode_attention_streams(70, 8, 128)
+    steps = plans.unequal_batches([{k: (v, max(1, len(v) - int(rng.integers(1, 9)))) for k, v in reqs.items()}])
+    model = load_model(folder, torch.bfloat16)
+    cache = model.new_cache(max_tokens=plans.max_live_tokens(steps), num_slots=70, max_seq_len=128)
+    player, outs = Replayer(Engine(model, cache, use_graphs=graphs)), {}
+    for s in steps:
+        logits = player.feed(s)
+        if logits is not None:
+            outs[s["step"]] = logits.cpu().numpy().copy()
+    got = plans.collect(steps, lambda i: outs[i], 300)
+    check_against_plain(folder, got, reqs, "bfloat16", f"seventy sequences, graphs {graphs}")
+
+
 def test_a_sequence_may_pass_max_position_embeddings(model_dirs, loaded):
     """The key is read and, as in the reference, bounds nothing (src/models/config.rs:30): configuration A
     says 128 positions, the request has 150 tokens, the last 20 decoded one by one."""

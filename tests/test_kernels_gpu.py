@@ -265,6 +265,43 @@ def test_mfma_decode_attention_over_thousands_of_keys(ops, window):
         close(out, want, 1e-2, f"far key {far}, window {window}")
 
 
+@pytest.mark.parametrize("window", [None, 100, 300])
+def test_mfma_decode_attention_streams_over_many_sequences(ops, window):
+    """From 512 (sequence, kv head) pairs on a workgroup walks a sequence's pages in one run and writes the
+    output itself: 64 sequences with lengths at and around page and chunk edges, one of them with a key that
+    stands out early in a long sequence."""
+    heads, kv_heads, dh = 16, 8, 32
+    rng = np.random.default_rng(77)
+    lens = [1, 32, 33, 256, 257, 512, 700, 5, 1025, 2048, 2049, 31] + [int(n) for n in rng.integers(1, 1500, 52)]
+    assert ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 300)
+
+    def boost(qkv, k, kp, table):
+        kf = f64(kp[table[9, 40 // 32].item(), 3, 40 % 32])            # sequence 9, kv head 3: query head 6
+        qkv[9, 6 * dh:7 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+    out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, window=window,
+                               boost=boost, kernel="decode")
+    close(out, want, 1e-2, f"streaming decode attention, window {window}")
+
+
+@pytest.mark.parametrize("window", [None, 4500])
+def test_mfma_decode_attention_streams_long_sequences_in_runs(ops, window):
+    """Long sequences with 64 (sequence, kv head) pairs and more are cut into 16 runs of whole chunks each, by
+    their own lengths, and the runs are joined in order: sequences of every size in one call (most of a short
+    one's runs are empty), and in the longest a key that stands out in the first run and in a late one."""
+    heads, kv_heads, dh = 8, 8, 32
+    lens = [16400, 700, 1, 4097, 257, 33, 9000, 2048]
+    assert ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 300)
+    for far in (3, 15000):
+        rng = np.random.default_rng(41 + far)
+
+        def boost(qkv, k, kp, table, far=far):
+            kf = f64(kp[table[0, far // 32].item(), 5, far % 32])          # sequence 0, kv head 5 = query head 5
+            qkv[0, 5 * dh:6 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16,
+                                   window=window, boost=boost, kernel="decode")
+        close(out, want, 1e-2, f"far key {far}, window {window}")
+
+
 @pytest.mark.parametrize("kernel", ["prefill", "decode"])
 def test_mfma_attention_finds_one_far_key(ops, kernel):
     rng = np.random.default_rng(19)
@@ -294,20 +331,41 @@ def test_mfma_attention_window_edges(ops, kernel, window):
 def test_fused_decode_attention(ops, heads, kv_heads, dh, window):
     """Norm, rotation, cache write and attention from the raw projection, against the plain parts; twice in
     a row on the same buffers, then one token further."""
+    fused_decode_case(ops, heads, kv_heads, dh, window, [1, 32, 33, 256, 257, 512, 700, 5])
+
+
+@pytest.mark.parametrize("window", [None, 40])
+def test_fused_decode_attention_streams_over_many_sequences(ops, window):
+    """The same from 512 (sequence, kv head) pairs on, where a workgroup walks a sequence's pages in one run,
+    and the one whose run ends at the new token stores its key and value before any page is read."""
+    rng = np.random.default_rng(3)
+    lens = [1, 32, 33, 256, 257, 512, 700, 5, 31, 64, 65, 1000] + [int(n) for n in rng.integers(1, 600, 52)]
+    assert ops.decode_attention_streams(len(lens), 8, max(lens) + 301)
+    fused_decode_case(ops, 16, 8, 32, window, lens)
+
+
+def test_fused_decode_attention_streams_long_sequences_in_runs(ops):
+    """And with long sequences cut into 16 runs each: the last run that is not empty holds the new token."""
+    lens = [16400, 700, 1, 4097, 257, 33, 8191, 8192]
+    assert ops.decode_attention_streams(len(lens), 8, max(lens) + 301)
+    fused_decode_case(ops, 8, 8, 32, None, lens, steps=1, repeats=1)
+
+
+def fused_decode_case(ops, heads, kv_heads, dh, window, lens, steps=2, repeats=2):
+    """`lens`: the sequences' lengths after the first step."""
     rng = np.random.default_rng(heads * 13 + dh)
-    lens = [1, 32, 33, 256, 257, 512, 700, 5]                # lengths after this step
     B = len(lens)
     k, v, kp, vp, table = paged(rng, [n + 1 for n in lens], kv_heads, dh, dtype=torch.bfloat16, spare=12)
     width = (heads + 2 * kv_heads) * dh
     qg, kg = t(1 + 0.2 * rng.normal(size=dh)), t(1 + 0.2 * rng.normal(size=dh))
     theta, eps = 50000.0, 1e-5
     inv_freq = t(P.rope_inv_freq(dh, theta))
-    for step in range(2):
+    for step in range(steps):
         cur = [n + step for n in lens]
         pos = [n - 1 for n in cur]
         raw = t(rng.normal(size=(B, width)) * 2, torch.bfloat16)
         raw64 = f64(raw)
-        for repeat in range(2):
+        for repeat in range(repeats):
             out = ops.attention_decode_fused_bf16(raw, qg, kg, eps, inv_freq, kp, vp, t(pos, torch.int32), table, B,
                                                   max(cur) + 300, heads, kv_heads, dh, window, 1.0 / np.sqrt(dh))
             assert torch.equal(raw, t(raw64, torch.bfloat16)), "the projection is read, not changed"
