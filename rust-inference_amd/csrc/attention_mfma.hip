@@ -587,34 +587,6 @@ __device__ __forceinline__ void norm_rotate_head(bf16_t* dst_lds, const bf16_t* 
     }
 }
 
-// The new token's key and value, which its page in memory does not hold yet, put into the fragments that
-// were read from that page: key r of the page from knew, its value from vnew (both in LDS).
-template <int DH>
-__device__ __forceinline__ void patch_new_token(PageFrags<DH>& f, const bf16_t* knew, const bf16_t* vnew, int r,
-                                                int lane) {
-    const int jg = lane >> 4, col = lane & 15;
-    const int i_new = (r >> 3) * 4 + (r & 3);                // the fragment row that holds key r
-    if (col == i_new) {
-#pragma unroll
-        for (int ks = 0; ks < DH / 32; ++ks) {
-            const uint4 kv = *reinterpret_cast<const uint4*>(&knew[ks * 32 + jg * 8]);
-            if ((r & 7) >= 4) f.k[1][ks].u = kv; else f.k[0][ks].u = kv;
-        }
-    }
-    if (jg == (r >> 3)) {                                    // lanes whose eight keys include key r
-        const int e = r & 7;
-#pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) {
-            const uint32_t v = vnew[dt * 16 + col];
-            uint32_t w[4] = {f.v[dt].u.x, f.v[dt].u.y, f.v[dt].u.z, f.v[dt].u.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (k == (e >> 1)) w[k] = (e & 1) ? ((w[k] & 0x0000FFFFu) | (v << 16)) : ((w[k] & 0xFFFF0000u) | v);
-            f.v[dt].u = make_uint4(w[0], w[1], w[2], w[3]);
-        }
-    }
-}
-
 // ------------------------------------------------------------------ decode, streaming
 // When the step has keys enough to fill the machine without cutting every sequence into chunks of 256 (many
 // sequences, or very long ones), a workgroup walks a whole run of a sequence's pages instead: its four
@@ -853,7 +825,29 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
         for (int ks = 0; ks < DH / 32; ++ks)
             c.q[0][ks].u = *reinterpret_cast<const uint4*>(&q_lds[col][ks * 32 + jg * 8]);
     }
-    if (has && page == qpos / PAGE) patch_new_token<DH>(f, knew, vnew, qpos % PAGE, lane);
+    if (has && page == qpos / PAGE) {                        // the new token's key and value are not in memory yet
+        const int r = qpos % PAGE;
+        const int i_new = (r >> 3) * 4 + (r & 3);            // the fragment row that holds key r
+        if (col == i_new) {
+#pragma unroll
+            for (int ks = 0; ks < DH / 32; ++ks) {
+                const uint4 kv = *reinterpret_cast<const uint4*>(&knew[ks * 32 + jg * 8]);
+                if ((r & 7) >= 4) f.k[1][ks].u = kv; else f.k[0][ks].u = kv;
+            }
+        }
+        if (jg == (r >> 3)) {                                // lanes whose eight keys include key r
+            const int e = r & 7;
+#pragma unroll
+            for (int dt = 0; dt < DH / 16; ++dt) {
+                const uint32_t v = vnew[dt * 16 + col];
+                uint32_t w[4] = {f.v[dt].u.x, f.v[dt].u.y, f.v[dt].u.z, f.v[dt].u.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (k == (e >> 1)) w[k] = (e & 1) ? ((w[k] & 0x0000FFFFu) | (v << 16)) : ((w[k] & 0xFFFF0000u) | v);
+                f.v[dt].u = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    }
     if (has) process_page<DH, 1>(c, f, page, lane, scale_log2, false);
     finish_columns<DH, 1>(c);
 
