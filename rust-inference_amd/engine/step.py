@@ -124,6 +124,12 @@ class _DecodeGraph:
         self.logits = None
 
 
+def _decode_bound(cache, longest: int) -> int:
+    """The bound on the sequences' lengths that sizes a decode step's launches: a power of two of tokens,
+    1,024 at least, the cache's limit at most."""
+    return min(cache.max_seq_len, max(1024, 1 << (longest - 1).bit_length()))
+
+
 class Engine:
     """A model, its cache, and the step function over them.
 
@@ -191,6 +197,11 @@ class Engine:
         def piece(i, n):
             return dev[off[i]:off[i] + n]
 
+        # A decode step launched from the host gets the bound a graph of it would have: kernels that choose
+        # their form by the bound then choose alike either way, and a step's result does not depend on
+        # whether it ran as a graph.
+        if not full_width and max(counts) == 1:
+            max_len = _decode_bound(cache, max_len)
         ctx = StepContext(T=T, B=B, new_counts=counts, slot_list=slots, starts=starts,
                           tokens=piece(0, T), tok_seq=piece(1, T), tok_pos=piece(2, T), cu_seqlens=piece(3, B + 1),
                           slots=piece(4, B), len_after=piece(5, B), want_rows=piece(6, len(want)),
@@ -220,8 +231,7 @@ class Engine:
         # as much as two or three steps).  Finer bounds were tried and gained nothing: the workgroups of
         # the empty chunks come last in the grid and cost little there.
         slots = np.fromiter((e.slot for e in entries), dtype=np.int32, count=batch)
-        longest = self.cache.longest(slots) + 1
-        bound = min(self.cache.max_seq_len, max(1024, 1 << (longest - 1).bit_length()))
+        bound = _decode_bound(self.cache, self.cache.longest(slots) + 1)
         dg = self._graphs.get((batch, bound))
         if dg is None:
             dg = self._graphs[(batch, bound)] = _DecodeGraph(batch, self.device)

@@ -286,6 +286,39 @@ def test_a_batch_of_seventy_sequences_with_eight_kv_heads(tmp_path, graphs):
     check_against_plain(folder, got, reqs, "bfloat16", f"seventy sequences, graphs {graphs}")
 
 
+def test_graphs_and_host_launches_choose_the_same_kernels(tmp_path):
+    """Eight sequences of 8,200 to 8,300 tokens with eight kv heads: a graph of the decode step is sized for
+    16,384 tokens, where the attention walks runs of pages, while the lengths themselves would still get a
+    workgroup per chunk of 256 keys.  A step launched from the host takes the graph's bound, so both give the
+    same logits bit for bit, and the logits of the plain implementation within rounding."""
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.kernels import ops
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 300, "hidden_size": 72,
+           "intermediate_size": 88, "num_hidden_layers": 1, "num_attention_heads": 8, "num_key_value_heads": 8,
+           "head_dim": 32, "rope_theta": 1e4, "rms_norm_eps": 1e-6, "tie_word_embeddings": True}
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=12, dtype=torch.bfloat16, matrix_std=0.12, gain_std=0.1)
+    assert ops.decode_attention_streams(8, 8, 16384) and not ops.decode_attention_streams(8, 8, 8310)
+    rng = np.random.default_rng(8)
+    prompts = [[int(t) for t in rng.integers(0, 300, n)] for n in rng.integers(8200, 8300, 8)]
+    nxt = [[int(t) for t in rng.integers(0, 300, 3)] for _ in prompts]
+    model = load_model(folder, torch.bfloat16)
+    outs = []
+    for graphs in (False, True):
+        cache = model.new_cache(max_tokens=8 * 8320, num_slots=8, max_seq_len=20000)
+        engine = Engine(model, cache, use_graphs=graphs)
+        slots = [cache.acquire() for _ in prompts]
+        engine.step([StepEntry(s, p, []) for s, p in zip(slots, prompts)])
+        outs.append([engine.step([StepEntry(s, [t[i]], "last") for s, t in zip(slots, nxt)]).clone() for i in range(3)])
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    # the last step against the plain implementation, for the longest request
+    i = int(np.argmax([len(p) for p in prompts]))
+    want = plain_logits(folder, prompts[i] + nxt[i])[-1:]
+    assert_logits_close(outs[1][2][i:i + 1].cpu().numpy(), want, "bfloat16", f"request {i} of {len(prompts[i]) + 3} tokens")
+
+
 def test_a_sequence_may_pass_max_position_embeddings(model_dirs, loaded):
     """The key is read and, as in the reference, bounds nothing (src/models/config.rs:30): configuration A
     says 128 positions, the request has 150 tokens, the last 20 decoded one by one."""
