@@ -130,6 +130,13 @@ def _decode_bound(cache, longest: int) -> int:
     return min(cache.max_seq_len, max(1024, 1 << (longest - 1).bit_length()))
 
 
+# Graphs an engine keeps: one per batch size and bound that a step has had.  A batch that shrinks as its
+# sequences end passes through every size below its first, and each graph holds the step's buffers (the
+# logits of its batch among them); past this many the graph that has gone unused the longest is dropped and
+# captured again if its size comes back.
+MAX_GRAPHS = 96
+
+
 class Engine:
     """A model, its cache, and the step function over them.
 
@@ -143,7 +150,8 @@ class Engine:
         self.device = model.rt.device
         self.use_graphs = use_graphs
         self._staging = None
-        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}       # in order of last use
+        self.max_graphs = MAX_GRAPHS
 
     def _stage(self, n: int) -> _Staging:
         if self._staging is None or self._staging.capacity < n:
@@ -232,8 +240,12 @@ class Engine:
         # the empty chunks come last in the grid and cost little there.
         slots = np.fromiter((e.slot for e in entries), dtype=np.int32, count=batch)
         bound = _decode_bound(self.cache, self.cache.longest(slots) + 1)
-        dg = self._graphs.get((batch, bound))
-        if dg is None:
+        dg = self._graphs.pop((batch, bound), None)
+        if dg is not None:
+            self._graphs[(batch, bound)] = dg                # the most recently used sits last
+        else:
+            while len(self._graphs) >= max(1, self.max_graphs):
+                self._graphs.pop(next(iter(self._graphs)))   # the one unused the longest
             dg = self._graphs[(batch, bound)] = _DecodeGraph(batch, self.device)
             width = self.cache.max_pages_per_slot
             need = 7 * (batch + 5) + len(self.cache.groups) * (batch * width + 4)

@@ -128,6 +128,31 @@ def test_graph_and_eager_decoding_give_the_same_logits(model_dirs, name, lengths
         assert torch.equal(a, b), "a captured step must compute what the launched one computes"
 
 
+def test_an_engine_keeps_a_bounded_number_of_graphs(model_dirs):
+    """With room for one graph, steps that alternate between two batch sizes drop and capture a graph every
+    time; the logits stay those of the launched steps, and the engine never holds more than it may."""
+    import torch
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.parts import load_model
+    model = load_model(model_dirs["B"], torch.bfloat16)
+    cfg, _ = read_model_f64(model_dirs["B"])
+    prompts = prompts_for(cfg, [33, 2, 40], 5)
+    outs = []
+    for graphs in (False, True):
+        eng = Engine(model, model.new_cache(max_tokens=3 * 96, num_slots=3, max_seq_len=96), use_graphs=graphs)
+        eng.max_graphs = 1
+        slots = [eng.cache.acquire() for _ in prompts]
+        eng.step([StepEntry(s, p, "last") for s, p in zip(slots, prompts)])
+        rows = []
+        for step in range(8):
+            live = slots if step % 2 == 0 else slots[:2]
+            rows.append(eng.step([StepEntry(s, [(5 * step + s) % 300], "last") for s in live]).clone())
+            assert len(eng._graphs) <= 1
+        outs.append(rows)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
 def test_temperature_sampling_is_seeded(model_dirs):
     from rust_inference_amd import Model
     cfg, _ = read_model_f64(model_dirs["A"])
