@@ -265,19 +265,20 @@ def test_mfma_decode_attention_over_thousands_of_keys(ops, window):
         close(out, want, 1e-2, f"far key {far}, window {window}")
 
 
-@pytest.mark.parametrize("window", [None, 100, 300])
-def test_mfma_decode_attention_streams_over_many_sequences(ops, window):
+@pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 100), (16, 8, 32, 300),
+                                                         (32, 8, 128, None), (32, 8, 128, 300), (8, 8, 64, None)])
+def test_mfma_decode_attention_streams_over_many_sequences(ops, heads, kv_heads, dh, window):
     """From 512 (sequence, kv head) pairs on a workgroup walks a sequence's pages in one run and writes the
     output itself: 64 sequences with lengths at and around page and chunk edges, one of them with a key that
     stands out early in a long sequence."""
-    heads, kv_heads, dh = 16, 8, 32
     rng = np.random.default_rng(77)
     lens = [1, 32, 33, 256, 257, 512, 700, 5, 1025, 2048, 2049, 31] + [int(n) for n in rng.integers(1, 1500, 52)]
     assert ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 300)
 
     def boost(qkv, k, kp, table):
-        kf = f64(kp[table[9, 40 // 32].item(), 3, 40 % 32])            # sequence 9, kv head 3: query head 6
-        qkv[9, 6 * dh:7 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        head = 3 * (heads // kv_heads)                                 # sequence 9, kv head 3: its first query head
+        kf = f64(kp[table[9, 40 // 32].item(), 3, 40 % 32])
+        qkv[9, head * dh:(head + 1) * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
     out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, window=window,
                                boost=boost, kernel="decode")
     close(out, want, 1e-2, f"streaming decode attention, window {window}")
@@ -334,21 +335,23 @@ def test_fused_decode_attention(ops, heads, kv_heads, dh, window):
     fused_decode_case(ops, heads, kv_heads, dh, window, [1, 32, 33, 256, 257, 512, 700, 5])
 
 
-@pytest.mark.parametrize("window", [None, 40])
-def test_fused_decode_attention_streams_over_many_sequences(ops, window):
+@pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 40), (32, 8, 128, None),
+                                                         (32, 8, 128, 40), (16, 8, 64, None)])
+def test_fused_decode_attention_streams_over_many_sequences(ops, heads, kv_heads, dh, window):
     """The same from 512 (sequence, kv head) pairs on, where a workgroup walks a sequence's pages in one run,
     and the one whose run ends at the new token stores its key and value before any page is read."""
     rng = np.random.default_rng(3)
     lens = [1, 32, 33, 256, 257, 512, 700, 5, 31, 64, 65, 1000] + [int(n) for n in rng.integers(1, 600, 52)]
-    assert ops.decode_attention_streams(len(lens), 8, max(lens) + 301)
-    fused_decode_case(ops, 16, 8, 32, window, lens)
+    assert ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 301)
+    fused_decode_case(ops, heads, kv_heads, dh, window, lens, steps=2 if dh == 32 else 1, repeats=2 if dh == 32 else 1)
 
 
-def test_fused_decode_attention_streams_long_sequences_in_runs(ops):
+@pytest.mark.parametrize("heads, kv_heads, dh", [(8, 8, 32), (32, 8, 128)])
+def test_fused_decode_attention_streams_long_sequences_in_runs(ops, heads, kv_heads, dh):
     """And with long sequences cut into 16 runs each: the last run that is not empty holds the new token."""
     lens = [16400, 700, 1, 4097, 257, 33, 8191, 8192]
-    assert ops.decode_attention_streams(len(lens), 8, max(lens) + 301)
-    fused_decode_case(ops, 8, 8, 32, None, lens, steps=1, repeats=1)
+    assert ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 301)
+    fused_decode_case(ops, heads, kv_heads, dh, None, lens, steps=1, repeats=1)
 
 
 def fused_decode_case(ops, heads, kv_heads, dh, window, lens, steps=2, repeats=2):
