@@ -463,7 +463,8 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
     const int d = threadIdx.x % DH, tp = threadIdx.x / DH;
     const int qpos = tok_pos[b];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    const int c_lo = lo / DECODE_CHUNK, c_hi = qpos / DECODE_CHUNK;
+    // window < 0: the entries are the runs of the streaming kernel, all of them written
+    const int c_lo = window < 0 ? 0 : lo / DECODE_CHUNK, c_hi = window < 0 ? max_chunks - 1 : qpos / DECODE_CHUNK;
     const int n = c_hi - c_lo + 1;
     const int parts = n <= JOIN_SERIAL ? 1 : JOIN_PARTS;
     const int per = (n + parts - 1) / parts;
@@ -595,7 +596,8 @@ __device__ __forceinline__ void norm_rotate_head(bf16_t* dst_lds, const bf16_t* 
 // system then sees one long stream per wavefront rather than a burst per workgroup with a start and an end
 // around it.  A sequence is cut into `splits` runs of whole chunks by its own length alone; with one run the
 // kernel writes the output itself and no join follows, with more the runs' results go to the workspace
-// [seqs, heads, splits, DH + 2] and the join adds them in run order.
+// [seqs, heads, splits, DH + 2] and the join adds them in run order (more than 16 of them in eight groups
+// side by side, as it does with chunks).
 #define STREAM_WAVES 4
 
 // FUSED: qkv is the raw projection; the kernel norms and rotates the group's queries for itself, and the
@@ -736,17 +738,22 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 }
 
 // Runs per sequence of the streaming kernel for a step of `seqs` sequences of up to `max_chunks` chunks, or 0
-// where the kernel of one workgroup per chunk is the faster one.  It depends on the step's size alone.
+// where the kernel of one workgroup per chunk is the faster one.  It depends on the step's size alone: one
+// run where there are 512 (sequence, kv head) pairs or more, else as many runs as bring the workgroups to
+// about a thousand, of eight chunks (64 pages, 16 a wavefront) at least, if that still makes 512 workgroups.
 // Measured at 8 kv heads of 128: with 64 sequences of 2,080 keys one run per sequence (512 workgroups, no
 // join) takes 94 us where the chunks and their join take 97 + 6; 8 sequences of 32,800 keys in 16 runs make
-// the step 2% shorter; with fewer workgroups than that the streams are too few to keep the memory busy (one
-// sequence of 131,000 keys in 16 runs: 12% longer), and at 32 or 48 sequences of 2,080 keys runs that still
-// need a join lose by 2%.
+// the step 2% shorter, 4 of them 2%, one sequence of 131,000 keys in 64 runs 10%.  Fewer or shorter streams
+// do not keep the memory busy (one sequence of 131,000 keys in 16 runs: 12% longer; runs of four chunks: no
+// gain), and at 32 or 48 sequences of 2,080 keys runs that still need a join lose by 2%.
+#define STREAM_WORKGROUPS 1024
+#define STREAM_MIN_CHUNKS 8
 static int stream_splits(int seqs, int kv_heads, int max_chunks) {
     const long rows = (long)seqs * kv_heads;
     if (rows >= 512) return 1;
-    if (rows >= 64 && max_chunks >= 64) return min(JOIN_SERIAL, max_chunks);
-    return 0;
+    const long splits = min((STREAM_WORKGROUPS + rows - 1) / rows, (long)max_chunks / STREAM_MIN_CHUNKS);
+    if (splits < 2 || rows * splits < 512) return 0;
+    return (int)splits;
 }
 
 extern "C" int ri_attention_decode_streams(int seqs, int kv_heads, int max_chunks) {
@@ -975,9 +982,7 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
             (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,                \
             (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,        \
             scale_log2, splits, tiled_out);                                                                       \
-        if (splits > 1)                                                                                           \
-            attn_decode_join_small_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos,  \
-                                                                               heads, -1, splits, tiled_out);     \
+        if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {
             RI_STREAM_CASE(32)
@@ -1034,9 +1039,7 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
             (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,                 \
             (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,        \
             scale_log2, splits, tiled_out);                                                                       \
-        if (splits > 1)                                                                                           \
-            attn_decode_join_small_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>((bf16_t*)out, workspace, tok_pos,  \
-                                                                               heads, -1, splits, tiled_out);     \
+        if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {
             RI_STREAM_CASE(32)

@@ -303,6 +303,25 @@ def test_mfma_decode_attention_streams_long_sequences_in_runs(ops, window):
         close(out, want, 1e-2, f"far key {far}, window {window}")
 
 
+def test_mfma_decode_attention_streams_one_very_long_sequence(ops):
+    """Two sequences, one of 66,000 keys: 33 runs each, joined in eight groups side by side; the short
+    sequence's runs are empty but the first.  A key that stands out in the first run, in a middle one, in the
+    last."""
+    heads, kv_heads, dh = 8, 8, 32
+    lens = [66000, 300]
+    assert ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 300)
+    for far in (100, 33000, 65990):
+        rng = np.random.default_rng(51 + far)
+
+        def boost(qkv, k, kp, table, far=far):
+            kf = f64(kp[table[0, far // 32].item(), 2, far % 32])          # sequence 0, kv head 2 = query head 2
+            qkv[0, 2 * dh:3 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, boost=boost,
+                                   kernel="decode")
+        close(out, want, 1e-2, f"far key {far}")
+        assert np.abs(want[0, 2]).max() > 0
+
+
 @pytest.mark.parametrize("kernel", ["prefill", "decode"])
 def test_mfma_attention_finds_one_far_key(ops, kernel):
     rng = np.random.default_rng(19)
