@@ -739,18 +739,22 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 
 // Runs per sequence of the streaming kernel for a step of `seqs` sequences of up to `max_chunks` chunks, or 0
 // where the kernel of one workgroup per chunk is the faster one.  It depends on the step's size alone: one
-// run where there are 512 (sequence, kv head) pairs or more, else as many runs as bring the workgroups to
-// about a thousand, of eight chunks (64 pages, 16 a wavefront) at least, if that still makes 512 workgroups.
+// run where there are 512 (sequence, kv head) pairs or more; else, from 64 chunks (16,384 keys) on, as many
+// runs as bring the workgroups to about a thousand, of eight chunks (64 pages, 16 a wavefront) at least, if
+// that still makes 512 workgroups.
 // Measured at 8 kv heads of 128: with 64 sequences of 2,080 keys one run per sequence (512 workgroups, no
 // join) takes 94 us where the chunks and their join take 97 + 6; 8 sequences of 32,800 keys in 16 runs make
 // the step 2% shorter, 4 of them 2%, one sequence of 131,000 keys in 64 runs 10%.  Fewer or shorter streams
 // do not keep the memory busy (one sequence of 131,000 keys in 16 runs: 12% longer; runs of four chunks: no
-// gain), and at 32 or 48 sequences of 2,080 keys runs that still need a join lose by 2%.
+// gain), and runs that need a join lose at a few thousand keys (2 runs at 48 sequences of 2,080 keys: -2.5%;
+// 4 runs at 16 sequences of 4,100: -1.5%; 32 sequences of 4,100 gain 2.5% and are left to the chunks with them).
 #define STREAM_WORKGROUPS 1024
 #define STREAM_MIN_CHUNKS 8
+#define STREAM_JOINED_FROM 64
 static int stream_splits(int seqs, int kv_heads, int max_chunks) {
     const long rows = (long)seqs * kv_heads;
     if (rows >= 512) return 1;
+    if (max_chunks < STREAM_JOINED_FROM) return 0;
     const long splits = min((STREAM_WORKGROUPS + rows - 1) / rows, (long)max_chunks / STREAM_MIN_CHUNKS);
     if (splits < 2 || rows * splits < 512) return 0;
     return (int)splits;
