@@ -23,9 +23,14 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 // every lane's 16-byte pieces stay aligned and the split depends on K alone); their sums are added
 // through LDS in wavefront order.  More wavefronts in flight per byte: it pays when the matrix has few
 // rows or long ones.
-#define GV_PRE 4              // partial sums of squares a thread fetches ahead of the weights
+// Partial sums of squares a thread fetches ahead of the weights.  A row has as many as the product before
+// wrote workgroups (up to 4,096 at Qwen3-8B sizes); what is not fetched ahead is fetched after the stream, one
+// more trip to memory at the end of every workgroup.  Sixteen a thread cover 4,096 (decode at batch 1: +1.5%);
+// where a row has 1,024 at most, four do, and the registers of more cost a small model 1.5%.
+#define GV_PRE_FEW 4
+#define GV_PRE_MANY 16
 
-template <int MT, bool SWIGLU, typename TO, int KS>
+template <int MT, bool SWIGLU, typename TO, int KS, int GV_PRE>
 __global__ void __launch_bounds__(GV_WAVES * RI_WAVE)
 gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N, int K,
                  NormLink link) {
@@ -176,12 +181,19 @@ template <int MT, bool SWIGLU, int KS>
 static void launch_gemv_ks(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
                            const NormLink& link, hipStream_t s) {
     const unsigned grid = gemv_grid(n, k);
-    if (out_dtype == RI_F32)
-        gemv_bf16_kernel<MT, SWIGLU, float, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>((float*)out, (const bf16_t*)x,
-                                                                                    (const bf16_t*)w, m, n, k, link);
-    else
-        gemv_bf16_kernel<MT, SWIGLU, bf16_t, KS><<<grid, GV_WAVES * RI_WAVE, 0, s>>>(
+    // one row of x whose norm is still to finish, with more partial sums than four a thread cover
+    const bool many = MT == 1 && link.ssq_in && link.n_in > GV_PRE_FEW * GV_WAVES * RI_WAVE;
+    if (out_dtype == RI_F32) {
+        if (many) gemv_bf16_kernel<MT, SWIGLU, float, KS, MT == 1 ? GV_PRE_MANY : GV_PRE_FEW><<<grid, GV_WAVES * RI_WAVE, 0, s>>>(
+            (float*)out, (const bf16_t*)x, (const bf16_t*)w, m, n, k, link);
+        else gemv_bf16_kernel<MT, SWIGLU, float, KS, GV_PRE_FEW><<<grid, GV_WAVES * RI_WAVE, 0, s>>>(
+            (float*)out, (const bf16_t*)x, (const bf16_t*)w, m, n, k, link);
+    } else {
+        if (many) gemv_bf16_kernel<MT, SWIGLU, bf16_t, KS, MT == 1 ? GV_PRE_MANY : GV_PRE_FEW><<<grid, GV_WAVES * RI_WAVE, 0, s>>>(
             (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, m, n, k, link);
+        else gemv_bf16_kernel<MT, SWIGLU, bf16_t, KS, GV_PRE_FEW><<<grid, GV_WAVES * RI_WAVE, 0, s>>>(
+            (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w, m, n, k, link);
+    }
 }
 
 template <int MT, bool SWIGLU>
