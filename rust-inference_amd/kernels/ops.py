@@ -274,11 +274,17 @@ def attention_prefill_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_tabl
     return out
 
 
+def decode_attention_runs(seqs: int, kv_heads: int, max_len: int) -> int:
+    """The runs per sequence in which the decode attention's streaming kernel walks a step of this size, or 0
+    where it takes one workgroup per chunk of 256 keys instead (host code only: it needs no GPU)."""
+    chunks = _get("ri_attention_decode_chunks")(int(max_len))
+    return _get("ri_attention_decode_streams")(int(seqs), int(kv_heads), chunks)
+
+
 def decode_attention_streams(seqs: int, kv_heads: int, max_len: int) -> bool:
     """Whether ``attention_decode_bf16`` walks a step of this size with its streaming kernel (whole runs of a
     sequence's pages per workgroup) rather than with one workgroup per chunk of 256 keys."""
-    chunks = _get("ri_attention_decode_chunks")(int(max_len))
-    return _get("ri_attention_decode_streams")(int(seqs), int(kv_heads), chunks) > 0
+    return decode_attention_runs(seqs, kv_heads, max_len) > 0
 
 
 def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table, seqs: int, max_len: int,

@@ -230,3 +230,25 @@ def test_runner_refuses_what_it_cannot_do(tmp_path, capsys):
     assert "tokenizer.json" in capsys.readouterr().err
     assert main([str(tmp_path), "-p", ""]) == 1
     assert "empty prompt" in capsys.readouterr().err
+
+
+def test_the_bound_that_sizes_a_decode_step():
+    """A power of two of tokens, 1,024 at least, the cache's limit at most: the same for a step that is
+    launched from the host and for its graph."""
+    from types import SimpleNamespace
+    from rust_inference_amd.engine.step import _decode_bound
+    cache = SimpleNamespace(max_seq_len=20000)
+    assert [_decode_bound(cache, n) for n in (1, 1024, 1025, 4096, 4097, 16384, 16385, 30000)] == \
+        [1024, 1024, 2048, 4096, 8192, 16384, 20000, 20000]
+
+
+def test_which_decode_steps_the_attention_walks_in_runs():
+    """The rule is host code of the kernel library: one run a sequence from 512 (sequence, kv head) pairs on;
+    below that, runs of eight chunks and more that make 512 workgroups, from 16,384 keys on; else chunks."""
+    from rust_inference_amd.kernels import ops
+    runs = ops.decode_attention_runs
+    assert runs(64, 8, 2100) == 1 and runs(256, 2, 300) == 1 and runs(63, 8, 2100) == 0
+    assert runs(8, 8, 32896) == 16 and runs(4, 8, 32896) == 16 and runs(1, 8, 131200) == 64
+    assert runs(1, 8, 32896) == 0                      # 16 runs of eight chunks would be 128 workgroups
+    assert runs(16, 8, 4200) == 0 and runs(48, 8, 2100) == 0 and runs(32, 8, 8192) == 0
+    assert runs(8, 8, 16384) == 8 and runs(8, 8, 16000) == 0
