@@ -136,6 +136,16 @@ int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* 
 int ri_argmax_workspace_bytes(int rows);
 int ri_argmax(int32_t* ids, const float* logits, void* workspace, int rows, int vocab, void* stream);
 
+// ri_argmax for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+// loops, harnesses that forbid hipMalloc): the workspace is a device array built into the library, half a
+// megabyte that each GPU the library runs on holds until the process ends, for at most
+// ri_argmax_static_max_rows() = 1024 rows; more rows are refused.  It calls no allocating routine.  The
+// reference has no counterpart (its argmax allocates its result: src/cuda/ops.rs:251-260).  Every call on a GPU uses
+// that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls in stream order
+// do not.  Same result as ri_argmax.
+int ri_argmax_static_max_rows(void);
+int ri_argmax_static(int32_t* ids, const float* logits, int rows, int vocab, void* stream);
+
 // Next-token selection, one row of float32 logits per sequence: repetition penalty over the token ids
 // marked in seen (a byte per vocabulary entry; row seen_rows[r] of it, or row r when seen_rows is NULL;
 // seen may be NULL), greedy when temperature <= 0, else temperature, top-k (0: off), top-p (1: off) and

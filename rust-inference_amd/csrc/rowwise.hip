@@ -1,5 +1,7 @@
 // Row-wise kernels: embedding gather, fused residual add + RMSNorm, SwiGLU, argmax.
 // One workgroup per row; all statistics in float32.
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -313,4 +315,47 @@ extern "C" int ri_argmax(int32_t* ids, const float* logits, void* workspace, int
     argmax_pick_kernel<<<rows, ARGMAX_SLICES, 0, s>>>(ids, part_v, part_i);
     RI_LAUNCH_CHECK("argmax");
     return 0;
+}
+
+// ---- the same argmax for callers that cannot allocate device memory
+// The (value, index) pairs of stage one lie in a file-scope device array instead of a workspace the caller
+// brings.  In host code the array's name stands for the symbol, not for its device address: the address is
+// asked for once per device (each GPU holds its own copy at its own address) and only that pointer is used
+// afterwards.  Every call on a GPU shares that GPU's array, so calls that overlap on one GPU race.
+#define ARGMAX_STATIC_MAX_ROWS 1024
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[ARGMAX_STATIC_MAX_ROWS * ARGMAX_SLICES * 8];
+
+static void* g_scratch_of_device[ARGMAX_STATIC_MAX_DEVICES];      // per device: the array's address there
+static std::mutex g_scratch_mutex;
+
+// The address of `scratch` on the current device (looked up at the first call on that device).
+static int scratch_of_current_device(void** out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    RI_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+    RI_REQUIRE(device >= 0 && device < ARGMAX_STATIC_MAX_DEVICES, "argmax_static: device %d is beyond the %d this library "
+               "keeps an address for", device, ARGMAX_STATIC_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    if (g_scratch_of_device[device] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        RI_REQUIRE(e == hipSuccess && ptr != nullptr, "argmax_static: hipGetSymbolAddress on device %d: %s", device,
+                   hipGetErrorString(e));
+        g_scratch_of_device[device] = ptr;
+    }
+    *out = g_scratch_of_device[device];
+    return 0;
+}
+
+extern "C" int ri_argmax_static_max_rows(void) { return ARGMAX_STATIC_MAX_ROWS; }
+
+extern "C" int ri_argmax_static(int32_t* ids, const float* logits, int rows, int vocab, void* stream) {
+    RI_REQUIRE(rows > 0 && vocab > 0, "argmax_static: rows %d, vocab %d", rows, vocab);
+    RI_REQUIRE(rows <= ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows, the built-in scratch holds %d at most "
+               "(use ri_argmax with a workspace of the caller's)", rows, ARGMAX_STATIC_MAX_ROWS);
+    void* ptr = nullptr;
+    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    // stage one writes every (value, index) pair that stage two reads: nothing has to start at zero
+    return ri_argmax(ids, logits, ptr, rows, vocab, stream);
 }
