@@ -2,12 +2,16 @@
 
 The model says which tensors it wants (name, shape, kind); the loader compares
 that with the folder and raises ONE error that lists every missing tensor, every
-unexpected one and every wrong shape.  Tensors keep the dtype they are stored in:
+wrong shape and dtype, and with them the tensors the model did not expect.  A folder
+whose only oddity is tensors the model does not read loads, as it does in the
+reference, which looks tensors up by name and never lists the rest
+(src/safetensors.rs:157-174); they are named in one warning.  Tensors keep the dtype they are stored in:
 bfloat16 stays bfloat16 and a tensor stored in 32-bit stays 32-bit; integer tables
 become int32.
 """
 from __future__ import annotations
 
+import warnings
 from dataclasses import dataclass
 
 import torch
@@ -40,7 +44,9 @@ def check_folder(folder: ModelFolder, expected: dict[str, TensorSpec]) -> None:
         info = folder.info(name)
         if tuple(info.shape) != tuple(spec.shape):
             misshapen.append(f"{name}: file has {list(info.shape)}, model wants {list(spec.shape)}")
-        if spec.kind == TABLE:
+        if info.dtype is None:
+            wrong_dtype.append(f"{name}: stored as {info.stored_as}, which this library does not read")
+        elif spec.kind == TABLE:
             if info.dtype not in (torch.int32, torch.int64):
                 wrong_dtype.append(f"{name}: {info.dtype} is not an integer table")
         elif info.dtype not in _KEPT:
@@ -48,7 +54,12 @@ def check_folder(folder: ModelFolder, expected: dict[str, TensorSpec]) -> None:
     for name in folder.names():
         if name not in expected:
             unexpected.append(name)
-    if missing or unexpected or misshapen or wrong_dtype:
+    if unexpected and not (missing or misshapen or wrong_dtype):
+        shown = ", ".join(unexpected[:8]) + (f" and {len(unexpected) - 8} more" if len(unexpected) > 8 else "")
+        warnings.warn(f"{folder.model_dir}: {len(unexpected)} tensors that the model does not read are ignored: {shown}",
+                      stacklevel=3)
+        return
+    if missing or misshapen or wrong_dtype:
         parts = []
         if missing:
             parts.append(f"missing ({len(missing)}): " + ", ".join(missing))

@@ -32,10 +32,11 @@ _NAMES = {v[0]: k for k, v in _DTYPES.items()}
 
 @dataclass(frozen=True)
 class TensorInfo:
-    dtype: torch.dtype
+    dtype: torch.dtype | None   # None: stored in a format this library does not read (see stored_as)
     shape: tuple
     start: int      # byte offsets into the file
     end: int
+    stored_as: str = ""         # the file's own name of the dtype
 
 
 class SafeTensorFile:
@@ -63,17 +64,17 @@ class SafeTensorFile:
         for name, raw in header.items():
             if name == "__metadata__":
                 continue
-            if raw["dtype"] not in _DTYPES:
-                raise UnsupportedError(f"{path}: tensor {name} has dtype {raw['dtype']}, supported: {', '.join(_DTYPES)}")
-            dtype, esize = _DTYPES[raw["dtype"]]
+            # a tensor in a format this library does not read (F16, U8, BOOL, ...) is refused when it is
+            # asked for, not when the file is opened: a folder may hold such tensors beside the model's
+            dtype, esize = _DTYPES.get(raw["dtype"], (None, None))
             shape = tuple(int(s) for s in raw["shape"])
             start, end = base + int(raw["data_offsets"][0]), base + int(raw["data_offsets"][1])
             numel = 1
             for s in shape:
                 numel *= s
-            if end - start != numel * esize or end > size or start < base:
+            if end > size or start < base or end < start or (esize is not None and end - start != numel * esize):
                 raise WeightsError(f"{path}: bad data offsets for {name}")
-            self.tensors[name] = TensorInfo(dtype, shape, start, end)
+            self.tensors[name] = TensorInfo(dtype, shape, start, end, str(raw["dtype"]))
 
     def names(self):
         return self.tensors.keys()
@@ -81,6 +82,8 @@ class SafeTensorFile:
     def load(self, name: str) -> torch.Tensor:
         """A read-only view of the mapped bytes as a tensor (copy it before writing)."""
         info = self.tensors[name]
+        if info.dtype is None:
+            raise UnsupportedError(f"{self.path}: tensor {name} has dtype {info.stored_as}, supported: {', '.join(_DTYPES)}")
         if info.end == info.start:
             return torch.empty(info.shape, dtype=info.dtype)
         with warnings.catch_warnings():

@@ -19,6 +19,16 @@ def read_model_f64(model_dir):
     return cfg, w
 
 
+def reference_fixture(name):
+    """The folder `tests/fixtures/<name>` of the reference, or None when it is not at hand: the folder the
+    environment variable RI_REFERENCE_FIXTURES names, else `reference/tests/fixtures` beside this checkout."""
+    here = os.path.dirname(os.path.dirname(os.path.realpath(__file__)))
+    for base in (os.environ.get("RI_REFERENCE_FIXTURES"), os.path.join(os.path.dirname(here), "reference", "tests", "fixtures")):
+        if base and os.path.isfile(os.path.join(base, name, "config.json")):
+            return os.path.join(base, name)
+    return None
+
+
 def rel_to_max(got, want):
     got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, f"shape {got.shape} against {want.shape}"

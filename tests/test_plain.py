@@ -10,8 +10,10 @@ import torch
 
 from plain import qwen3_plain as P
 
-FIXTURE = "/root/reference/tests/fixtures/tiny-qwen3"
-needs_fixture = pytest.mark.skipif(not os.path.exists(FIXTURE), reason="the reference tree is not mounted")
+from helpers import reference_fixture
+
+FIXTURE = reference_fixture("tiny-qwen3")
+needs_fixture = pytest.mark.skipif(FIXTURE is None, reason="the reference's fixtures are not at hand (RI_REFERENCE_FIXTURES)")
 
 
 def fixture_model():

@@ -54,8 +54,10 @@ def test_bad_files_are_refused(tmp_path):
         SafeTensorFile(str(p))
     header = json.dumps({"w": {"dtype": "F8_E4M3", "shape": [4], "data_offsets": [0, 4]}}).encode()
     p.write_bytes(struct.pack("<Q", len(header)) + header + b"\0" * 4)
+    f8 = SafeTensorFile(str(p))                          # a format this library does not read is refused when
+    assert f8.tensors["w"].dtype is None                 # the tensor is asked for, not when the file is opened
     with pytest.raises(UnsupportedError, match="F8_E4M3"):
-        SafeTensorFile(str(p))
+        f8.load("w")
     with pytest.raises(WeightsError, match="neither"):
         ModelFolder(str(tmp_path / "nowhere"))
 
@@ -85,6 +87,27 @@ def test_random_model_folder_loads_and_is_seeded(tmp_path):
     tied = write_random_model(str(tmp_path / "m4"), TINY_A, seed=0, dtype=torch.float32)
     wt = load_checked(tied, expected_tensors(spec_of(TINY_A)))
     assert "lm_head.weight" not in wt and wt["model.embed_tokens.weight"].dtype == torch.float32
+
+
+def test_tensors_the_model_does_not_read_are_ignored_with_a_warning(tmp_path):
+    """The reference looks tensors up by name and never lists the rest (src/safetensors.rs:157-174): a folder
+    with a buffer of another kind beside the model's tensors loads; an expected tensor in such a format does not."""
+    d = write_random_model(str(tmp_path / "m"), TINY_A, seed=0)
+    f = ModelFolder(d)
+    t = {n: f.load(n).clone() for n in f.names()}
+    t["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.zeros(8, dtype=torch.float16)
+    t["model.masked_bias"] = torch.zeros(3, dtype=torch.uint8)
+    os.remove(os.path.join(d, "model.safetensors"))
+    from safetensors.torch import save_file as st_save
+    st_save(t, os.path.join(d, "model.safetensors"))
+    exp = expected_tensors(spec_of(TINY_A))
+    with pytest.warns(UserWarning, match="2 tensors that the model does not read are ignored.*masked_bias"):
+        w = load_checked(d, exp)
+    assert set(w) == set(exp) - {"lm_head.weight"}
+    t["model.norm.weight"] = t["model.norm.weight"].to(torch.float16)
+    st_save(t, os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError, match=r"wrong dtype \(1\): model.norm.weight: stored as F16"):
+        load_checked(d, exp)
 
 
 def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
