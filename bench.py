@@ -11,6 +11,7 @@ greedily on the device.  Prints one JSON line: decoded tokens a second at batch 
 """
 import argparse
 import json
+import os
 import sys
 import time
 
@@ -89,6 +90,10 @@ def main() -> int:
     cfg["max_position_embeddings"] = args.context
     torch.manual_seed(2)
     model = random_model(cfg, seed=2, dtype=torch.bfloat16)
+    if os.environ.get("RI_PREFETCH"):                      # experiment switch: prefetch weights beside the products
+        from rust_inference_amd.parts.runtime import WeightStream
+        model.rt.weight_stream = WeightStream(model.rt.device, int(os.environ.get("RI_PREFETCH_WGS", 512)),
+                                              int(os.environ.get("RI_PREFETCH_AHEAD", 1)))
     vocab = cfg["vocab_size"]
     gen = torch.Generator().manual_seed(2)
 

@@ -25,6 +25,7 @@ int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const void* pendin
                    int tiled, void* stream);
 
 // Plain residual add on gathered rows, no norm: out[row] = residual[src] + pending[src], float32.
+// With rows == NULL out may be residual itself (an add in place).
 int ri_add_rows(float* out, const float* residual, const void* pending, int pending_dtype,
                 const int32_t* rows, int n_rows, int dim, void* stream);
 
@@ -35,6 +36,8 @@ int ri_add_rows(float* out, const float* residual, const void* pending, int pend
 // inside a page): [pages, kv_heads, head_dim, page_size], both of cache_dtype.
 // cu_seqlens (int32 [seqs + 1], may be NULL), seqs and max_new (most new tokens of a sequence) let values be
 // written a page at a time; without them every element is written on its own.
+// k_pages and v_pages both NULL: nothing goes to the cache; k is normed and rotated in place like q (for a
+// caller that changes q and k once more before a second call moves k and v into their pages).
 int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
                              const float* inv_freq, int rot_dim, const int32_t* tok_pos, const int32_t* tok_seq,
                              const int32_t* cu_seqlens, int seqs, int max_new,
@@ -128,6 +131,20 @@ int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, c
                                       int k, int swiglu, const float* ssq_in, int n_in, float eps, int dim,
                                       float* residual, const float* next_gain, void* xg_out, float* ssq_out,
                                       int tiled, void* stream);
+
+// out[m, :] = bfloat16(xg[m, :] * inv[m]), inv[m] = 1 / sqrt(sum_j ssq[m, j] / dim + eps): finishes a norm whose
+// scaling was left to a product (xg = bfloat16(r * gain) and n_in partial sums of r^2 per row), for a reader
+// that cannot do it.  x_tiled: xg lies in the matrix cores' order (at most 64 rows); out is always in rows.
+int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float eps, int dim, int rows, int x_tiled,
+                   void* stream);
+
+// Reads `bytes` bytes from `data` (16-byte aligned) with `workgroups` workgroups and throws them away: what is
+// read lands in the memory-side cache for the kernel that wants it next.  sink: one device word that is
+// practically never written (it keeps the loads alive), may be NULL.
+int ri_prefetch(const void* data, long bytes, int workgroups, void* sink, void* stream);
+
+// x[t, i] += bias[i] in place (bias float32 [dim], x of dtype [rows, dim]).
+int ri_add_bias(void* x, int dtype, const float* bias, int rows, int dim, void* stream);
 
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
 int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);

@@ -9,11 +9,12 @@
 #include "common.h"
 
 #define QK_MAX_PAIRS 4   // pairs per lane: head_dim / 2 <= 64 * QK_MAX_PAIRS
+#define QK_MAX_TAIL 8    // elements per lane behind the rotated part: head_dim <= 64 * QK_MAX_TAIL
 
 template <typename TA, typename TC>
 __global__ void qk_norm_rope_kv_write_kernel(
     TA* __restrict__ qkv, const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
-    const float* __restrict__ inv_freq, const int32_t* __restrict__ tok_pos,
+    const float* __restrict__ inv_freq, int rot_dim, const int32_t* __restrict__ tok_pos,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ page_table, int table_width,
     TC* __restrict__ k_pages, TC* __restrict__ v_pages, int tokens, int heads, int kv_heads, int head_dim,
     int page_size) {
@@ -23,12 +24,16 @@ __global__ void qk_norm_rope_kv_write_kernel(
     const long item = (long)blockIdx.x * waves_per_block + threadIdx.x / RI_WAVE;
     if (item >= (long)tokens * all_heads) return;          // whole wavefront leaves together
     const int t = (int)(item / all_heads), hh = (int)(item % all_heads);
-    const int half = head_dim / 2;
+    // the first rot_dim elements of a head are rotated in pairs (i, i + rot_dim / 2); the rest, if any, is
+    // normed only (a rotation over part of the head).  Without a rotation the pairing only shares out the work.
+    const int half = rot_dim / 2;
     TA* x = qkv + (size_t)t * all_heads * head_dim + (size_t)hh * head_dim;
 
     const int pos = tok_pos[t];
     TC* dst = nullptr;          // where a k head goes
-    if (hh >= heads) {
+    if (hh >= heads && k_pages == nullptr) {
+        if (hh >= heads + kv_heads) return;            // no pages given: k is changed in place like q, v is left alone
+    } else if (hh >= heads) {
         const int kvh = (hh - heads) % kv_heads;
         const int page = page_table[(size_t)tok_seq[t] * table_width + pos / page_size];
         const size_t head_base = ((size_t)page * kv_heads + kvh) * page_size * head_dim;
@@ -41,8 +46,9 @@ __global__ void qk_norm_rope_kv_write_kernel(
         dst = k_pages + head_base + (size_t)(pos % page_size) * head_dim;
     }
 
-    // lane owns pairs i = lane, lane + 64, ...: elements (i, i + half)
-    float x1[QK_MAX_PAIRS], x2[QK_MAX_PAIRS];
+    // lane owns pairs i = lane, lane + 64, ...: elements (i, i + half), and of the elements behind the
+    // rotated part every 64th
+    float x1[QK_MAX_PAIRS], x2[QK_MAX_PAIRS], xt[QK_MAX_TAIL];
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < QK_MAX_PAIRS; ++j) {
@@ -52,6 +58,15 @@ __global__ void qk_norm_rope_kv_write_kernel(
             x1[j] = to_f32(x[i]);
             x2[j] = to_f32(x[i + half]);
             ss += x1[j] * x1[j] + x2[j] * x2[j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < QK_MAX_TAIL; ++j) {
+        const int i = 2 * half + lane + j * RI_WAVE;
+        xt[j] = 0.f;
+        if (i < head_dim) {
+            xt[j] = to_f32(x[i]);
+            ss += xt[j] * xt[j];
         }
     }
     const float* gain = hh < heads ? q_gain : k_gain;
@@ -73,6 +88,14 @@ __global__ void qk_norm_rope_kv_write_kernel(
         }
         if (dst) { from_f32(dst + i, a); from_f32(dst + i + half, b); }
         else     { from_f32(x + i, a);   from_f32(x + i + half, b); }
+    }
+#pragma unroll
+    for (int j = 0; j < QK_MAX_TAIL; ++j) {
+        const int i = 2 * half + lane + j * RI_WAVE;
+        if (i >= head_dim) continue;
+        const float a = gain ? xt[j] * inv * gain[i] : xt[j];
+        if (dst) from_f32(dst + i, a);
+        else     from_f32(x + i, a);
     }
 }
 
@@ -205,7 +228,9 @@ static bool vec_path_fits(int head_dim, int page_size) {
     const int half = head_dim / 2;
     if (half % 8) return false;
     const int lph = half / 8;
-    return lph <= 64 && (lph & (lph - 1)) == 0 && page_size % VW_TOKENS == 0;
+    // (the page-wise value writer holds 32 tokens of a head in LDS: 64 KB at most without asking for more)
+    return lph <= 64 && (lph & (lph - 1)) == 0 && page_size % VW_TOKENS == 0 &&
+           (size_t)VW_TOKENS * (head_dim + 1) * sizeof(float) <= 65536;
 }
 
 template <typename TA, typename TC>
@@ -216,7 +241,8 @@ static void launch_qk(void* qkv, const float* q_gain, const float* k_gain, float
                       hipStream_t s) {
     // one new token per sequence: a single launch that writes the few values element by element is cheaper
     // than two
-    if (cu_seqlens && max_new > 1 && vec_path_fits(head_dim, page_size)) {
+    const bool whole = head_dim % 2 == 0 && (!inv_freq || rot_dim == head_dim);      // what the 16-byte kernels rotate
+    if (cu_seqlens && max_new > 1 && whole && k_pages && vec_path_fits(head_dim, page_size)) {
         qk_norm_rope_k_write_vec_kernel<TA, TC><<<tokens, 256, head_dim * sizeof(float), s>>>(
             (TA*)qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, table_width, (TC*)k_pages, heads,
             kv_heads, head_dim, page_size);
@@ -230,8 +256,8 @@ static void launch_qk(void* qkv, const float* q_gain, const float* k_gain, float
     const long items = (long)tokens * (heads + 2 * kv_heads);
     const int waves = 4;
     qk_norm_rope_kv_write_kernel<TA, TC><<<(unsigned)((items + waves - 1) / waves), waves * RI_WAVE, 0, s>>>(
-        (TA*)qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, table_width,
-        (TC*)k_pages, (TC*)v_pages, tokens, heads, kv_heads, head_dim, page_size);
+        (TA*)qkv, q_gain, k_gain, eps, inv_freq, inv_freq ? rot_dim : (head_dim & ~1), tok_pos, tok_seq, page_table,
+        table_width, (TC*)k_pages, (TC*)v_pages, tokens, heads, kv_heads, head_dim, page_size);
 }
 
 extern "C" int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q_gain, const float* k_gain, float eps,
@@ -242,12 +268,14 @@ extern "C" int ri_qk_norm_rope_kv_write(void* qkv, int act_dtype, const float* q
                                         int kv_heads, int head_dim, int page_size, int num_pages, void* stream) {
     RI_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0, "qk_norm_rope_kv_write: tokens %d, heads %d, kv heads %d",
                tokens, heads, kv_heads);
-    RI_REQUIRE(head_dim >= 2 && head_dim % 2 == 0 && head_dim <= 2 * RI_WAVE * QK_MAX_PAIRS,
-               "qk_norm_rope_kv_write: head_dim %d must be even and at most %d", head_dim, 2 * RI_WAVE * QK_MAX_PAIRS);
-    RI_REQUIRE(!inv_freq || rot_dim == head_dim,
-               "qk_norm_rope_kv_write: rotation of %d of %d elements: only whole heads are rotated here", rot_dim,
-               head_dim);
-    RI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "qk_norm_rope_kv_write: page geometry");
+    RI_REQUIRE(head_dim >= 1 && head_dim <= 2 * RI_WAVE * QK_MAX_PAIRS,
+               "qk_norm_rope_kv_write: head_dim %d must be between 1 and %d", head_dim, 2 * RI_WAVE * QK_MAX_PAIRS);
+    RI_REQUIRE(!inv_freq || (rot_dim >= 2 && rot_dim % 2 == 0 && rot_dim <= head_dim),
+               "qk_norm_rope_kv_write: a rotation of %d of %d elements: the rotated part is even and no longer than "
+               "the head", rot_dim, head_dim);
+    RI_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "qk_norm_rope_kv_write: key pages without value pages");
+    RI_REQUIRE(k_pages == nullptr || (page_size > 0 && table_width > 0 && num_pages > 0),
+               "qk_norm_rope_kv_write: page geometry");
     RI_REQUIRE((long)tokens * (heads + 2 * kv_heads) / 4 < 2147483647L, "qk_norm_rope_kv_write: too many tokens");
     RI_REQUIRE(!cu_seqlens || (seqs > 0 && seqs <= 65535 && max_new > 0 && kv_heads <= 65535),
                "qk_norm_rope_kv_write: seqs %d, max_new %d", seqs, max_new);

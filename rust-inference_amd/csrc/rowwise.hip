@@ -172,8 +172,9 @@ extern "C" int ri_add_rmsnorm(void* out, int out_dtype, float* residual, const v
     return 0;
 }
 
+// (out may be residual itself when rows is NULL: every element is read and then written by one thread)
 template <typename TP>
-__global__ void add_rows_kernel(float* __restrict__ out, const float* __restrict__ residual,
+__global__ void add_rows_kernel(float* out, const float* residual,
                                 const TP* __restrict__ pending, const int32_t* __restrict__ rows, int dim) {
     const int row = blockIdx.x;
     const size_t src = (size_t)(rows ? rows[row] : row) * dim;
@@ -195,6 +196,33 @@ extern "C" int ri_add_rows(float* out, const float* residual, const void* pendin
     else
         RI_REQUIRE(false, "add_rows: pending dtype %d", pending_dtype);
     RI_LAUNCH_CHECK("add_rows");
+    return 0;
+}
+
+// ------------------------------------------------------------------ a norm that a product was to finish
+// out[m, :] = bfloat16(xg[m, :] * inv[m]) with inv[m] = 1 / sqrt(sum_j ssq[m, j] / dim + eps): the rows of a
+// norm that was left to the product after it (see NormLink in common.h), for a reader that cannot take the
+// norm over.  The partial sums are added in a fixed order.  xg lies in rows or in the matrix cores' order.
+__global__ void finish_norm_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ xg, const float* __restrict__ ssq,
+                                   int n_in, float eps, int dim, int x_tiled) {
+    __shared__ float scratch[16];
+    const int m = blockIdx.x;
+    float part = 0.f;
+    for (int j = threadIdx.x; j < n_in; j += blockDim.x) part += ssq[(size_t)m * n_in + j];
+    const float inv = 1.0f / sqrtf(block_sum(part, scratch) / (float)dim + eps);
+    const int k_tiles = (dim + 31) / 32;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        const bf16_t v = x_tiled ? xg[tiled_at(m, d, k_tiles)] : xg[(size_t)m * dim + d];
+        out[(size_t)m * dim + d] = f32_to_bf16(bf16_to_f32(v) * inv);
+    }
+}
+
+extern "C" int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float eps, int dim, int rows,
+                              int x_tiled, void* stream) {
+    RI_REQUIRE(rows > 0 && dim > 0 && n_in > 0, "finish_norm: rows %d, dim %d, %d partial sums", rows, dim, n_in);
+    RI_REQUIRE(!x_tiled || rows <= 64, "finish_norm: %d rows in the matrix cores' order (64 at most)", rows);
+    finish_norm_kernel<<<rows, 256, 0, (hipStream_t)stream>>>((bf16_t*)out, (const bf16_t*)xg, ssq, n_in, eps, dim, x_tiled);
+    RI_LAUNCH_CHECK("finish_norm");
     return 0;
 }
 
@@ -247,6 +275,25 @@ extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int in
     else
         RI_REQUIRE(false, "swiglu: dtype %d", dtype);
     RI_LAUNCH_CHECK("swiglu");
+    return 0;
+}
+
+// ------------------------------------------------------------------ bias
+// x[t, i] += bias[i] in place, the sum in float32 (for parts with biased products; the reference's family
+// has none: src/models/qwen3.rs:60-69).
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int dim) {
+    T* row = x + (size_t)blockIdx.x * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) from_f32(row + d, to_f32(row[d]) + bias[d]);
+}
+
+extern "C" int ri_add_bias(void* x, int dtype, const float* bias, int rows, int dim, void* stream) {
+    RI_REQUIRE(rows > 0 && dim > 0, "add_bias: rows %d, dim %d", rows, dim);
+    RI_REQUIRE(dtype == RI_F32 || dtype == RI_BF16, "add_bias: dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == RI_F32) add_bias_kernel<float><<<rows, 256, 0, s>>>((float*)x, bias, dim);
+    else add_bias_kernel<bf16_t><<<rows, 256, 0, s>>>((bf16_t*)x, bias, dim);
+    RI_LAUNCH_CHECK("add_bias");
     return 0;
 }
 

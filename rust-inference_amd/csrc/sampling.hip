@@ -38,7 +38,7 @@ __device__ __forceinline__ uint32_t ordered_bits(float f) {
 struct RowView {
     const float* logits;
     const uint8_t* seen;     // may be NULL
-    float penalty, inv_temperature;
+    float penalty, temperature;      // temperature: the divisor of every logit (1 when the row is taken greedily)
     bool wide;               // the row starts on a 16-byte boundary and the vocabulary is a multiple of 4
     __device__ __forceinline__ float penalise(float l, bool was_seen) const {
         return was_seen ? (l > 0.f ? l / penalty : l * penalty) : l;
@@ -158,7 +158,7 @@ __device__ u64 descend_from(const RowView& row, int vocab, float smax, u64 floor
             __syncthreads();
             const uint32_t value_bits = (uint32_t)(prefix >> SMP_ID_BITS);
             for_each_logit(row, 0, vocab, SMP_THREADS, [&](int i, float l) {
-                const float s = l * row.inv_temperature;
+                const float s = l / row.temperature;
                 if (ordered_bits(s) == value_bits && composite(s, i) >= floor_key) {
                     const int k = atomicAdd(tie_count, 1);
                     if (k < SMP_TIES) ties[k] = i;
@@ -191,7 +191,7 @@ __device__ u64 descend_from(const RowView& row, int vocab, float smax, u64 floor
         __syncthreads();
         const u64 hi_mask = shift == 48 ? 0 : (~(u64)0) << (shift + 8);
         for_each_logit(row, 0, vocab, SMP_THREADS, [&](int i, float l) {
-            const float s = l * row.inv_temperature;
+            const float s = l / row.temperature;
             const u64 c = composite(s, i);
             if (c >= floor_key && (c & hi_mask) == (prefix & hi_mask)) {
                 const u64 w = MASS ? fixed_mass(s, smax) : 1;
@@ -228,7 +228,7 @@ __device__ __forceinline__ RowView row_view(const float* logits, const uint8_t* 
     row.logits = logits + (size_t)r * vocab;
     row.seen = (seen && penalty != 1.0f) ? seen + (size_t)(seen_rows ? seen_rows[r] : r) * vocab : nullptr;
     row.penalty = penalty;
-    row.inv_temperature = temperature > 0.f ? 1.0f / temperature : 1.0f;
+    row.temperature = temperature > 0.f ? temperature : 1.0f;      // logit / temperature, a true division (src/sampling.rs:93-94)
     row.wide = vocab % 4 == 0 && ((uintptr_t)row.logits & 15) == 0 && ((uintptr_t)row.seen & 3) == 0;
     return row;
 }
@@ -268,7 +268,7 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
     }
 
     float smax = -INFINITY;
-    for_each_logit(row, 0, vocab, SMP_THREADS, [&](int, float l) { smax = fmaxf(smax, l * row.inv_temperature); });
+    for_each_logit(row, 0, vocab, SMP_THREADS, [&](int, float l) { smax = fmaxf(smax, l / row.temperature); });
     smax = block_max(smax, fscratch);
 
     u64 floor_key = 0, incl = 0;
@@ -278,7 +278,7 @@ sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits, const
     // would cost seven more passes; one exact integer sum does it
     u64 z = 0;
     for_each_logit(row, 0, vocab, SMP_THREADS, [&](int i, float l) {
-        const float s = l * row.inv_temperature;
+        const float s = l / row.temperature;
         if (composite(s, i) >= floor_key) z += fixed_mass(s, smax);
     });
     for (int m = RI_WAVE / 2; m > 0; m >>= 1) z += __shfl_xor(z, m, RI_WAVE);
@@ -423,7 +423,7 @@ split_max_kernel(SplitPlan p) {
     const int r = blockIdx.y, begin = blockIdx.x * p.slice, end = min(p.vocab, begin + p.slice);
     const RowView row = row_view(p.logits, p.seen, p.seen_rows, r, p.vocab, p.temperature, p.penalty);
     float smax = -INFINITY;
-    for_each_logit(row, begin, end, SW_THREADS, [&](int, float l) { smax = fmaxf(smax, l * row.inv_temperature); });
+    for_each_logit(row, begin, end, SW_THREADS, [&](int, float l) { smax = fmaxf(smax, l / row.temperature); });
     smax = block_max(smax, fscratch);
     if (threadIdx.x == 0 && begin < end)
         atomicMax(reinterpret_cast<unsigned int*>(p.ws + (size_t)r * SW_WORDS + SW_SMAX), ordered_bits(smax));
@@ -451,7 +451,7 @@ split_pass_kernel(SplitPlan p, int desc, int digit) {
         unsigned int* count = reinterpret_cast<unsigned int*>(ws_row + SW_TIE_COUNT + desc);
         int* ties = reinterpret_cast<int*>(ws_row + SW_TIES) + (size_t)desc * SMP_TIES;
         for_each_logit(row, begin, end, SW_THREADS, [&](int i, float l) {
-            const float s = l * row.inv_temperature;
+            const float s = l / row.temperature;
             if (ordered_bits(s) == value_bits && composite(s, i) >= d.floor_key) {
                 const unsigned int k = atomicAdd(count, 1u);
                 if (k < SMP_TIES) ties[k] = i;
@@ -464,7 +464,7 @@ split_pass_kernel(SplitPlan p, int desc, int digit) {
     __syncthreads();
     const u64 hi_mask = shift == 48 ? 0 : (~(u64)0) << (shift + 8);
     for_each_logit(row, begin, end, SW_THREADS, [&](int i, float l) {
-        const float s = l * row.inv_temperature;
+        const float s = l / row.temperature;
         const u64 c = composite(s, i);
         if (c >= d.floor_key && (c & hi_mask) == (d.prefix & hi_mask)) {
             const u64 w = MASS ? fixed_mass(s, smax) : 1;

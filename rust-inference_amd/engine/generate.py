@@ -17,6 +17,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Sequence
 
+from .. import profiler
 from ..errors import CacheError, ShapeError
 from ..sampling import DeviceHistory, SamplingParams, SequenceSampler, sample_batch
 from .step import StepEntry
@@ -109,7 +110,8 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
         history = None
         if sampling.repetition_penalty != 1.0 and logits.is_cuda:
             history = DeviceHistory([s.sampler for s in live], logits.shape[1], logits.device)
-        picks = sample_batch(logits, [s.sampler for s in live], history)
+        with profiler.section(profiler.SAMPLING):
+            picks = sample_batch(logits, [s.sampler for s in live], history)
         stats.prompt_tokens += sum(len(s.prompt) for s in live)
         stats.prefill_seconds += time.perf_counter() - t0      # includes the first sample, as in the reference
         for s, tok in zip(live, picks):
@@ -140,7 +142,8 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
                 s.sampler.history.append(s.next_token)
             if history is not None:
                 history.mark([s.sampler.seen_row for s in live], [s.next_token for s in live])
-            picks = sample_batch(logits, [s.sampler for s in live], history)
+            with profiler.section(profiler.SAMPLING):
+                picks = sample_batch(logits, [s.sampler for s in live], history)
             for s, tok in zip(live, picks):
                 s.next_token = int(tok)
                 s.generated += 1

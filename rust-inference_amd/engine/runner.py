@@ -118,7 +118,11 @@ def main(argv=None) -> int:
         print("error: --chat wraps text and needs a tokenizer.json", file=sys.stderr)
         return 1
     raw = list(args.prompt or [])
-    id_prompts = [parse_ids(p) for p in (args.prompt_ids or [])]
+    try:
+        id_prompts = [parse_ids(p) for p in (args.prompt_ids or [])]
+    except ValueError:
+        print("error: --prompt-ids takes token ids separated by commas or spaces", file=sys.stderr)
+        return 1
     if not raw and not id_prompts:
         lines = [ln.rstrip("\n") for ln in sys.stdin]
         raw = [ln for ln in lines if ln.strip()] if args.batch else ["\n".join(lines).strip()]
@@ -126,13 +130,23 @@ def main(argv=None) -> int:
     for p in raw:
         if args.chat:
             p = chat_prompt(p, args.think)                             # src/bin/runner.rs:233
-        prompts.append(tokenizer.encode(p).ids if tokenizer is not None else parse_ids(p))
+        if tokenizer is not None:
+            prompts.append(tokenizer.encode(p).ids)
+            continue
+        try:
+            prompts.append(parse_ids(p))
+        except ValueError:
+            print(f"error: the prompt is text, and {args.tokenizer or args.model_dir} has no tokenizer.json to encode "
+                  "it with: give token ids (-p \"5 17 3\" or --prompt-ids 5,17,3)", file=sys.stderr)
+            return 1
     if not prompts or any(len(p) == 0 for p in prompts):
         print("error: empty prompt", file=sys.stderr)                  # src/bin/runner.rs:235-237
         return 1
 
+    from .. import profiler
     from ..api import Model
     from ..errors import InferenceError
+    profiler.enable(args.profile)                                      # src/bin/runner.rs:207
     t0 = time.perf_counter()
     try:
         per_seq = args.pages_per_seq * 32
@@ -178,4 +192,5 @@ def main(argv=None) -> int:
         per_step = 1e3 * st.decode_seconds / st.decode_steps if st.decode_steps else 0.0
         print(f"profile: {st.batches} batches, {st.decode_steps} decode steps, {per_step:.3f} ms per step",
               file=sys.stderr)
+        print("\n" + profiler.report(), file=sys.stderr)                # src/bin/runner.rs:252-254
     return 0

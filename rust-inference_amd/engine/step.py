@@ -18,6 +18,7 @@ import itertools
 import numpy as np
 import torch
 
+from .. import profiler
 from ..cache import native as cache_native
 from ..errors import ShapeError
 from ..parts.context import StepContext
@@ -53,34 +54,6 @@ def _one_token_wanted(e: StepEntry) -> bool:
     if len(e.tokens) != 1:
         return False
     return e.want == "last" or e.want == "all" or (not isinstance(e.want, str) and wanted_indices(1, e.want) == [0])
-
-
-def plan_step(entries: Sequence[StepEntry], lengths: Sequence[int], vocab_size: int):
-    """The host-side layout of a step: flat tokens, each token's sequence and position, where
-    each sequence starts among them, and the wanted rows, as int32 arrays.  ``lengths[i]`` is
-    entry i's cache length before the step."""
-    if not entries:
-        raise ShapeError("a step needs at least one entry")
-    counts = [len(e.tokens) for e in entries]
-    for b, (e, n) in enumerate(zip(entries, counts)):
-        if n < 1:
-            raise ShapeError(f"entry {b} (slot {e.slot}) brings no token")
-    total = sum(counts)
-    tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int64, count=total)
-    if tokens.min() < 0 or tokens.max() >= vocab_size:
-        bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
-        raise ShapeError(f"token id {bad} is outside the vocabulary of {vocab_size}")       # src/ops/embedding.rs:20-22
-    cu = np.zeros(len(entries) + 1, dtype=np.int32)
-    np.cumsum(counts, out=cu[1:])
-    if total == len(entries):                                  # one token each: the common step
-        tok_seq = np.arange(total, dtype=np.int32)
-        tok_pos = np.asarray(lengths, dtype=np.int32)
-    else:
-        tok_seq = np.repeat(np.arange(len(entries), dtype=np.int32), counts)
-        tok_pos = (np.arange(total, dtype=np.int32) - np.repeat(cu[:-1] - np.asarray(lengths, dtype=np.int32), counts))
-    want_rows = np.asarray([int(cu[b]) + i for b, (e, n) in enumerate(zip(entries, counts))
-                            for i in wanted_indices(n, e.want)], dtype=np.int32)
-    return tokens.astype(np.int32), tok_seq, tok_pos.astype(np.int32), cu, want_rows
 
 
 class _Staging:
@@ -223,7 +196,8 @@ class Engine:
         the entries and of each entry's wanted places.  (With graphs the logits of a decode step
         live in the graph's own buffer and are overwritten by the next decode step of that size.)"""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
-        if self.use_graphs and entries and all(_one_token_wanted(e) for e in entries):
+        # (section timers read events around the kernels, which a captured graph does not hold)
+        if self.use_graphs and not profiler.enabled() and entries and all(_one_token_wanted(e) for e in entries):
             return self._graph_step(entries)
         ctx = self.build_context(entries)
         logits = self.model.forward(ctx, self.cache)
@@ -259,12 +233,21 @@ class Engine:
         # the same keys and values to the same places twice changes nothing, and per-sequence
         # state is put back to where it was before the rehearsal
         saved = self.cache.snapshot_state()
-        self.model.forward(ctx, self.cache)
+        stream = getattr(self.model.rt, "weight_stream", None)
+        if stream is not None:
+            with stream.recording():                          # the rehearsal also tells the order of the weights
+                self.model.forward(ctx, self.cache)
+        else:
+            self.model.forward(ctx, self.cache)
         self.cache.restore_state(saved)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            dg.logits = self.model.forward(ctx, self.cache)
+            if stream is not None:
+                with stream.playing(stream.order):
+                    dg.logits = self.model.forward(ctx, self.cache)
+            else:
+                dg.logits = self.model.forward(ctx, self.cache)
         dg.graph, dg.ctx = graph, ctx
         dg.graph.replay()
         self.cache.commit(ctx.slot_list, ctx.new_counts)

@@ -54,6 +54,9 @@ _SIGNATURES = {
     "ri_gemm_skinny_packed_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                           c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_add_bias": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "ri_prefetch": [c_void_p, ctypes.c_long, c_int, c_void_p, c_void_p],
+    "ri_finish_norm": [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -146,15 +149,25 @@ def add_rmsnorm(residual: torch.Tensor, pending, gain: torch.Tensor, eps: float,
     return out
 
 
-def add_rows(residual: torch.Tensor, pending, rows: torch.Tensor | None = None) -> torch.Tensor:
-    """float32 ``residual[rows] + pending[rows]`` without a norm."""
+def add_rows(residual: torch.Tensor, pending, rows: torch.Tensor | None = None, in_place: bool = False) -> torch.Tensor:
+    """float32 ``residual[rows] + pending[rows]`` without a norm; with ``in_place`` (all rows) the sum is
+    written into ``residual`` itself."""
     t, dim = residual.shape
     n = t if rows is None else rows.shape[0]
-    out = torch.empty((n, dim), dtype=torch.float32, device=residual.device)
+    if in_place and rows is not None:
+        raise ShapeError("an add in place takes all rows")
+    out = residual if in_place else torch.empty((n, dim), dtype=torch.float32, device=residual.device)
     _call("ri_add_rows", _dev(out, "out"), _dev(residual, "residual", torch.float32),
           _opt(pending, "pending", None, (t, dim)), code(pending.dtype) if pending is not None else F32,
           _opt(rows, "rows", torch.int32), n, dim, _stream())
     return out
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``x[t, :] += bias`` in place (float32 bias, the sum in float32); returns ``x``."""
+    rows, dim = x.shape
+    _call("ri_add_bias", _dev(x, "x"), code(x.dtype), _dev(bias, "bias", torch.float32, (dim,)), rows, dim, _stream())
+    return x
 
 
 def swiglu(y: torch.Tensor) -> torch.Tensor:
@@ -221,22 +234,31 @@ def mark_seen(seen: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor) -> N
 def qk_norm_rope_kv_write(qkv, q_gain, k_gain, eps, inv_freq, tok_pos, tok_seq, page_table, k_pages, v_pages,
                           heads: int, kv_heads: int, head_dim: int, cu_seqlens=None, max_new: int = 0) -> None:
     """In place on ``qkv: [T, (H + 2 Hkv) dh]``: per-head norm and rotation of q and k; k and v go to their
-    pages.  With ``cu_seqlens`` (int32 ``[seqs + 1]``) and ``max_new`` values are written a page at a time."""
+    pages.  ``inv_freq`` (float32 ``[r]``, ``r <= dh / 2``) rotates the first ``2 r`` elements of every head in
+    pairs ``(i, i + r)``; what lies behind them is normed only.  With ``cu_seqlens`` (int32 ``[seqs + 1]``) and
+    ``max_new`` values are written a page at a time."""
     tokens = qkv.shape[0]
     width = (heads + 2 * kv_heads) * head_dim
-    num_pages, hkv, page_size, dh = k_pages.shape
-    if (hkv, dh) != (kv_heads, head_dim) or tuple(v_pages.shape) != (num_pages, hkv, dh, page_size):
-        raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv heads "
-                         f"of {head_dim}")
-    half = head_dim // 2
+    if k_pages is None:                       # nothing goes to the cache: k is changed in place like q
+        if v_pages is not None:
+            raise ShapeError("key pages and value pages come together or not at all")
+        num_pages, page_size = 0, 0
+    else:
+        num_pages, hkv, page_size, dh = k_pages.shape
+        if (hkv, dh) != (kv_heads, head_dim) or tuple(v_pages.shape) != (num_pages, hkv, dh, page_size):
+            raise ShapeError(f"pages are {list(k_pages.shape)} / {list(v_pages.shape)}, the mixer has {kv_heads} kv "
+                             f"heads of {head_dim}")
+    rot_dim = head_dim if inv_freq is None else 2 * inv_freq.shape[0]
+    if inv_freq is not None and (inv_freq.dim() != 1 or not 2 <= rot_dim <= head_dim):
+        raise ShapeError(f"inv_freq is {list(inv_freq.shape)}: a head of {head_dim} takes 1 to {head_dim // 2} frequencies")
     _call("ri_qk_norm_rope_kv_write", _dev(qkv, "qkv", None, (tokens, width)), code(qkv.dtype),
           _opt(q_gain, "q_gain", torch.float32, (head_dim,)), _opt(k_gain, "k_gain", torch.float32, (head_dim,)),
-          float(eps), _opt(inv_freq, "inv_freq", torch.float32, (half,)), head_dim,
+          float(eps), _opt(inv_freq, "inv_freq", torch.float32), rot_dim,
           _dev(tok_pos, "tok_pos", torch.int32, (tokens,)), _dev(tok_seq, "tok_seq", torch.int32, (tokens,)),
           _opt(cu_seqlens, "cu_seqlens", torch.int32), 0 if cu_seqlens is None else cu_seqlens.shape[0] - 1,
           int(max_new), _dev(page_table, "page_table", torch.int32), page_table.shape[1],
-          _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), code(k_pages.dtype), tokens, heads, kv_heads, head_dim,
-          page_size, num_pages, _stream())
+          _opt(k_pages, "k_pages"), _opt(v_pages, "v_pages"), code(qkv.dtype if k_pages is None else k_pages.dtype),
+          tokens, heads, kv_heads, head_dim, page_size, num_pages, _stream())
 
 
 def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, kv_heads: int, head_dim: int,
@@ -253,6 +275,7 @@ def attention(qkv, k_pages, v_pages, tok_pos, tok_seq, page_table, heads: int, k
 
 
 MFMA_HEAD_DIMS = (32, 64, 128)
+MAX_HEAD_DIM = 512          # what the general attention and q/k kernels take (any size from 1 up to it)
 
 
 def mfma_attention_fits(dtype, head_dim: int, group: int, page_size: int, decode: bool) -> bool:
@@ -337,6 +360,18 @@ def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_p
 
 
 # ---------------------------------------------------------------- products
+# Called with the weight tensor a product is about to stream (the copy it really reads), before its kernel
+# is launched: ``parts.runtime.WeightStream`` learns the order of a step's weights from it.
+weight_hook = None
+
+
+def prefetch(w: torch.Tensor, workgroups: int, sink: torch.Tensor | None = None, stream: int | None = None) -> None:
+    """Reads the whole of ``w`` and throws it away (see csrc/prefetch.hip), on ``stream`` (a raw handle) or
+    the current one."""
+    _call("ri_prefetch", _dev(w, "w"), w.numel() * w.element_size(), int(workgroups),
+          _opt(sink, "sink", torch.int32), _stream() if stream is None else stream)
+
+
 def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``x @ w.T`` in true 32-bit arithmetic; ``x`` float32 ``[M, K]``, ``w`` float32 or bfloat16 ``[N, K]``."""
     m, k = x.shape
@@ -353,6 +388,8 @@ def gemv_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu
     m, k = x.shape
     n = w.shape[0] // 2 if swiglu else w.shape[0]
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if weight_hook is not None:
+        weight_hook(w)
     _call("ri_gemv_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
           _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
     return out
@@ -434,6 +471,8 @@ def gemm_skinny_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bf
         raise ShapeError("a tiled result is bfloat16 and whole")
     flags = (TILED_X if isinstance(x, TiledRows) else 0) | (TILED_OUT if tiled_out else 0)
     xd = _dev(x.data, "x", torch.bfloat16) if isinstance(x, TiledRows) else _dev(x, "x", torch.bfloat16)
+    if weight_hook is not None:
+        weight_hook(wpacked)
     if tiled_out:
         out = TiledRows.empty(m, n, x.device)
         od = _dev(out.data, "out")
@@ -455,6 +494,19 @@ class NormedLater:
         self.shape, self.dtype, self.device = xg.shape, xg.dtype, xg.device
 
 
+def finish_norm(later: NormedLater) -> torch.Tensor:
+    """The normed bfloat16 rows ``[M, dim]`` of a ``NormedLater``, for a reader that cannot take the norm
+    over (``xg`` was rounded once already, so this differs from the plain norm by one more rounding)."""
+    xg = later.xg
+    tiled = isinstance(xg, TiledRows)
+    m, dim = xg.shape
+    out = torch.empty((m, dim), dtype=torch.bfloat16, device=later.device)
+    _call("ri_finish_norm", _dev(out, "out"), _dev(xg.data if tiled else xg, "xg", torch.bfloat16),
+          _dev(later.ssq, "ssq", torch.float32, (m, later.ssq.shape[1])), later.ssq.shape[1], later.eps, later.dim, m,
+          int(tiled), _stream())
+    return out
+
+
 def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16, swiglu: bool = False,
                          tiled_out: bool = False):
     """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by
@@ -469,6 +521,8 @@ def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloa
         raise ShapeError("a tiled result is bfloat16")
     x_tiled = isinstance(x, TiledRows)
     out = TiledRows.empty(m, n, x.device) if tiled_out else torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if weight_hook is not None:
+        weight_hook(wpacked)
     _call("ri_gemm_mid_packed_bf16", _dev(out.data if tiled_out else out, "out"), code(out_dtype),
           _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
           int(swiglu), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), _stream())
@@ -501,6 +555,8 @@ def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfl
         wd = _dev(w, "w", torch.bfloat16, (n * (2 if swiglu else 1), k))
     x_tiled = isinstance(xr, TiledRows)
     xd = _dev(xr.data, "x", torch.bfloat16) if x_tiled else _dev(xr, "x", torch.bfloat16, (m, k))
+    if weight_hook is not None:
+        weight_hook(w)
     # the packed kernel takes the layouts of x and of its result as one more argument
     layout = ((TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0),) if packed else ()
     if later is not None:

@@ -5,10 +5,11 @@ import math
 
 import torch
 
+from .. import profiler
 from ..cache import KVNeed
 from ..errors import ConfigError
 from ..kernels import ops
-from ..weights.loader import GAIN, MATRIX, TensorSpec
+from ..weights.loader import BIAS, GAIN, MATRIX, TensorSpec
 from .base import Mixer
 from .registry import build_part, register_part
 from .spec import PartSpec
@@ -35,20 +36,26 @@ class GroupedQueryAttention(Mixer):
     ``(q . k) / sqrt(head_dim)``; softmax statistics and the accumulator are float32.
     The three projections are one product with the row-concatenated weight
     ``[q; k; v]``: every output row's dot product is the same as with three products.
+
+    ``qkv_bias`` and ``o_bias`` add ``{q,k,v}_proj.bias`` and ``o_proj.bias`` to the products (the
+    reference's family has no bias anywhere, src/models/qwen3.rs:60-69; families that differ from it in
+    this alone need no other mixer).  A biased output product adds into the stream the plain way.
     """
 
     links_norms = True
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, prefix: str, qk_norm: bool = True,
-                 eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None):
+                 eps: float = 1e-6, position: PartSpec | None = None, window: int | None = None,
+                 qkv_bias: bool = False, o_bias: bool = False):
         if heads < 1 or kv_heads < 1 or heads % kv_heads:
             raise ConfigError(f"{heads} attention heads not divisible by {kv_heads} kv heads")
-        if head_dim % 16:
-            raise ConfigError(f"head_dim {head_dim}: the attention kernels take multiples of 16")
+        if not 1 <= head_dim <= ops.MAX_HEAD_DIM:
+            raise ConfigError(f"head_dim {head_dim}: the attention kernels take 1 to {ops.MAX_HEAD_DIM}")
         if window is not None and window < 1:
             raise ConfigError(f"window {window} must be positive")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.prefix, self.qk_norm, self.eps, self.window = prefix, qk_norm, eps, window
+        self.qkv_bias, self.o_bias = qkv_bias, o_bias
         self.scale = 1.0 / math.sqrt(head_dim)                      # src/attention.rs:28
         self.position = build_part("position", position or PartSpec("none"))
 
@@ -63,6 +70,12 @@ class GroupedQueryAttention(Mixer):
         if self.qk_norm:
             t[p + "q_norm.weight"] = TensorSpec((dh,), GAIN)
             t[p + "k_norm.weight"] = TensorSpec((dh,), GAIN)
+        if self.qkv_bias:
+            t[p + "q_proj.bias"] = TensorSpec((self.heads * dh,), BIAS)
+            t[p + "k_proj.bias"] = TensorSpec((self.kv_heads * dh,), BIAS)
+            t[p + "v_proj.bias"] = TensorSpec((self.kv_heads * dh,), BIAS)
+        if self.o_bias:
+            t[p + "o_proj.bias"] = TensorSpec((d,), BIAS)
         t.update(self.position.tensors())
         return t
 
@@ -74,6 +87,11 @@ class GroupedQueryAttention(Mixer):
         self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]))
         self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
         self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
+        self.b_qkv = self.b_o = None
+        if self.qkv_bias:
+            self.b_qkv = rt.place_gain(torch.cat([weights[p + n + "_proj.bias"] for n in "qkv"], 0))
+        if self.o_bias:
+            self.b_o = rt.place_gain(weights[p + "o_proj.bias"])
         self.position.bind(weights, rt)
 
     def takes_tiled_at(self, m: int) -> bool:
@@ -85,23 +103,48 @@ class GroupedQueryAttention(Mixer):
 
     def forward(self, x, ctx, store, page_table, link=None):
         rt = self.rt
-        qkv = rt.linear_packed(x, self.w_qkv)
+        with profiler.section(profiler.QKV_PROJECTION):
+            qkv = rt.linear_packed(x, self.w_qkv)
+            if self.b_qkv is not None:
+                ops.add_bias(qkv, self.b_qkv)
         self.position.apply(qkv, ctx, self.heads, self.kv_heads, self.head_dim)
         group = self.heads // self.kv_heads
-        if (ctx.is_decode and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, True)
+        table = self.position.rotation_table()
+        whole = table is None or 2 * table.shape[0] == self.head_dim      # the fused kernel rotates whole heads
+        after_norm = getattr(self.position, "acts_after_norm", False)
+        if (ctx.is_decode and whole and not after_norm
+                and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, True)
                 and (ctx.B <= FUSED_DECODE_MAX_SEQS
                      or ops.decode_attention_streams(ctx.B, self.kv_heads, ctx.max_len))):
             # one token per sequence: norm, rotation, cache write and attention are one kernel
-            o = ops.attention_decode_fused_bf16(qkv, self.q_gain, self.k_gain, self.eps,
-                                                self.position.rotation_table(), store.k_pages, store.v_pages,
-                                                ctx.tok_pos, page_table, ctx.B, ctx.max_len, self.heads,
-                                                self.kv_heads, self.head_dim, self.window, self.scale,
-                                                tiled_out=rt.takes_tiled(self.w_o, ctx.B))
-            return rt.linear_packed(o, self.w_o, link=link)
-        ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, self.position.rotation_table(),
-                                  ctx.tok_pos, ctx.tok_seq, page_table, store.k_pages, store.v_pages,
-                                  self.heads, self.kv_heads, self.head_dim, ctx.cu_seqlens, ctx.max_new)
-        return rt.linear_packed(self.attend(qkv, ctx, store, page_table), self.w_o, link=link)
+            with profiler.section(profiler.ATTENTION):
+                o = ops.attention_decode_fused_bf16(qkv, self.q_gain, self.k_gain, self.eps, table, store.k_pages,
+                                                    store.v_pages, ctx.tok_pos, page_table, ctx.B, ctx.max_len,
+                                                    self.heads, self.kv_heads, self.head_dim, self.window, self.scale,
+                                                    tiled_out=rt.takes_tiled(self.w_o, ctx.B))
+            return self.project_out(o, link)
+        with profiler.section(profiler.QK_NORM_ROPE_APPEND):
+            shape = (self.heads, self.kv_heads, self.head_dim)
+            if after_norm:
+                # an encoding that acts on the normed q and k: norm (and rotation) in place, the encoding,
+                # then the move of k and v into their pages
+                ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, table, ctx.tok_pos, ctx.tok_seq,
+                                          page_table, None, None, *shape)
+                self.position.apply_normed(qkv, ctx, *shape)
+                ops.qk_norm_rope_kv_write(qkv, None, None, self.eps, None, ctx.tok_pos, ctx.tok_seq, page_table,
+                                          store.k_pages, store.v_pages, *shape, ctx.cu_seqlens, ctx.max_new)
+            else:
+                ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, table, ctx.tok_pos, ctx.tok_seq,
+                                          page_table, store.k_pages, store.v_pages, *shape, ctx.cu_seqlens, ctx.max_new)
+        with profiler.section(profiler.ATTENTION):
+            o = self.attend(qkv, ctx, store, page_table)
+        return self.project_out(o, link)
+
+    def project_out(self, o, link):
+        with profiler.section(profiler.OUT_PROJECTION):
+            if self.b_o is None:
+                return self.rt.linear_packed(o, self.w_o, link=link)
+            return ops.add_bias(self.rt.linear_packed(o, self.w_o), self.b_o)
 
     def attend(self, qkv, ctx, store, page_table):
         """The attention kernel that fits the step: matrix cores for bfloat16 (one new token per

@@ -63,13 +63,22 @@ class FeedForward(Part):
 
 
 class PositionEncoding(Part):
-    """How positions enter a mixer.  ``rotation_table()`` returns the float32 inverse
-    frequencies ``[head_dim / 2]`` for the fused rotate-half kernel, or None when
-    this encoding does not rotate; ``apply(qkv, ctx, heads, kv_heads, head_dim)`` may
-    change q and k in place before the fused kernel for encodings of another kind."""
+    """How positions enter a mixer.  ``rotation_table()`` returns float32 inverse frequencies ``[r]``
+    (``r <= head_dim / 2``) for the fused kernel, which rotates the first ``2 r`` elements of every q and k
+    head in pairs ``(i, i + r)`` by ``pos * inv_freq[i]`` after the per-head norm, or None when this
+    encoding does not rotate.  An encoding of another kind changes q and k itself, in place, in the fused
+    projection ``qkv: [T, (heads + 2 kv_heads) * head_dim]``: in ``apply`` before the per-head norm, or,
+    when it sets ``acts_after_norm``, in ``apply_normed`` after the norm (and after the rotation, if it
+    also has a table) and before k and v go to the cache; the mixer then runs the norm, the encoding and
+    the cache write as three steps instead of one kernel."""
+
+    acts_after_norm = False
 
     def rotation_table(self):
         return None
 
     def apply(self, qkv, ctx, heads, kv_heads, head_dim):
+        return None
+
+    def apply_normed(self, qkv, ctx, heads, kv_heads, head_dim):
         return None

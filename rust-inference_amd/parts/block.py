@@ -3,6 +3,8 @@ from __future__ import annotations
 
 import torch
 
+from .. import profiler
+from ..kernels import ops
 from .registry import build_part, register_part
 
 # A decode step of at most this many tokens leaves its norms to the products around them (the
@@ -65,12 +67,13 @@ class ResidualStream:
                 return later
             # prepared for another reader: the sum is complete, norm it the plain way
         if self.pending is not None and self.pending.dim() == 3 and not getattr(norm, "accepts_parts", False):
-            self.pending = self.pending.sum(0)       # a norm that does not know about parts
-        if (tiled and rows is None and getattr(norm, "can_tile", False) and out_dtype == torch.bfloat16
-                and self.sum.shape[0] <= TILED_MAX_ROWS):
-            out = norm.apply(self.sum, self.pending, out_dtype, rows, tiled=True)
-        else:
-            out = norm.apply(self.sum, self.pending, out_dtype, rows)
+            self.flush()                             # a norm that does not know about parts: they go into the sum first
+        with profiler.section(profiler.NORM):
+            if (tiled and rows is None and getattr(norm, "can_tile", False) and out_dtype == torch.bfloat16
+                    and self.sum.shape[0] <= TILED_MAX_ROWS):
+                out = norm.apply(self.sum, self.pending, out_dtype, rows, tiled=True)
+            else:
+                out = norm.apply(self.sum, self.pending, out_dtype, rows)
         if rows is None:
             self.pending = None      # the kernel wrote sum + pending back
         return out
@@ -79,8 +82,8 @@ class ResidualStream:
         """Add the waiting branch without a norm (only arrangements that push twice need it)."""
         self.later = None            # its sum is in the stream already
         if self.pending is not None:
-            pending = self.pending.sum(0) if self.pending.dim() == 3 else self.pending
-            self.sum.add_(pending.to(self.sum.dtype))
+            for part in (self.pending.unbind(0) if self.pending.dim() == 3 else (self.pending,)):
+                ops.add_rows(self.sum, part, in_place=True)       # parts in order, each sum in float32
             self.pending = None
 
 

@@ -3,6 +3,7 @@ from __future__ import annotations
 
 import torch
 
+from .. import profiler
 from ..weights.loader import MATRIX, TensorSpec
 from .base import FeedForward
 from .registry import register_part
@@ -42,6 +43,7 @@ class SwiGLU(FeedForward):
         rt = self.rt
         # the activation is in the epilogue of the decode-size kernels, which hand the down product its rows
         # in the order it loads fastest when that product is a packed one too
-        a = rt.linear_packed(x, self.w_gate_up, tiled_out=rt.takes_tiled(self.w_down, x.shape[0]))
-        # may come in parts: the stream's next norm adds them
-        return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)
+        with profiler.section(profiler.MLP):
+            a = rt.linear_packed(x, self.w_gate_up, tiled_out=rt.takes_tiled(self.w_down, x.shape[0]))
+            # may come in parts: the stream's next norm adds them
+            return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)

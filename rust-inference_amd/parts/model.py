@@ -9,6 +9,7 @@ import torch
 from ..cache import Cache, KVNeed
 from ..config import load_config
 from ..errors import ConfigError, ShapeError
+from .. import profiler
 from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec, load_checked
 from ..weights.random_init import random_tensors
@@ -109,15 +110,24 @@ class DecoderModel:
 
     # ---- cache
     def cache_needs(self) -> list:
-        """The need of every cache entry the schedule names."""
+        """The need of every cache entry the schedule names.  A layer says what it keeps per sequence
+        through its arrangement's ``cache_need()`` (by default its mixer's): one need, or a tuple of
+        them for a run that names a tuple of entries."""
         needs = [None] * self.spec.num_cache_entries
         for r in self.schedule:
-            if r.cache is None:
+            entries = r.entries()
+            if not entries:
                 continue
-            need = self.layers[r.layer].mixer.cache_need()
-            if needs[r.cache] is not None and needs[r.cache] != need:
-                raise ConfigError(f"cache entry {r.cache} is used with two different needs")
-            needs[r.cache] = need
+            layer = self.layers[r.layer]
+            asked = layer.cache_need() if hasattr(layer, "cache_need") else layer.mixer.cache_need()
+            asked = tuple(asked) if isinstance(asked, (tuple, list)) else (asked,)
+            if len(asked) != len(entries):
+                raise ConfigError(f"layer {r.layer} keeps {len(asked)} things per sequence, its run names "
+                                  f"{len(entries)} cache entries")
+            for entry, need in zip(entries, asked):
+                if needs[entry] is not None and needs[entry] != need:
+                    raise ConfigError(f"cache entry {entry} is used with two different needs")
+                needs[entry] = need
         return needs
 
     def new_cache(self, max_tokens: int, num_slots: int, max_seq_len: int | None = None, **kw) -> Cache:
@@ -131,7 +141,8 @@ class DecoderModel:
     def forward(self, ctx, cache: Cache) -> torch.Tensor:
         """float32 logits ``[n_want, vocab]`` for the wanted rows of this step's tokens."""
         rt = self.rt
-        stream = ResidualStream(self.embedding.forward(ctx.tokens))
+        with profiler.section(profiler.EMBEDDING):
+            stream = ResidualStream(self.embedding.forward(ctx.tokens))
         for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]
             follower = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
@@ -139,19 +150,25 @@ class DecoderModel:
             stream.next_entry_norm = entry() if entry else None
             tiled = getattr(follower, "entry_takes_tiled", None)
             stream.next_entry_tiled = tiled(stream.sum.shape[0]) if tiled else False
-            store, table = None, None
-            if run.cache is not None:
-                need = cache.needs[run.cache]
+            stores, tables = [], []
+            for entry in run.entries():
+                need = cache.needs[entry]
                 if isinstance(need, KVNeed):
-                    store = cache.kv(run.cache)
-                    table = ctx.page_tables[store.group_index]
-                elif need is not None:
-                    store = cache.state(run.cache)
+                    stores.append(cache.kv(entry))
+                    tables.append(ctx.page_tables[stores[-1].group_index])
+                else:
+                    stores.append(cache.state(entry) if need is not None else None)
+                    tables.append(None)
+            if isinstance(run.cache, (tuple, list)):          # a layer with several entries gets them all, in order
+                store, table = tuple(stores), tuple(tables)
+            else:
+                store, table = (stores[0], tables[0]) if stores else (None, None)
             layer.forward(stream, ctx, store, table, rt.dtype)
         if ctx.n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=rt.device)
         h = stream.normed(self.final_norm, rt.dtype, rows=ctx.want_rows)      # only the wanted rows
-        logits = self.head.forward(h)
+        with profiler.section(profiler.LM_HEAD):
+            logits = self.head.forward(h)
         if logits.shape != (ctx.n_want, self.spec.vocab_size):
             raise ShapeError(f"logits are {list(logits.shape)}")
         return logits

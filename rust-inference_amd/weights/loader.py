@@ -22,6 +22,7 @@ from .safetensors_io import ModelFolder
 MATRIX = "matrix"     # linear and embedding weights: N(0, 0.02) when random
 GAIN = "gain"         # norm gains: 1 + N(0, 0.1) when random; always used in 32-bit
 TABLE = "table"       # integer tables
+BIAS = "bias"         # biases of products: drawn like matrices when random, used in 32-bit like gains
 
 
 @dataclass(frozen=True)

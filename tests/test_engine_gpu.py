@@ -231,8 +231,8 @@ def test_trace_run_program(model_dirs, tmp_path, dtype_name):
 @pytest.mark.parametrize("seed", range(8))
 def test_configurations_drawn_at_random(tmp_path, seed):
     """Every size a configuration may have, drawn from lists that mix what the fast kernels take (head
-    sizes 32, 64, 128, widths that are multiples of 8) with what only the general ones do (head sizes 48,
-    80, 160, 256, odd widths, seven query heads a group): whole, last 32 one by one and an unequal
+    sizes 32, 64, 128, widths that are multiples of 8) with what only the general ones do (head sizes 8, 24,
+    40, 48, 72, 80, 160, 256, 320, odd widths, seven query heads a group): whole, last 32 one by one and an unequal
     batch, in both dtypes, against the plain implementation."""
     from rust_inference_amd.engine.replay import Replayer, engine_for_trace
     from rust_inference_amd.parts import load_model
@@ -243,7 +243,7 @@ def test_configurations_drawn_at_random(tmp_path, seed):
            "hidden_size": int(rng.choice([33, 50, 72, 75, 104, 129, 136, 264])),
            "intermediate_size": int(rng.choice([9, 37, 88, 101, 232, 250])),
            "num_hidden_layers": int(rng.integers(1, 4)), "num_attention_heads": kv * group, "num_key_value_heads": kv,
-           "head_dim": int(rng.choice([16, 32, 48, 64, 80, 128, 160, 256])),
+           "head_dim": int(rng.choice([8, 16, 24, 32, 40, 48, 64, 72, 80, 128, 160, 256, 320])),
            "rope_theta": float(rng.choice([1e4, 5e4, 1e6])), "rms_norm_eps": float(rng.choice([1e-6, 1e-5, 3e-6])),
            "tie_word_embeddings": bool(rng.integers(0, 2)), "max_position_embeddings": 512}
     folder = write_random_model(str(tmp_path / "m"), cfg, seed=seed, dtype=torch.bfloat16, matrix_std=0.12, gain_std=0.1)

@@ -181,6 +181,15 @@ def test_the_command_line_generates_what_the_plain_implementation_does(model_dir
     assert two.returncode == 0, two.stderr
     assert [[int(t) for t in ln.split()] for ln in two.stdout.strip().splitlines()] == [w[0] for w in want]
     assert "profile: 1 batches, 5 decode steps" in two.stderr
+    # the section table of src/profiler.rs:113-123 (src/bin/runner.rs:252-254): device time per kind of work
+    table = two.stderr[two.stderr.index("section "):].splitlines()
+    assert table[0].split() == ["section", "total(s)", "share", "calls"]
+    rows = {ln[:30].strip(): ln[30:].split() for ln in table[1:] if ln.strip()}
+    assert {"embedding", "attn q/k/v proj", "attention", "attn o proj", "rmsnorm", "dense mlp", "lm head",
+            "sampling"} <= set(rows)
+    assert rows["attention"][2] == "12" and rows["sampling"][2] == "6" and rows["lm head"][2] == "6"   # 2 layers x 6 steps
+    assert abs(sum(float(r[1].rstrip("%")) for r in rows.values()) - 100.0) < 1.0
+    assert "section " not in one.stderr                        # off unless asked for
     stop = want[1][0][2]
     cut = subprocess.run(base + ["-p", " ".join(map(str, prompts[1])), "--stop-token-ids", str(stop)],
                          capture_output=True, text=True, timeout=120)

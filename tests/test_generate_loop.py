@@ -3,7 +3,8 @@ import pytest
 import torch
 
 from rust_inference_amd.cache import Cache, KVNeed
-from rust_inference_amd.engine import generate, plan_batches, plan_step, StepEntry, wanted_indices
+from plain.step_layout_plain import plan_step
+from rust_inference_amd.engine import generate, plan_batches, StepEntry, wanted_indices
 from rust_inference_amd.errors import CacheError, ShapeError
 from rust_inference_amd.sampling import SamplingParams
 
@@ -230,6 +231,13 @@ def test_runner_refuses_what_it_cannot_do(tmp_path, capsys):
     assert "tokenizer.json" in capsys.readouterr().err
     assert main([str(tmp_path), "-p", ""]) == 1
     assert "empty prompt" in capsys.readouterr().err
+    # a text prompt where there is no tokenizer.json, and ids that are none: `error: ...` and exit status 1,
+    # as every other failure (src/bin/runner.rs:225-237), not a traceback
+    assert main([str(tmp_path), "-p", "once upon a time"]) == 1
+    err = capsys.readouterr().err
+    assert err.startswith("error: the prompt is text") and "tokenizer.json" in err and "Traceback" not in err
+    assert main([str(tmp_path), "--prompt-ids", "5,x,7"]) == 1
+    assert capsys.readouterr().err.startswith("error: --prompt-ids")
 
 
 def test_the_bound_that_sizes_a_decode_step():

@@ -83,6 +83,43 @@ def test_add_rmsnorm_adds_the_parts_of_a_split_product(ops):
     close(ops.add_rmsnorm(res2, p2, g2, 1e-6, torch.float32, rows), want, 2e-6, "gathered rows over parts")
 
 
+@pytest.mark.parametrize("pending_dtype", [torch.float32, torch.bfloat16])
+def test_add_rows_in_place_and_bias(ops, pending_dtype):
+    rng = np.random.default_rng(12)
+    res, pend = t(rng.normal(size=(7, 104))), t(rng.normal(size=(7, 104)), pending_dtype)
+    want = f64(res) + f64(pend)
+    got = ops.add_rows(res, pend, in_place=True)
+    assert got.data_ptr() == res.data_ptr()
+    close(res, want, 1e-7, "the sum is written into the residual itself")
+    bias = t(rng.normal(size=104))
+    x = t(rng.normal(size=(5, 104)), pending_dtype)
+    want = f64(x) + f64(bias)
+    close(ops.add_bias(x, bias), want, 1e-7 if pending_dtype == torch.float32 else 5e-3, "bias")
+
+
+@pytest.mark.parametrize("m, dim, partials, tiled", [(1, 104, 1, False), (5, 4096, 256, False), (16, 584, 37, True),
+                                                      (40, 4096, 4096, True)])
+def test_a_norm_left_to_a_product_can_be_finished_alone(ops, m, dim, partials, tiled):
+    """xg = bfloat16(r * gain) and partial sums of r^2 per row: the normed rows are xg / sqrt(sum / dim + eps)."""
+    rng = np.random.default_rng(m + dim)
+    r, gain = rng.normal(size=(m, dim)), 1 + 0.1 * rng.normal(size=dim)
+    xg = t(r * gain, torch.bfloat16)
+    ssq = rng.dirichlet(np.ones(partials), size=m) * (r * r).sum(1, keepdims=True)      # any split of the sums
+    if tiled:
+        data = ops.TiledRows.empty(m, dim, DEV)
+        data.data.zero_()
+        padded = torch.zeros((data.data.shape[0] * 16, data.data.shape[1] * 32), dtype=torch.bfloat16, device=DEV)
+        padded[:m, :dim] = xg
+        data.data.copy_(padded.view(-1, 16, data.data.shape[1], 4, 8).permute(0, 2, 3, 1, 4).reshape(data.data.shape))
+        assert torch.equal(data.rows(), xg)
+        src = data
+    else:
+        src = xg
+    got = ops.finish_norm(ops.NormedLater(src, t(ssq), 1e-6, dim))
+    want = f64(xg) / np.sqrt((r * r).sum(1, keepdims=True) / dim + 1e-6)
+    close(got, want, 5e-3, "finished norm")
+
+
 def test_add_rmsnorm_fused_equals_unfused_bit_for_bit(ops):
     # src/ops/norm.rs:84-98
     a, r = t([[0.5, -1.0, 2.0, 0.25]]), t([[1.0, 1.0, -1.0, 0.0]])
@@ -116,7 +153,8 @@ def paged(rng, lens, hkv, dh, page_size=32, dtype=torch.float32, spare=3):
 
 @pytest.mark.parametrize("paged_values", [False, True])
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
-@pytest.mark.parametrize("heads, kv_heads, dh", [(6, 2, 48), (4, 4, 128), (9, 1, 16), (2, 1, 256), (5, 5, 64), (8, 2, 32)])
+@pytest.mark.parametrize("heads, kv_heads, dh", [(6, 2, 48), (4, 4, 128), (9, 1, 16), (2, 1, 256), (5, 5, 64), (8, 2, 32),
+                                                 (4, 2, 8), (6, 3, 24), (3, 1, 40), (2, 2, 2), (2, 1, 328), (4, 2, 512)])
 def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh, paged_values):
     rng = np.random.default_rng(heads * dh)
     lens_before, new = [37, 0, 63, 30], [3, 2, 5, 70]            # writes cross page boundaries; one spans four pages
@@ -158,6 +196,43 @@ def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh, paged_value
     assert np.array_equal(f64(qkv2), qkv)
 
 
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("dh, rot", [(64, 16), (48, 24), (40, 8), (7, 4), (9, 0), (130, 128), (512, 64)])
+def test_rotation_over_part_of_the_head(ops, dtype, rel, dh, rot):
+    """The first `rot` elements of a head are rotated in pairs (i, i + rot/2) by frequencies of their own, the rest
+    is normed only; `rot` 0: no rotation at all, which an odd head size allows."""
+    rng = np.random.default_rng(dh + rot)
+    heads, kv_heads, new = 3, 1, [5, 40]
+    _, _, kp, vp, table = paged(rng, new, kv_heads, dh, dtype=dtype)
+    kp.zero_(); vp.zero_()
+    tokens = sum(new)
+    qkv_t = t(rng.normal(size=(tokens, (heads + 2 * kv_heads) * dh)) * 2, dtype)
+    qkv = f64(qkv_t)
+    tok_seq = [b for b, n in enumerate(new) for _ in range(n)]
+    tok_pos = [i for n in new for i in range(n)]
+    qg, kg = 1 + 0.2 * rng.normal(size=dh), 1 + 0.2 * rng.normal(size=dh)
+    inv = (1.0 / 10000.0 ** (np.arange(rot // 2) * 2.0 / max(rot, 1))).astype(np.float32) if rot else None
+    ops.qk_norm_rope_kv_write(qkv_t, t(qg), t(kg), 1e-5, None if inv is None else t(inv), t(tok_pos, torch.int32),
+                              t(tok_seq, torch.int32), table, kp, vp, heads, kv_heads, dh)
+
+    def want(x, gain):
+        y = P.rms_norm(x, f64(t(gain)), 1e-5)
+        if rot:
+            ang = (np.asarray(tok_pos, dtype=np.float32)[:, None] * inv[None, :]).astype(np.float32).astype(np.float64)
+            y = np.concatenate([P.apply_rope(y[..., :rot], ang), y[..., rot:]], -1)
+        return y
+    q = qkv[:, :heads * dh].reshape(tokens, heads, dh)
+    k = qkv[:, heads * dh:(heads + kv_heads) * dh].reshape(tokens, kv_heads, dh)
+    close(qkv_t[:, :heads * dh].reshape(tokens, heads, dh), want(q, qg), rel, "q")
+    tab = table.cpu().numpy()
+    k_want = want(k, kg)
+    for i in range(tokens):
+        close(kp[tab[tok_seq[i], tok_pos[i] // 32], :, tok_pos[i] % 32], k_want[i], rel, f"k of token {i}")
+    with pytest.raises(Exception, match="frequencies"):
+        ops.qk_norm_rope_kv_write(qkv_t, t(qg), t(kg), 1e-5, t(np.ones(dh // 2 + 1, dtype=np.float32)), t(tok_pos, torch.int32),
+                                  t(tok_seq, torch.int32), table, kp, vp, heads, kv_heads, dh)
+
+
 def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None, boost=None, kernel="generic"):
     k, v, kp, vp, table = paged(rng, lens, kv_heads, dh, dtype=dtype, spare=12)
     tokens = sum(new)
@@ -194,7 +269,10 @@ def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None,
 
 
 @pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
-@pytest.mark.parametrize("heads, kv_heads, dh", [(4, 2, 16), (6, 2, 48), (8, 1, 128), (3, 3, 64), (9, 1, 32)])
+@pytest.mark.parametrize("heads, kv_heads, dh", [(4, 2, 16), (6, 2, 48), (8, 1, 128), (3, 3, 64), (9, 1, 32),
+                                                 # any head size: the reference's own attention test runs 8
+                                                 # (src/attention.rs:189-219); odd ones; beyond 256
+                                                 (4, 2, 8), (6, 2, 24), (2, 1, 40), (3, 1, 7), (2, 2, 1), (2, 1, 328), (2, 1, 512)])
 def test_attention_prompts_pieces_and_single_tokens(ops, dtype, rel, heads, kv_heads, dh):
     rng = np.random.default_rng(heads + dh)
     # a whole prompt, a piece of five tokens at the end of 300, one token at 257 (a tile's first key), one at 1
@@ -678,9 +756,9 @@ def test_kernels_refuse_what_they_cannot_do(ops):
         ops.swiglu(torch.zeros(2, 4))
     with pytest.raises(KernelError, match="1 to 8"):
         ops.gemv_bf16(torch.zeros(9, 16, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV))
-    with pytest.raises(KernelError, match="multiple of 16"):
-        ops.attention(torch.zeros(1, 3 * 24, device=DEV), torch.zeros(1, 1, 32, 24, device=DEV),
-                      torch.zeros(1, 1, 24, 32, device=DEV), t([0], torch.int32), t([0], torch.int32),
-                      t([[0]], torch.int32), 1, 1, 24, None, 1.0)
+    with pytest.raises(KernelError, match="between 1 and 512"):
+        ops.attention(torch.zeros(1, 3 * 520, device=DEV), torch.zeros(1, 1, 32, 520, device=DEV),
+                      torch.zeros(1, 1, 520, 32, device=DEV), t([0], torch.int32), t([0], torch.int32),
+                      t([[0]], torch.int32), 1, 1, 520, None, 1.0)
     with pytest.raises(ShapeError, match="contiguous"):
         ops.swiglu(torch.zeros(4, 8, device=DEV)[:, ::2])

@@ -884,3 +884,216 @@ def test_a_norm_of_its_own(tmp_path, dtype_name):
         got = plans.collect(steps, lambda i: outs[i], CENTRED["vocab_size"])
         for rid, toks in reqs.items():
             assert_logits_close(got[rid], centred_plain(w, toks), dtype_name, f"centred norm, {what}, {rid}")
+
+
+# ------------------------------------------------------------------------------------------------ more parts than four
+SANDWICH = {"architectures": ["ToySandwichForCausalLM"], "vocab_size": 101, "hidden_size": 56, "inter": 72, "heads": 4,
+            "kv_heads": 2, "head_dim": 24, "rotated": 8, "period": 29, "eps": 1e-5, "theta": 10000.0}
+
+
+def register_sandwich():
+    """A layer with six named parts and two things kept per sequence: norms before AND after its attention
+    branch, a second mixer with a state of its own beside the attention, an attention with biases whose
+    position encoding rotates a third of each head and then, after the per-head norm, adds a learned row.
+
+        x = n1(h);  r = h + n1b(attention(x)) + running_sum(x);  h' = r + ff(n2(r))
+    """
+    from rust_inference_amd.cache import StateNeed
+    from rust_inference_amd.config import ModelConfig, register_architecture
+    from rust_inference_amd.parts import LayerSpec, Mixer, ModelSpec, PartSpec, PositionEncoding, Run, register_part
+    from rust_inference_amd.parts.registry import build_part
+    from rust_inference_amd.weights import MATRIX, TensorSpec
+
+    @register_part("position", "toy_part_rotary_then_add")
+    class PartRotaryThenAdd(PositionEncoding):
+        acts_after_norm = True
+
+        def __init__(self, rotated, theta, period, head_dim, name):
+            self.rotated, self.theta, self.period, self.head_dim, self.name = rotated, theta, period, head_dim, name
+
+        def tensors(self):
+            return {self.name: TensorSpec((self.period, self.head_dim), MATRIX)}
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.table = weights[self.name].to(rt.device, torch.float32)
+            i = torch.arange(self.rotated // 2, dtype=torch.float32)
+            self.inv_freq = (1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float32),
+                                             2.0 * i / float(self.rotated))).to(rt.device).contiguous()
+
+        def rotation_table(self):
+            return self.inv_freq                              # shorter than head_dim / 2: part of the head rotates
+
+        def apply_normed(self, qkv, ctx, heads, kv_heads, head_dim):
+            add = self.table[ctx.tok_pos.long() % self.period]
+            qk = qkv[:, :(heads + kv_heads) * head_dim].unflatten(1, (heads + kv_heads, head_dim))
+            qk.copy_((qk.float() + add[:, None, :]).to(qkv.dtype))
+
+    @register_part("mixer", "toy_running_sum")
+    class RunningSum(Mixer):
+        """y_t = W . (x_0 + .. + x_t) / 8: the state is the running sum, per sequence."""
+        def __init__(self, hidden, name):
+            self.hidden, self.name = hidden, name
+
+        def tensors(self):
+            return {self.name: TensorSpec((self.hidden, self.hidden), MATRIX)}
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.w = weights[self.name].to(rt.device, torch.float32)
+
+        def cache_need(self):
+            return StateNeed((self.hidden,), torch.float32)
+
+        def forward(self, x, ctx, store, page_table):
+            out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            begin = 0
+            for slot, n in zip(ctx.slot_list, ctx.new_counts):
+                total = store[slot] + torch.cumsum(x[begin:begin + n].float(), 0)
+                out[begin:begin + n] = (total / 8.0) @ self.w.T
+                store[slot] = total[-1]
+                begin += n
+            return out
+
+    @register_part("arrangement", "toy_sandwich")
+    class Sandwich:
+        def __init__(self, layer_spec):
+            p = layer_spec.parts                              # six parts by name: whatever this arrangement asks for
+            assert set(p) == {"mixer_norm", "mixer", "after_mixer_norm", "side_mixer", "feed_forward_norm", "feed_forward"}
+            self.mixer_norm = build_part("norm", p["mixer_norm"])
+            self.mixer = build_part("mixer", p["mixer"])
+            self.after_mixer_norm = build_part("norm", p["after_mixer_norm"])
+            self.side_mixer = build_part("mixer", p["side_mixer"])
+            self.feed_forward_norm = build_part("norm", p["feed_forward_norm"])
+            self.feed_forward = build_part("feed_forward", p["feed_forward"])
+
+        def parts(self):
+            return (self.mixer_norm, self.mixer, self.after_mixer_norm, self.side_mixer, self.feed_forward_norm,
+                    self.feed_forward)
+
+        def cache_need(self):
+            return (self.mixer.cache_need(), self.side_mixer.cache_need())    # keys and values, and a state
+
+        def forward(self, stream, ctx, store, page_table, act_dtype):
+            (kv, state), (table, _) = store, page_table
+            x = stream.normed(self.mixer_norm, act_dtype)
+            branch = self.mixer.forward(x, ctx, kv, table).float()
+            stream.push(self.after_mixer_norm.apply(branch, None, torch.float32))     # the norm of the branch alone
+            stream.push(self.side_mixer.forward(x, ctx, state, None))
+            stream.push(self.feed_forward.forward(stream.normed(self.feed_forward_norm, act_dtype), ctx))
+
+    @dataclass(frozen=True)
+    class SandwichConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        inter: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        rotated: int = 0
+        period: int = 0
+        eps: float = 1e-5
+        theta: float = 1e4
+        ARCHITECTURE: ClassVar[str] = "ToySandwichForCausalLM"
+        MODEL_TYPE: ClassVar[str] = "toy_sandwich"
+
+        @classmethod
+        def from_dict(cls, raw):
+            import dataclasses
+            return cls(**{f.name: raw[f.name] for f in dataclasses.fields(cls)})
+
+    def spec(c):
+        d = c.hidden_size
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"dim": d, "eps": c.eps, "name": name})
+
+        def layer(p):
+            return LayerSpec("toy_sandwich", parts={
+                "mixer_norm": norm(p + "n1"), "after_mixer_norm": norm(p + "n1b"), "feed_forward_norm": norm(p + "n2"),
+                "side_mixer": PartSpec("toy_running_sum", {"hidden": d, "name": p + "sum.weight"}),
+                "feed_forward": PartSpec("swiglu", {"hidden": d, "inter": c.inter, "prefix": p + "ff."}),
+                "mixer": PartSpec("attention", {
+                    "hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim, "prefix": p + "attn.",
+                    "qk_norm": True, "eps": c.eps, "window": None, "qkv_bias": True, "o_bias": True,
+                    "position": PartSpec("toy_part_rotary_then_add", {
+                        "rotated": c.rotated, "theta": c.theta, "period": c.period, "head_dim": c.head_dim,
+                        "name": p + "attn.position.weight"})})})
+        return ModelSpec(
+            architecture="ToySandwichForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
+            embedding=PartSpec("table", {"vocab": c.vocab_size, "dim": d, "name": "embed.weight"}),
+            layers=(layer("l0."), layer("l1.")),
+            schedule=(Run(0, (0, 1)), Run(1, (2, 3))),          # a run names both of its layer's cache entries
+            final_norm=norm("final.weight"),
+            head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": False}),
+            max_positions=256)
+
+    register_architecture("ToySandwichForCausalLM", SandwichConfig, spec, model_types=("toy_sandwich",))
+
+
+def sandwich_plain(w, ids):
+    c = SANDWICH
+    h = P.embedding(w["embed.weight"], ids)
+    pos = np.arange(len(ids))
+    rot, dh = c["rotated"], c["head_dim"]
+    inv = (np.float32(1.0) / np.power(np.float32(c["theta"]), (np.float32(2.0) * np.arange(rot // 2, dtype=np.float32))
+                                      / np.float32(rot), dtype=np.float32)).astype(np.float32)
+    ang = (pos.astype(np.float32)[:, None] * inv[None, :]).astype(np.float32).astype(np.float64)
+
+    def attn(x, p):
+        s = x.shape[0]
+        add = w[p + "attn.position.weight"][pos % c["period"]][:, None, :]
+
+        def head(name, n, gain):
+            y = (x @ w[f"{p}attn.{name}_proj.weight"].T + w[f"{p}attn.{name}_proj.bias"]).reshape(s, n, dh)
+            if gain is None:
+                return y
+            y = P.rms_norm(y, w[p + gain], c["eps"])
+            return np.concatenate([P.apply_rope(y[..., :rot], ang), y[..., rot:]], -1) + add
+        o = P.attention(head("q", c["heads"], "attn.q_norm.weight"), head("k", c["kv_heads"], "attn.k_norm.weight"),
+                        head("v", c["kv_heads"], None))
+        return o.reshape(s, -1) @ w[p + "attn.o_proj.weight"].T + w[p + "attn.o_proj.bias"]
+
+    for p in ("l0.", "l1."):
+        x = P.rms_norm(h, w[p + "n1"], c["eps"])
+        r = h + P.rms_norm(attn(x, p), w[p + "n1b"], c["eps"]) + (np.cumsum(x, 0) / 8.0) @ w[p + "sum.weight"].T
+        h = r + P.swiglu_mlp(P.rms_norm(r, w[p + "n2"], c["eps"]), w[p + "ff.gate_proj.weight"],
+                             w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+    return P.rms_norm(h, w["final.weight"], c["eps"]) @ w["head.weight"].T
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_a_layer_of_six_parts_that_keeps_two_things_per_sequence(tmp_path, dtype_name):
+    """Registered here, built by the unchanged model class and stepped by the unchanged engine: a layer whose
+    arrangement names six parts, whose run names two cache entries (keys and values, and a state), with a
+    head size of 24, biased products, a rotation over a third of the head and an encoding that acts after
+    the per-head norm.  Whole, token by token and in unequal batches on a cache whose slots come back."""
+    register_sandwich()
+    from rust_inference_amd.cache import KVNeed, StateNeed
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    from safetensors import safe_open
+    folder = write_random_model(str(tmp_path / "m"), SANDWICH, seed=21, dtype=torch.float32, matrix_std=0.12)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
+    assert {"l0.n1b", "l1.sum.weight", "l0.attn.q_proj.bias", "l1.attn.o_proj.bias", "l0.attn.position.weight"} <= set(w)
+    model = load_model(folder, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
+    needs = model.cache_needs()
+    assert needs[0] == needs[2] == KVNeed(2, 24, None) and isinstance(needs[1], StateNeed) and needs[1] == needs[3]
+    rng = np.random.default_rng(22)
+    reqs = {f"r{i}": [int(x) for x in rng.integers(0, SANDWICH["vocab_size"], n)] for i, n in enumerate([50, 7, 33, 70])}
+    for what, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 20)),
+                        ("batches", plans.unequal_batches([
+                            {k: (v, max(1, len(v) - 12)) for k, v in list(reqs.items())[:2]},
+                            {k: (v, max(1, len(v) - 30)) for k, v in list(reqs.items())[2:]}]))):
+        engine = engine_for_trace(model, plans.max_live_tokens(steps))
+        player, outs = Replayer(engine), {}
+        for s in steps:
+            logits = player.feed(s)
+            if logits is not None:
+                outs[s["step"]] = logits.cpu().numpy()
+        engine.cache.check_consistent()
+        got = plans.collect(steps, lambda i: outs[i], SANDWICH["vocab_size"])
+        for rid, toks in reqs.items():
+            assert_logits_close(got[rid], sandwich_plain(w, toks), dtype_name, f"sandwich, {what}, {rid}")
