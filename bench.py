@@ -7,11 +7,12 @@ The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
 context of 4,096.  A step is one decode step: every live sequence gets one more token, chosen
 greedily on the device.  Prints one JSON line: decoded tokens a second at batch 8 (`value`), the
-2,048-token prefill, the decode step's share of the HBM roofline, and decoding at batch 1 and 64.
+2,048-token prefill, the decode step's share of the HBM roofline, and decoding at batch 1 and 64
+(`points`: tokens a second, and beside each its milliseconds a step, the GB/s of the bytes the step has
+to read and their share of the HBM peak).
 """
 import argparse
 import json
-import os
 import sys
 import time
 
@@ -90,10 +91,6 @@ def main() -> int:
     cfg["max_position_embeddings"] = args.context
     torch.manual_seed(2)
     model = random_model(cfg, seed=2, dtype=torch.bfloat16)
-    if os.environ.get("RI_PREFETCH"):                      # experiment switch: prefetch weights beside the products
-        from rust_inference_amd.parts.runtime import WeightStream
-        model.rt.weight_stream = WeightStream(model.rt.device, int(os.environ.get("RI_PREFETCH_WGS", 512)),
-                                              int(os.environ.get("RI_PREFETCH_AHEAD", 1)))
     vocab = cfg["vocab_size"]
     gen = torch.Generator().manual_seed(2)
 
@@ -153,9 +150,12 @@ def main() -> int:
     achieved = step_bytes / (dt / args.steps) / 1e9
     points = {}
     if not args.no_points:
-        for b in (1, 64):
-            pdt, _ = decode_run(b, max(8, args.steps // 2), max(2, args.warmup // 2))
-            points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / pdt, 1)
+        for b in (1, 64):                # the same number of steps as the headline run, each with its own roofline
+            pdt, pctx = decode_run(b, args.steps, args.warmup)
+            points[f"decode_b{b}"] = round(b * args.steps / pdt, 1)
+            points[f"decode_b{b}_ms"] = round(1e3 * pdt / args.steps, 3)
+            points[f"decode_b{b}_gbs"] = round(decode_bytes(cfg, layers, b, pctx) / (pdt / args.steps) / 1e9, 1)
+            points[f"decode_b{b}_frac"] = round(points[f"decode_b{b}_gbs"] / HBM_PEAK_GBS, 4)
 
     flops = prefill_flops(cfg, layers, args.prompt)
     out = {

@@ -138,11 +138,6 @@ int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, c
 int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float eps, int dim, int rows, int x_tiled,
                    void* stream);
 
-// Reads `bytes` bytes from `data` (16-byte aligned) with `workgroups` workgroups and throws them away: what is
-// read lands in the memory-side cache for the kernel that wants it next.  sink: one device word that is
-// practically never written (it keeps the loads alive), may be NULL.
-int ri_prefetch(const void* data, long bytes, int workgroups, void* sink, void* stream);
-
 // x[t, i] += bias[i] in place (bias float32 [dim], x of dtype [rows, dim]).
 int ri_add_bias(void* x, int dtype, const float* bias, int rows, int dim, void* stream);
 

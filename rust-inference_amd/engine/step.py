@@ -233,21 +233,12 @@ class Engine:
         # the same keys and values to the same places twice changes nothing, and per-sequence
         # state is put back to where it was before the rehearsal
         saved = self.cache.snapshot_state()
-        stream = getattr(self.model.rt, "weight_stream", None)
-        if stream is not None:
-            with stream.recording():                          # the rehearsal also tells the order of the weights
-                self.model.forward(ctx, self.cache)
-        else:
-            self.model.forward(ctx, self.cache)
+        self.model.forward(ctx, self.cache)
         self.cache.restore_state(saved)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            if stream is not None:
-                with stream.playing(stream.order):
-                    dg.logits = self.model.forward(ctx, self.cache)
-            else:
-                dg.logits = self.model.forward(ctx, self.cache)
+            dg.logits = self.model.forward(ctx, self.cache)
         dg.graph, dg.ctx = graph, ctx
         dg.graph.replay()
         self.cache.commit(ctx.slot_list, ctx.new_counts)

@@ -129,12 +129,48 @@ def find_or_build() -> str:
     return build(alt)
 
 
+# Host-only sources: no kernels in them, so they also build for the host alone (with sanitizers).
+HOST_ONLY = ("host_cache.hip", "runtime.hip")
+
+
+def build_host_sanitized(out_dir: str) -> str:
+    """The host-only sources (the cache's bookkeeping, the writer of a step's layout) as a library of their
+    own, built for the host alone with the address and undefined-behaviour sanitizers.  For tests on a
+    machine without a GPU: the Python process that loads it must have the sanitizer's runtime preloaded
+    (``sanitizer_runtime()``), and ``RI_KERNEL_LIBRARY`` tells ``load()`` to take this file."""
+    hipcc = _hipcc()
+    os.makedirs(out_dir, exist_ok=True)
+    lib_path = os.path.join(out_dir, "libri_host_sanitized.so")
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())
+    cmd = [hipcc, "--cuda-host-only", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-fno-omit-frame-pointer",
+           "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           *[os.path.join(CSRC, f) for f in HOST_ONLY], "-o", lib_path]
+    proc = subprocess.run(cmd, capture_output=True, text=True, env=env)
+    if proc.returncode != 0:
+        raise KernelError(f"the sanitized host build failed:\n{proc.stderr[-4000:]}")
+    return lib_path
+
+
+def sanitizer_runtime() -> str:
+    """The address sanitizer's shared runtime of the compiler that ``build_host_sanitized`` uses."""
+    clang = os.path.join(os.path.dirname(os.path.realpath(_hipcc())), "..", "lib", "llvm", "bin", "clang")
+    for cand in (clang, "/opt/rocm/lib/llvm/bin/clang", "/opt/rocm/llvm/bin/clang"):
+        if os.path.exists(cand):
+            out = subprocess.run([cand, "-print-file-name=libclang_rt.asan-x86_64.so"], capture_output=True, text=True)
+            path = out.stdout.strip()
+            if out.returncode == 0 and os.path.isabs(path) and os.path.exists(path):
+                return path
+    raise KernelError("the address sanitizer's runtime library was not found beside the compiler")
+
+
 def load() -> ctypes.CDLL:
     """The kernel library, loaded once per process.  Raises KernelError when it
-    cannot be had: there is no other implementation to fall back to."""
+    cannot be had: there is no other implementation to fall back to.  ``RI_KERNEL_LIBRARY``
+    names a library to load instead of the one in the tree (a sanitized host build, in tests)."""
     global _lib
     if _lib is None:
-        path = find_or_build()
+        path = os.environ.get("RI_KERNEL_LIBRARY") or find_or_build()
         try:
             _lib = ctypes.CDLL(path)
         except OSError as e:

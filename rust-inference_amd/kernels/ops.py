@@ -55,7 +55,6 @@ _SIGNATURES = {
                                           c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "ri_add_bias": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
-    "ri_prefetch": [c_void_p, ctypes.c_long, c_int, c_void_p, c_void_p],
     "ri_finish_norm": [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -360,18 +359,6 @@ def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_p
 
 
 # ---------------------------------------------------------------- products
-# Called with the weight tensor a product is about to stream (the copy it really reads), before its kernel
-# is launched: ``parts.runtime.WeightStream`` learns the order of a step's weights from it.
-weight_hook = None
-
-
-def prefetch(w: torch.Tensor, workgroups: int, sink: torch.Tensor | None = None, stream: int | None = None) -> None:
-    """Reads the whole of ``w`` and throws it away (see csrc/prefetch.hip), on ``stream`` (a raw handle) or
-    the current one."""
-    _call("ri_prefetch", _dev(w, "w"), w.numel() * w.element_size(), int(workgroups),
-          _opt(sink, "sink", torch.int32), _stream() if stream is None else stream)
-
-
 def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``x @ w.T`` in true 32-bit arithmetic; ``x`` float32 ``[M, K]``, ``w`` float32 or bfloat16 ``[N, K]``."""
     m, k = x.shape
@@ -388,8 +375,6 @@ def gemv_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu
     m, k = x.shape
     n = w.shape[0] // 2 if swiglu else w.shape[0]
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    if weight_hook is not None:
-        weight_hook(w)
     _call("ri_gemv_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
           _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
     return out
@@ -471,8 +456,6 @@ def gemm_skinny_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bf
         raise ShapeError("a tiled result is bfloat16 and whole")
     flags = (TILED_X if isinstance(x, TiledRows) else 0) | (TILED_OUT if tiled_out else 0)
     xd = _dev(x.data, "x", torch.bfloat16) if isinstance(x, TiledRows) else _dev(x, "x", torch.bfloat16)
-    if weight_hook is not None:
-        weight_hook(wpacked)
     if tiled_out:
         out = TiledRows.empty(m, n, x.device)
         od = _dev(out.data, "out")
@@ -521,8 +504,6 @@ def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloa
         raise ShapeError("a tiled result is bfloat16")
     x_tiled = isinstance(x, TiledRows)
     out = TiledRows.empty(m, n, x.device) if tiled_out else torch.empty((m, n), dtype=out_dtype, device=x.device)
-    if weight_hook is not None:
-        weight_hook(wpacked)
     _call("ri_gemm_mid_packed_bf16", _dev(out.data if tiled_out else out, "out"), code(out_dtype),
           _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
           int(swiglu), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), _stream())
@@ -555,8 +536,6 @@ def linked_product(x, w: torch.Tensor, n: int, packed: bool, out_dtype=torch.bfl
         wd = _dev(w, "w", torch.bfloat16, (n * (2 if swiglu else 1), k))
     x_tiled = isinstance(xr, TiledRows)
     xd = _dev(xr.data, "x", torch.bfloat16) if x_tiled else _dev(xr, "x", torch.bfloat16, (m, k))
-    if weight_hook is not None:
-        weight_hook(w)
     # the packed kernel takes the layouts of x and of its result as one more argument
     layout = ((TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0),) if packed else ()
     if later is not None:

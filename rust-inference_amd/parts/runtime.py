@@ -61,63 +61,6 @@ def _packed_pays(n: int, k: int) -> bool:
     return n * k * 2 <= PACKED_MAX_BYTES and not (tiles > COMPUTE_UNITS and 0 < last_round < COMPUTE_UNITS // 2)
 
 
-class WeightStream:
-    """Reads every weight of a captured decode step toward the compute units one product ahead.
-
-    A decode step is a chain of products that each stream one matrix from HBM; between two of them (the
-    launch, the first loads' way to memory, the tail of the kernel before) HBM delivers nothing.  The
-    matrices depend on nothing, so while product ``j`` runs, a kernel on a second stream reads the matrix of
-    product ``j + ahead`` and throws it away: it lands in the memory-side cache, and its product streams it
-    from there.  The order of a step's weights is learnt from one step that is launched the plain way
-    (``recording``); a captured step then forks a prefetch before every product (``playing``).  No part knows:
-    the product wrappers in ``kernels.ops`` report the tensor they are about to read."""
-
-    def __init__(self, device, workgroups: int = 512, ahead: int = 1, max_bytes: int = 220_000_000):
-        self.device = device
-        self.workgroups, self.ahead, self.max_bytes = workgroups, ahead, max_bytes
-        self.side = torch.cuda.Stream(device)                    # default priority, like every stream here
-        self.sink = torch.zeros(1, dtype=torch.int32, device=device)
-        self.order: list = []
-        self._plan, self._at = None, 0
-
-    class _Mode:
-        def __init__(self, owner, hook, join):
-            self.owner, self.hook, self.join = owner, hook, join
-
-        def __enter__(self):
-            self.before, ops.weight_hook = ops.weight_hook, self.hook
-            return self.owner
-
-        def __exit__(self, *exc):
-            ops.weight_hook = self.before
-            if self.join:
-                torch.cuda.current_stream(self.owner.device).wait_stream(self.owner.side)
-            return False
-
-    def recording(self):
-        """Learn the order of a step's weights (the step runs as it would without this)."""
-        self.order = []
-        return self._Mode(self, self.order.append, False)
-
-    def playing(self, order):
-        """Fork a prefetch of the weight ``ahead`` products on before every product of the step."""
-        self._plan, self._at = list(order), 0
-        return self._Mode(self, self._before_product, True)
-
-    def _before_product(self, w) -> None:
-        plan, j = self._plan, self._at
-        self._at += 1
-        if plan is None or j >= len(plan) or plan[j] is not w:
-            self._plan = None                                    # another step than the one learnt: no guesses
-            return
-        nxt = plan[(j + self.ahead) % len(plan)]                 # past the end: the next step's first weights
-        if nxt.numel() * nxt.element_size() > self.max_bytes:
-            return
-        main = torch.cuda.current_stream(self.device)
-        self.side.wait_stream(main)                              # it starts when the product before this one is done
-        ops.prefetch(nxt, self.workgroups, self.sink, stream=self.side.cuda_stream)
-
-
 class PackedWeight:
     """A bfloat16 weight as the library product wants it (row-major) and, for decode-size products,
     packed into MFMA tiles."""
@@ -144,7 +87,6 @@ class Runtime:
             raise KernelError(f"this library computes on the GPU only, not on {self.device}")
         self.dtype = dtype
         self._mm_out_dtype = None
-        self.weight_stream = None          # a WeightStream when captured decode steps prefetch their weights
 
     # ---- weights
     def place_matrix(self, w: torch.Tensor) -> torch.Tensor:
@@ -256,8 +198,6 @@ class Runtime:
     def _library_mm(self, x, w, out_dtype):
         # The reference hands every product to a vendor library (src/cuda/mod.rs:186-232);
         # so does this path, for the shapes its own kernels do not cover.
-        if ops.weight_hook is not None:
-            ops.weight_hook(w)
         if out_dtype == torch.float32:
             if self._mm_out_dtype is None:
                 try:
