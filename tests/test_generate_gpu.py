@@ -24,21 +24,37 @@ def plain_greedy_with_margins(model_dir, prompts, steps, stop=()):
     return out
 
 
-def assert_same_tokens(got, want, dtype_name):
+def assert_same_tokens(got, want, dtype_name, model_dir=None, prompts=None, stop=()):
     """Token for token; in bfloat16 a sequence may part from the plain one only at a place where the
-    plain implementation's two best logits are closer than bfloat16 rounding of the logits."""
+    plain implementation's two best logits are closer than bfloat16 rounding of the logits.  With the model
+    folder and the prompts at hand the tokens after such a place are not let go unchecked: the plain
+    implementation is run again from the engine's own tokens up to there, and the engine's next tokens are
+    held to that continuation in the same way."""
     for i, (g, (toks, margins)) in enumerate(zip(got, want)):
-        for j, (a, b) in enumerate(zip(g, toks)):
-            if a != b:
-                assert dtype_name == "bfloat16" and margins[j] < 0.08, \
-                    f"request {i}, token {j}: {a} against {b} (margin {margins[j]:.3f}, {dtype_name})"
+        base = 0                                  # tokens of g before this point were forced on the plain side
+        while True:
+            parted = None
+            for j, (a, b) in enumerate(zip(g[base:], toks)):
+                if a != b:
+                    assert dtype_name == "bfloat16" and margins[j] < 0.08, \
+                        f"request {i}, token {base + j}: {a} against {b} (margin {margins[j]:.3f}, {dtype_name})"
+                    parted = base + j
+                    break
+            if parted is None:
+                # one side may have ended on a stop token (which is not put out) where the other picked another
+                # token: the same parting of ways, seen as a difference in length
+                j = min(len(g) - base, len(toks))
+                assert len(g) - base == len(toks) or (dtype_name == "bfloat16" and j < len(margins) and margins[j] < 0.08), \
+                    f"request {i}: {len(g)} tokens against {base + len(toks)}"
                 break
-        else:
-            # one side may have ended on a stop token (which is not put out) where the other picked another token:
-            # the same parting of ways, seen as a difference in length
-            j = min(len(g), len(toks))
-            assert len(g) == len(toks) or (dtype_name == "bfloat16" and j < len(margins) and margins[j] < 0.08), \
-                f"request {i}: {len(g)} tokens against {len(toks)}"
+            if model_dir is None or parted + 1 >= len(g):
+                break
+            # go on from the engine's own choice: the plain implementation continues prompt + g[:parted + 1]
+            cfg, w = read_model_f64(model_dir)
+            left = len(g) - (parted + 1)          # the plain side's first token is g's token parted + 1
+            toks, rows = P.greedy(cfg, w, list(prompts[i]) + list(g[:parted + 1]), left, stop)
+            margins = [float(np.sort(r)[-1] - np.sort(r)[-2]) for r in rows]
+            base = parted + 1
 
 
 def prompts_for(cfg, lengths, seed):
@@ -58,7 +74,8 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name, lengths, st
     prompts = prompts_for(cfg, lengths, 3)
     model = Model.load(model_dirs[name], dtype=dtype_name, max_batch=4, max_seq_len=96, use_graphs=use_graphs)
     res = model.generate(prompts, max_new_tokens=steps)
-    assert_same_tokens(res.tokens, plain_greedy_with_margins(model_dirs[name], prompts, steps), dtype_name)
+    assert_same_tokens(res.tokens, plain_greedy_with_margins(model_dirs[name], prompts, steps), dtype_name,
+                       model_dirs[name], prompts)
     assert res.finish_reasons == ["length"] * len(prompts)
     assert res.stats.prompt_tokens == sum(lengths) and res.stats.decode_tokens == len(prompts) * (steps - 1)
     model.cache.check_consistent()
@@ -85,7 +102,8 @@ def test_batches_of_tens_of_sequences(model_dirs, requests):
         outs.append(res)
     assert outs[0].tokens == outs[1].tokens and outs[0].finish_reasons == outs[1].finish_reasons
     assert "stop" in outs[0].finish_reasons
-    assert_same_tokens(outs[0].tokens, plain_greedy_with_margins(model_dirs["D"], prompts, 12, stop), "bfloat16")
+    assert_same_tokens(outs[0].tokens, plain_greedy_with_margins(model_dirs["D"], prompts, 12, stop), "bfloat16",
+                       model_dirs["D"], prompts, stop)
 
 
 def test_stop_tokens_and_batches_one_after_another(model_dirs):
