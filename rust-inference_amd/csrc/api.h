@@ -93,11 +93,6 @@ int ri_gemm_f32(float* out, const float* x, const void* w, int w_dtype, int m, i
 int ri_gemv_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
                  void* stream);
 
-// The same product on the matrix cores for M <= 16: eight wavefronts split K, weights stream straight
-// into the MFMA operand.  Same swiglu convention.
-int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k, int swiglu,
-                        void* stream);
-
 // The same with the weights packed ahead of time into MFMA tiles: [ceil(n/16)][ceil(k/32)][64 lanes][8],
 // lane l of a tile holding row l % 16, k 8 * (l / 16)..+8, zero beyond n and k; with swiglu the up matrix's
 // ceil(n/16) row tiles follow the gate's.
@@ -138,11 +133,27 @@ int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, c
 int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float eps, int dim, int rows, int x_tiled,
                    void* stream);
 
+// The packed product for 17 to 64 rows of x: four wavefronts a workgroup on four neighbouring row tiles share
+// the tiles of x through LDS.  parts > 1 cuts K into that many stretches whose float32 sums go to
+// out[parts][m][n]; ri_gemm_wide_packed_bf16_parts says how many parts fill the machine
+// for a matrix.  tiled as in ri_gemm_skinny_packed_bf16.
+int ri_gemm_wide_packed_bf16_parts(int n, int k);
+int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
+                             int swiglu, int parts, int tiled, int depth, void* stream);
+// (depth: 1 or 2 slices of eight weight fragments that a wavefront keeps in flight.  With parts > 1 and swiglu
+// the parts are [parts][m][2 n]: gate sums then up sums, the activation left to ri_sum_parts.)
+// out[m, i] = sum over p, in order, of parts[p][m][i] (float32 parts; out float32 or bfloat16, in rows or, for
+// bfloat16 and at most 64 rows, in the matrix cores' order).  swiglu: the parts' rows are 2 x width, gate sums
+// then up sums, and out[m, i] = silu(sum gate) * (sum up).
+int ri_sum_parts(void* out, int out_dtype, const float* parts, int n_parts, int rows, int width, int swiglu, int tiled,
+                 void* stream);
+
 // x[t, i] += bias[i] in place (bias float32 [dim], x of dtype [rows, dim]).
 int ri_add_bias(void* x, int dtype, const float* bias, int rows, int dim, void* stream);
 
 // out[t, i] = silu(y[t, i]) * y[t, inter + i]; y: [tokens, 2 * inter].
-int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream);
+// tiled: the bfloat16 result (at most 64 rows, inter a multiple of 8) in the matrix cores' order.
+int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, int tiled, void* stream);
 
 // ids[r] = first index of the maximum of logits[r, :] (float32).  workspace: ri_argmax_workspace_bytes(rows).
 int ri_argmax_workspace_bytes(int rows);

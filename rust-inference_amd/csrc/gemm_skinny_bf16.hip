@@ -3,9 +3,14 @@
 // a workgroup of four or eight wavefronts owns 16 rows of w, each wavefront its share of K; the weight
 // fragments go from global memory straight into the A operand (lane l: row l % 16, eight
 // consecutive k at 8 * (l / 16)), the rows of x into the B operand the same way (they come from
-// the L2 cache), and the eight partial sums are added through LDS in wavefront order.  Rows of x
+// the L2 cache), and the partial sums are added through LDS in wavefront order.  Rows of x
 // beyond M are zero columns, so a row's result does not depend on how many rows there are.
 // Optional SwiGLU epilogue for the fused gate|up matrix: out = silu(x . gate^T) * (x . up^T).
+// The weights are packed for the matrix cores ahead of time: the matrix is cut into tiles of 16 rows by
+// 32 k, each tile stored as the 1 KB that one MFMA A operand is (lane l's 16 bytes: row l % 16,
+// k 8 * (l / 16) ..+8), tiles of one row block consecutive in k.  A wavefront's loads are then whole
+// contiguous kilobytes, which is what the memory system streams fastest.
+// packed: [row_tiles][k_tiles][64 lanes][8]; for SwiGLU the up matrix's tiles follow the gate's.
 #include "api.h"
 #include "common.h"
 
@@ -24,64 +29,6 @@ union Frag {
 
 __device__ __forceinline__ float silu_sk(float z) { return z / (1.0f + expf(-z)); }
 
-template <int SK_WAVES, bool SWIGLU, typename TO>
-__global__ void __launch_bounds__(SK_WAVES * 64)
-gemm_skinny_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int M, int N,
-                        int K, int kslice) {
-    __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][4][64];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int i = lane & 15, jg = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    const bool row_ok = n0 + i < N, x_ok = i < M;
-    const int k_begin = wave * kslice, k_end = min(K, k_begin + kslice);
-    const bf16_t* wp = w + (size_t)(row_ok ? n0 + i : 0) * K + jg * 8;
-    const bf16_t* up = SWIGLU ? w + (size_t)(N + (row_ok ? n0 + i : 0)) * K + jg * 8 : nullptr;
-    const bf16_t* xp = x + (size_t)(x_ok ? i : 0) * K + jg * 8;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
-    for (int k = k_begin; k < k_end; k += 32 * SK_CHUNK) {
-        Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];
-#pragma unroll
-        for (int c = 0; c < SK_CHUNK; ++c) {
-            const int kk = k + c * 32;
-            const bool ok = kk + jg * 8 < k_end;          // K and the slices are multiples of 8: all eight or none
-            wf[c].u = (ok && row_ok) ? load_stream16(wp + kk) : zero;
-            if (SWIGLU) uf[c].u = (ok && row_ok) ? load_stream16(up + kk) : zero;
-            xf[c].u = (ok && x_ok) ? *reinterpret_cast<const uint4*>(xp + kk) : zero;
-        }
-#pragma unroll
-        for (int c = 0; c < SK_CHUNK; ++c) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
-            if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        red[0][wave][r][lane] = acc[r];
-        if (SWIGLU) red[1][wave][r][lane] = accu[r];
-    }
-    __syncthreads();
-    const int t = threadIdx.x;
-    if (t < 256) {
-        const int ln = t & 63, r = t >> 6;
-        float g = 0.f, u = 0.f;
-#pragma unroll
-        for (int wv = 0; wv < SK_WAVES; ++wv) {
-            g += red[0][wv][r][ln];
-            if (SWIGLU) u += red[1][wv][r][ln];
-        }
-        const int n = n0 + 4 * (ln >> 4) + r, m = ln & 15;    // D[row n, column m]
-        if (m < M && n < N) from_f32(out + (size_t)m * N + n, SWIGLU ? silu_sk(g) * u : g);
-    }
-}
-
-// The same product with the weights packed for the matrix cores ahead of time: the matrix is cut into
-// tiles of 16 rows by 32 k, each tile stored as the 1 KB that one MFMA A operand is (lane l's 16 bytes:
-// row l % 16, k 8 * (l / 16) ..+8), tiles of one row block consecutive in k.  A wavefront's loads are
-// then whole contiguous kilobytes, which is what the memory system streams fastest.
-// packed: [row_tiles][k_tiles][64 lanes][8]; for SwiGLU the up matrix's tiles follow the gate's.
 #define SK_ROWS (16 / SK_WAVES)   // rows of x whose sums of squares one wavefront adds up
 #define SK_PRE 4                  // partial sums of squares a lane fetches ahead of the weights
 
@@ -422,36 +369,5 @@ extern "C" int ri_gemm_mid_packed_bf16(void* out, int out_dtype, const void* x, 
     }
 #undef RI_MID_CASE
     RI_LAUNCH_CHECK("gemm_mid_packed_bf16");
-    return 0;
-}
-
-template <int WAVES, bool SWIGLU>
-static void launch_skinny(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k,
-                          hipStream_t s) {
-    const int kslice = ((k + WAVES - 1) / WAVES + 31) / 32 * 32;
-    const unsigned grid = (n + 15) / 16;
-    if (out_dtype == RI_F32)
-        gemm_skinny_bf16_kernel<WAVES, SWIGLU, float><<<grid, WAVES * 64, 0, s>>>((float*)out, x, w, m, n, k, kslice);
-    else
-        gemm_skinny_bf16_kernel<WAVES, SWIGLU, bf16_t><<<grid, WAVES * 64, 0, s>>>((bf16_t*)out, x, w, m, n, k, kslice);
-}
-
-extern "C" int ri_gemm_skinny_bf16(void* out, int out_dtype, const void* x, const void* w, int m, int n, int k,
-                                   int swiglu, void* stream) {
-    RI_REQUIRE(m > 0 && m <= 16, "gemm_skinny_bf16: %d rows of x, this kernel takes 1 to 16", m);
-    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
-    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_skinny_bf16: out dtype %d", out_dtype);
-    hipStream_t s = (hipStream_t)stream;
-    const bf16_t* xb = (const bf16_t*)x;
-    const bf16_t* wb = (const bf16_t*)w;
-    const bool eight = skinny_waves(n, k) == 8;
-    if (swiglu) {
-        if (eight) launch_skinny<8, true>(out, out_dtype, xb, wb, m, n, k, s);
-        else       launch_skinny<4, true>(out, out_dtype, xb, wb, m, n, k, s);
-    } else {
-        if (eight) launch_skinny<8, false>(out, out_dtype, xb, wb, m, n, k, s);
-        else       launch_skinny<4, false>(out, out_dtype, xb, wb, m, n, k, s);
-    }
-    RI_LAUNCH_CHECK("gemm_skinny_bf16");
     return 0;
 }

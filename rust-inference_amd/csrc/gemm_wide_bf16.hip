@@ -1,0 +1,249 @@
+// Products of 17 to 64 rows of x with a matrix packed for the matrix cores (pack_for_mfma):
+// out[M, N] = x[M, K] . w[N, K]^T, bfloat16 in, float32 sums.
+//
+// At this many rows the weights are still the traffic from memory (a step of 64 sequences reads every
+// weight once for 64 tokens), but every kilobyte of them meets RT kilobytes of x (RT tiles of 16 rows).  A
+// wavefront that fetches those for itself from the L2 cache asks that cache for four times what memory
+// delivers.  Here the four wavefronts of a workgroup work on four neighbouring row tiles of the matrix over
+// the same stretch of K and share the tiles of x through LDS: a slice of WD_SLICE steps (of 32 k) is copied
+// in once for all of them, in two buffers that take turns, so that there is one barrier a slice and the
+// copy of the next slice is in registers while this one is multiplied.  A wavefront keeps WD_SLICE weight
+// fragments in flight as a ring: a register asks for its step of the next slice as soon as the matrix
+// cores have taken the one it held.
+//
+// A matrix of a few thousand rows has too few groups of four row tiles to give every compute unit work,
+// so K is cut into `parts` stretches (blockIdx.y) whose float32 sums go to out[part][M][N] for a reader
+// that adds them in order (the residual stream's norm, or ri_sum_parts below).  A row's result does not
+// depend on the number of rows: rows beyond M are zero columns, every tile of x has accumulators of its own.
+#include "api.h"
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+union FragW {
+    bf16x8 v;
+    uint4 u;
+};
+
+#define WD_WAVES 4        // wavefronts of a workgroup: one row tile of the matrix each
+#define WD_SLICE 8        // MFMA steps (of 32 k) per slice of x in LDS
+
+__device__ __forceinline__ float silu_wd(float z) { return z / (1.0f + expf(-z)); }
+
+template <int RT, bool SWIGLU, typename TO, int NS>
+__global__ void __launch_bounds__(WD_WAVES * 64)
+gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked, int M,
+                        int N, int K, int k_tiles, int part_tiles, int row_tiles, int tiled) {
+    constexpr int PIECES = RT * WD_SLICE * 64;               // 16-byte pieces of x in a slice
+    constexpr int PER_THREAD = PIECES / (WD_WAVES * 64);     // of which a thread copies this many
+    static_assert(PIECES % (WD_WAVES * 64) == 0, "the copy divides evenly");
+    __shared__ uint4 xs[2][RT][WD_SLICE][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nt = blockIdx.x * WD_WAVES + wave;
+    const bool live_tile = nt < row_tiles;                    // past the edge: works on tile 0 again and stores nothing
+    const int kt_begin = blockIdx.y * part_tiles, kt_end = min(k_tiles, kt_begin + part_tiles);
+    const int slices = (kt_end - kt_begin + WD_SLICE - 1) / WD_SLICE;
+    const int ntc = live_tile ? nt : 0;
+    const bf16_t* wp = wpacked + ((size_t)ntc * k_tiles * 64 + lane) * 8;
+    const bf16_t* up = SWIGLU ? wpacked + ((size_t)(row_tiles + ntc) * k_tiles * 64 + lane) * 8 : nullptr;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    const bool x_tiled = tiled & TILED_X;
+    const int jg = lane >> 4;
+
+    // Every load below is issued whatever the indices are, from an address pulled back inside the data, and
+    // what lies outside is replaced by zero afterwards (x) or meets zeros (weights past the stretch's end meet
+    // a slice of x that is zero there).  A load inside a branch would end the pipelining: the compiler cannot
+    // count the loads in flight across a branch that may not have issued one, and waits for all of them.
+    // piece j of this thread's share of a slice: (tile of x, step) = q / WD_SLICE, q % WD_SLICE with
+    // q = wave + j * WD_WAVES; the 64 lanes of a wavefront copy one fragment (64 x 16 bytes)
+    auto fetch = [&](int j, int slice) -> uint4 {
+        const int q = wave + j * WD_WAVES;
+        const int step = q % WD_SLICE, rt = q / WD_SLICE;
+        const int row = rt * 16 + (lane & 15);
+        const int kt = kt_begin + slice * WD_SLICE + step;
+        const int ktc = min(kt, k_tiles - 1);
+        // rows beyond M and columns beyond K are zero (the packed matrix is zero beyond K too)
+        const bool ok = row < M && kt < kt_end && kt * 32 + jg * 8 < K;
+        const bf16_t* p = x_tiled ? x + (((size_t)rt * k_tiles + ktc) * 64 + lane) * 8
+                                  : x + (size_t)min(row, M - 1) * K + min(ktc * 32 + jg * 8, K - 8);
+        uint4 v = *reinterpret_cast<const uint4*>(p);
+        v.x = ok ? v.x : 0u;
+        v.y = ok ? v.y : 0u;
+        v.z = ok ? v.z : 0u;
+        v.w = ok ? v.w : 0u;
+        return v;
+    };
+    auto stash = [&](int j, int buf, const uint4& v) {
+        const int q = wave + j * WD_WAVES;
+        xs[buf][q / WD_SLICE][q % WD_SLICE][lane] = v;
+    };
+
+    floatx4 acc[RT], accu[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = accu[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // the weights of the first NS slices are asked for before anything else: a ring of NS * WD_SLICE registers
+    const int kt_last = kt_end - 1;
+    FragW wf[NS][WD_SLICE], uf[NS][WD_SLICE];
+#pragma unroll
+    for (int ss = 0; ss < NS; ++ss)
+#pragma unroll
+        for (int c = 0; c < WD_SLICE; ++c) {
+            const int kt = min(kt_begin + ss * WD_SLICE + c, kt_last);
+            wf[ss][c].u = load_stream16(wp + (size_t)kt * 512);
+            if (SWIGLU) uf[ss][c].u = load_stream16(up + (size_t)kt * 512);
+        }
+    uint4 stage[PER_THREAD];
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) stage[j] = fetch(j, 0);
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) stash(j, 0, stage[j]);
+    __syncthreads();
+
+    // (the number of slices is rounded up to a multiple of NS: a slice past the end is zeros of x against the
+    // stretch's last weights again)
+    const int rounds = (slices + NS - 1) / NS;
+    for (int round = 0; round < rounds; ++round) {
+#pragma unroll
+        for (int ss = 0; ss < NS; ++ss) {
+            const int s = round * NS + ss;
+            const int buf = s & 1;
+#pragma unroll
+            for (int j = 0; j < PER_THREAD; ++j) stage[j] = fetch(j, s + 1);   // past the last slice: zeros
+            const int kt0 = kt_begin + s * WD_SLICE;
+#pragma unroll
+            for (int c = 0; c < WD_SLICE; ++c) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    FragW xf;
+                    xf.u = xs[buf][rt][c][lane];
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ss][c].v, xf.v, acc[rt], 0, 0, 0);
+                    if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[ss][c].v, xf.v, accu[rt], 0, 0, 0);
+                }
+                // this register's step NS slices on (past the end: the stretch's last tile again, which then
+                // meets zeros of x)
+                const int next = min(kt0 + NS * WD_SLICE + c, kt_last);
+                wf[ss][c].u = load_stream16(wp + (size_t)next * 512);
+                if (SWIGLU) uf[ss][c].u = load_stream16(up + (size_t)next * 512);
+            }
+#pragma unroll
+            for (int j = 0; j < PER_THREAD; ++j) stash(j, buf ^ 1, stage[j]);
+            __syncthreads();       // the next slice is in place; this one may be overwritten after the next
+        }
+    }
+
+    if (!live_tile) return;
+    // D[row n, column m] of a tile: register r of lane l holds n = 4 * (l / 16) + r, m = l % 16.
+    // A product in parts stores its sums as they are; with the activation still to come, the gate sums fill
+    // columns 0..N-1 and the up sums N..2N-1 of rows 2 N wide.
+    const bool raw = gridDim.y > 1;
+    const int width = (SWIGLU && raw) ? 2 * N : N;
+    out += (size_t)blockIdx.y * M * width;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int m = rt * 16 + (lane & 15);
+        if (m >= M) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = nt * 16 + 4 * jg + r;
+            if (n >= N) continue;
+            if (SWIGLU && raw) {
+                from_f32(out + (size_t)m * width + n, acc[rt][r]);
+                from_f32(out + (size_t)m * width + N + n, accu[rt][r]);
+                continue;
+            }
+            const float v = SWIGLU ? silu_wd(acc[rt][r]) * accu[rt][r] : acc[rt][r];
+            from_f32(out + ((tiled & TILED_OUT) ? tiled_at(m, n, (N + 31) / 32) : (size_t)m * N + n), v);
+        }
+    }
+}
+
+// Into how many stretches K is cut: enough workgroups for every compute unit to have one, whole slices each
+// (measured on 4096 x 12288 at 64 rows: 66, 38, 26 and 26 us with 1, 2, 4 and 8 stretches; every stretch more is
+// another float32 copy of the result for the reader to add).
+extern "C" int ri_gemm_wide_packed_bf16_parts(int n, int k) {
+    const int groups = ((n + 15) / 16 + WD_WAVES - 1) / WD_WAVES;
+    const int k_tiles = (k + 31) / 32;
+    int parts = 1;
+    while (parts < 16 && groups * parts < 256 && k_tiles / (parts * 2) >= 2 * WD_SLICE) parts *= 2;
+    return parts;
+}
+
+template <int RT, bool SWIGLU, int NS>
+static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts,
+                        int tiled, hipStream_t s) {
+    const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
+    const int part_tiles = ((k_tiles + parts - 1) / parts + WD_SLICE - 1) / WD_SLICE * WD_SLICE;
+    dim3 grid((row_tiles + WD_WAVES - 1) / WD_WAVES, parts);
+    if (out_dtype == RI_F32)
+        gemm_wide_packed_kernel<RT, SWIGLU, float, NS><<<grid, WD_WAVES * 64, 0, s>>>(
+            (float*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
+    else
+        gemm_wide_packed_kernel<RT, SWIGLU, bf16_t, NS><<<grid, WD_WAVES * 64, 0, s>>>(
+            (bf16_t*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
+}
+
+// depth: slices of weights a wavefront keeps in flight (1 or 2)
+extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
+                                        int k, int swiglu, int parts, int tiled, int depth, void* stream) {
+    RI_REQUIRE(m > 0 && m <= 64, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 64", m);
+    RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_wide_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_wide_packed_bf16: out dtype %d", out_dtype);
+    RI_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || out_dtype == RI_F32),
+               "gemm_wide_packed_bf16: %d parts of K (more than one needs float32 sums)", parts);
+    RI_REQUIRE(!(tiled & ~(TILED_X | TILED_OUT)) && (!(tiled & TILED_OUT) || (out_dtype == RI_BF16 && parts == 1)),
+               "gemm_wide_packed_bf16: layout flags %d (a tiled result is bfloat16 and whole)", tiled);
+    RI_REQUIRE(depth == 1 || depth == 2, "gemm_wide_packed_bf16: depth %d", depth);
+    hipStream_t s = (hipStream_t)stream;
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)wpacked;
+#define RI_WIDE_GO(RT, SG, NS) launch_wide<RT, SG, NS>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s)
+#define RI_WIDE_CASE(RT)                                                                  \
+    if (swiglu) { if (depth == 2) RI_WIDE_GO(RT, true, 2); else RI_WIDE_GO(RT, true, 1); } \
+    else        { if (depth == 2) RI_WIDE_GO(RT, false, 2); else RI_WIDE_GO(RT, false, 1); }
+    if (m <= 16)      { RI_WIDE_CASE(1) }
+    else if (m <= 32) { RI_WIDE_CASE(2) }
+    else if (m <= 48) { RI_WIDE_CASE(3) }
+    else              { RI_WIDE_CASE(4) }
+#undef RI_WIDE_CASE
+#undef RI_WIDE_GO
+    RI_LAUNCH_CHECK("gemm_wide_packed_bf16");
+    return 0;
+}
+
+// ------------------------------------------------------------------ adding the parts of a split product
+// out[m, i] = sum over p, in order, of parts[p][m][i], for a reader that cannot add them itself; with swiglu the
+// rows of the parts are gate sums then up sums (2 x width) and out[m, i] = silu(sum gate) * (sum up).
+template <typename TO>
+__global__ void sum_parts_kernel(TO* __restrict__ out, const float* __restrict__ parts, int n_parts, long part_stride,
+                                 int width, int swiglu, int tiled, long total) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const int m = (int)(e / width), i = (int)(e - (long)m * width);
+    const float* p = parts + (long)m * (swiglu ? 2 * width : width) + i;
+    float g = 0.f, u = 0.f;
+    for (int q = 0; q < n_parts; ++q) {
+        g += p[q * part_stride];
+        if (swiglu) u += p[q * part_stride + width];
+    }
+    from_f32(out + (tiled ? tiled_at(m, i, (width + 31) / 32) : e), swiglu ? silu_wd(g) * u : g);
+}
+
+extern "C" int ri_sum_parts(void* out, int out_dtype, const float* parts, int n_parts, int rows, int width, int swiglu,
+                            int tiled, void* stream) {
+    RI_REQUIRE(n_parts > 0 && rows > 0 && width > 0, "sum_parts: %d parts of %d x %d", n_parts, rows, width);
+    RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "sum_parts: out dtype %d", out_dtype);
+    RI_REQUIRE(!tiled || (out_dtype == RI_BF16 && rows <= 64), "sum_parts: a tiled result is bfloat16 and at most 64 rows");
+    const long total = (long)rows * width;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    const long stride = total * (swiglu ? 2 : 1);
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == RI_F32)
+        sum_parts_kernel<float><<<blocks, 256, 0, s>>>((float*)out, parts, n_parts, stride, width, swiglu, tiled, total);
+    else
+        sum_parts_kernel<bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)out, parts, n_parts, stride, width, swiglu, tiled, total);
+    RI_LAUNCH_CHECK("sum_parts");
+    return 0;
+}

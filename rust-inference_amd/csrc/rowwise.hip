@@ -241,7 +241,10 @@ __global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ y, int 
 }
 
 // Eight bfloat16 elements per thread with 16-byte loads and stores, for inter a multiple of 8.
-__global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y, int inter8, long total8) {
+// tiled: the result lies in the matrix cores' order (at most 64 rows): eight columns from a multiple of 8 on are
+// neighbours there too.
+__global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y, int inter8, long total8,
+                                     int tiled) {
     const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= total8) return;
     const long t = e / inter8;
@@ -256,11 +259,14 @@ __global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __r
         const float b = silu(__uint_as_float(gw[k] & 0xFFFF0000u)) * __uint_as_float(uw[k] & 0xFFFF0000u);
         o[k] = pack_bf16x2(a, b);
     }
-    *reinterpret_cast<uint4*>(out + e * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    const size_t at = tiled ? tiled_at((int)t, i * 8, (inter8 * 8 + 31) / 32) : (size_t)e * 8;
+    *reinterpret_cast<uint4*>(out + at) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, void* stream) {
+extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int inter, int tiled, void* stream) {
     RI_REQUIRE(tokens > 0 && inter > 0, "swiglu: tokens %d, inter %d", tokens, inter);
+    RI_REQUIRE(!tiled || (dtype == RI_BF16 && inter % 8 == 0 && tokens <= 64),
+               "swiglu: a tiled result is bfloat16, at most 64 rows and a multiple of 8 wide");
     const long total = (long)tokens * inter;
     RI_REQUIRE((total + 255) / 256 <= 2147483647L, "swiglu: %ld elements exceed one launch", total);
     const unsigned grid = (unsigned)((total + 255) / 256);
@@ -269,7 +275,7 @@ extern "C" int ri_swiglu(void* out, const void* y, int dtype, int tokens, int in
         swiglu_kernel<float><<<grid, 256, 0, s>>>((float*)out, (const float*)y, inter, total);
     else if (dtype == RI_BF16 && inter % 8 == 0)
         swiglu_bf16x8_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y,
-                                                                                  inter / 8, total / 8);
+                                                                                  inter / 8, total / 8, tiled);
     else if (dtype == RI_BF16)
         swiglu_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, inter, total);
     else

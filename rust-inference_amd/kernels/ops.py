@@ -37,7 +37,6 @@ _SIGNATURES = {
                                        c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "ri_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemv_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-    "ri_gemm_skinny_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_sample": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_float,
                   c_void_p],
     "ri_mark_seen": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -45,6 +44,10 @@ _SIGNATURES = {
                         c_float, c_float, c_void_p],
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_mid_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "ri_gemm_wide_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_void_p],
+    "ri_gemm_wide_packed_bf16_parts": [c_int, c_int],
+    "ri_sum_parts": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_attention_decode_streams": [c_int, c_int, c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
@@ -53,7 +56,7 @@ _SIGNATURES = {
                             c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "ri_gemm_skinny_packed_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                           c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
-    "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "ri_swiglu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "ri_add_bias": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "ri_finish_norm": [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_int, c_void_p],
     "ri_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -169,13 +172,18 @@ def add_bias(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     return x
 
 
-def swiglu(y: torch.Tensor) -> torch.Tensor:
-    """``silu(y[:, :I]) * y[:, I:]`` for ``y: [T, 2 I]``."""
+def swiglu(y: torch.Tensor, tiled_out: bool = False):
+    """``silu(y[:, :I]) * y[:, I:]`` for ``y: [T, 2 I]``; ``tiled_out``: the bfloat16 result as ``TiledRows``
+    (at most 64 rows, ``I`` a multiple of 8)."""
     tokens, two_i = y.shape
     if two_i % 2:
         raise ShapeError(f"swiglu input has an odd width {two_i}")
-    out = torch.empty((tokens, two_i // 2), dtype=y.dtype, device=y.device)
-    _call("ri_swiglu", _dev(out, "out"), _dev(y, "y"), code(y.dtype), tokens, two_i // 2, _stream())
+    inter = two_i // 2
+    tiled_out = tiled_out and y.dtype == torch.bfloat16 and tokens <= 64 and inter % 8 == 0
+    out = TiledRows.empty(tokens, inter, y.device) if tiled_out else torch.empty((tokens, inter), dtype=y.dtype,
+                                                                                   device=y.device)
+    _call("ri_swiglu", _dev(out.data if tiled_out else out, "out"), _dev(y, "y"), code(y.dtype), tokens, inter,
+          int(tiled_out), _stream())
     return out
 
 
@@ -380,17 +388,6 @@ def gemv_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu
     return out
 
 
-def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, swiglu: bool = False) -> torch.Tensor:
-    """``x @ w.T`` for up to 16 bfloat16 rows on the matrix cores, the weights read once; ``swiglu`` as
-    in ``gemv_bf16``."""
-    m, k = x.shape
-    n = w.shape[0] // 2 if swiglu else w.shape[0]
-    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    _call("ri_gemm_skinny_bf16", _dev(out, "out"), code(out_dtype), _dev(x, "x", torch.bfloat16),
-          _dev(w, "w", torch.bfloat16, (w.shape[0], k)), m, n, k, int(swiglu), _stream())
-    return out
-
-
 def pack_for_mfma(w: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
     """A bfloat16 weight ``[N, K]`` cut into MFMA A-operand tiles: ``[ceil(N/16), ceil(K/32), 64, 8]``, lane
     ``l`` of a tile holding row ``l % 16`` and ``k = 8 * (l // 16) ..+8``, zero beyond N and K.  With
@@ -507,6 +504,53 @@ def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloa
     _call("ri_gemm_mid_packed_bf16", _dev(out.data if tiled_out else out, "out"), code(out_dtype),
           _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
           int(swiglu), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), _stream())
+    return out
+
+
+def wide_product_parts(n: int, k: int) -> int:
+    """Into how many stretches of K ``gemm_wide_packed_bf16`` cuts a product with an ``n x k`` matrix so
+    that the machine is full (host code only)."""
+    return _get("ri_gemm_wide_packed_bf16_parts")(int(n), int(k))
+
+
+def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16, swiglu: bool = False,
+                          parts: int = 1, tiled_out: bool = False, depth: int = 2):
+    """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by ``pack_for_mfma``,
+    the tiles of x shared by a workgroup's wavefronts through LDS: the product for steps of 17 to 64 tokens.
+    ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
+    that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
+    ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``."""
+    m, k = x.shape
+    row_tiles = -(-n // 16)
+    want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
+    if tuple(wpacked.shape) != want:
+        raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
+    if parts != 1 and (out_dtype != torch.float32 or tiled_out):
+        raise ShapeError("a product in parts has float32 sums in rows")
+    if tiled_out and out_dtype != torch.bfloat16:
+        raise ShapeError("a tiled result is bfloat16")
+    x_tiled = isinstance(x, TiledRows)
+    if tiled_out:
+        out = TiledRows.empty(m, n, x.device)
+    else:
+        out = torch.empty((m, n) if parts == 1 else (parts, m, 2 * n if swiglu else n), dtype=out_dtype, device=x.device)
+    _call("ri_gemm_wide_packed_bf16", _dev(out.data if tiled_out else out, "out"), code(out_dtype),
+          _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
+          int(swiglu), int(parts), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), int(depth), _stream())
+    return out
+
+
+def sum_parts(parts: torch.Tensor, out_dtype=torch.bfloat16, tiled_out: bool = False, swiglu: bool = False):
+    """``parts.sum(0)`` of float32 ``[parts, M, n]``, added in order, as ``out_dtype`` (bfloat16 also as
+    ``TiledRows``); with ``swiglu`` the rows are gate sums then up sums and the result ``silu(gate) * up``."""
+    p, m, n = parts.shape
+    if swiglu:
+        if n % 2:
+            raise ShapeError(f"gate and up sums side by side have an even width, not {n}")
+        n //= 2
+    out = TiledRows.empty(m, n, parts.device) if tiled_out else torch.empty((m, n), dtype=out_dtype, device=parts.device)
+    _call("ri_sum_parts", _dev(out.data if tiled_out else out, "out"), code(torch.bfloat16 if tiled_out else out_dtype),
+          _dev(parts, "parts", torch.float32), p, m, n, int(swiglu), int(tiled_out), _stream())
     return out
 
 

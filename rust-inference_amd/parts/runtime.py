@@ -35,6 +35,17 @@ SKINNY_MAX_ROWS = 16
 MID_MAX_ROWS = 64
 MID_MAX_BYTES = 20_000_000
 MID_TILED_ROWS = 32
+# 33 to 64 rows against a matrix with long rows whose result goes into the residual stream (`down`): the wide
+# kernel (ops.gemm_wide_packed_bf16: four row tiles a workgroup, the tiles of x shared through LDS) with K cut
+# into stretches that the next norm adds up.  Measured at Qwen3-8B sizes as graphs, in us, against the library
+# and the kernel above: 4096 x 12288 at 64 rows 26.0 : 38.8 : 38.6, at 32 rows 23.0 : 29.0 : 29.2; in the model
+# (where the norm that adds the stretches takes 3 us longer) decode at 64 sequences went from 7,150 to 7,340
+# tok/s and at 48 from 5,910 to 6,160, and at 24 and 32 it lost 1 to 3% to the kernel above.  On the
+# other matrices it only draws level (6144 x 4096 at 64 rows, with the kernel that adds its four stretches:
+# 21.7 : 18.3 : 24.4; 4096 x 4096 17.2 : 12.5 : 17.2; gate|up 51.0 : 52.1 : 52.4) and is not used.  All three
+# reach 3.9 TB/s on gate|up at 64 rows and 5 TB/s at 32, whatever they do with x: more weights in flight (a
+# ring of sixteen steps instead of eight) or more workgroups (K in stretches) change nothing there.
+WIDE_MIN_K = 8192
 SPLIT_K = 4096
 # Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation
 # rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
@@ -149,6 +160,8 @@ class Runtime:
             return False
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
+        if MID_TILED_ROWS < m <= MID_MAX_ROWS and not pw.swiglu and pw.k >= WIDE_MIN_K:
+            return True                                          # the wide kernel (where the reader adds its parts)
         return SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and self._mid_pays(pw, m, True)
 
     def linear_packed(self, x, pw: PackedWeight, out_dtype=None, parts_ok: bool = False, link=None,
@@ -187,13 +200,20 @@ class Runtime:
                 if not mine[1]:
                     return ops.gemv_bf16(ops.as_rows(x), pw.w, out_dtype, swiglu=pw.swiglu)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
+            if (MID_TILED_ROWS < m <= MID_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
+                    and pw.k >= WIDE_MIN_K):
+                # a long K at 33 to 64 rows: K in stretches, every stretch a workgroup that shares the tiles of x
+                # through LDS; the stream's next norm adds the stretches' sums
+                x = self.normed_now(x) if later else x
+                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=ops.wide_product_parts(pw.n, pw.k),
+                                                 depth=1)
             if (SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and pw.packed is not None
                     and self._mid_pays(pw, m, isinstance(x, ops.TiledRows))):
                 x = self.normed_now(x) if later else x
                 return ops.gemm_mid_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu,
                                                 tiled_out=tiled_out and out_dtype == torch.bfloat16)
         y = self.linear(x, pw.w, None if pw.swiglu else out_dtype)
-        return ops.swiglu(y) if pw.swiglu else y
+        return ops.swiglu(y, tiled_out=tiled_out) if pw.swiglu else y
 
     def _library_mm(self, x, w, out_dtype):
         # The reference hands every product to a vendor library (src/cuda/mod.rs:186-232);

@@ -536,22 +536,6 @@ def test_gemv_bf16(ops, m, out_dtype):
         assert torch.equal(ops.gemv_bf16(x, w, out_dtype)[m - 1:], ops.gemv_bf16(x[m - 1:].contiguous(), w, out_dtype))
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 13, 16])
-@pytest.mark.parametrize("n, k", [(37, 584), (100, 96), (4096, 4096), (50, 12288)])
-def test_gemm_skinny_bf16(ops, m, n, k):
-    rng = np.random.default_rng(m + n)
-    x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
-    want = f64(x) @ f64(w).T
-    close(ops.gemm_skinny_bf16(x, w, torch.float32), want, 3e-6, "skinny product")
-    close(ops.gemm_skinny_bf16(x, w, torch.bfloat16), want, 5e-3, "skinny product, bfloat16 out")
-    wgu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
-    y = f64(x) @ f64(wgu).T
-    close(ops.gemm_skinny_bf16(x, wgu, torch.float32, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 5e-6, "with swiglu")
-    if m > 1:      # a row's result does not depend on the other rows: bit for bit
-        assert torch.equal(ops.gemm_skinny_bf16(x, w, torch.float32)[m - 1:],
-                           ops.gemm_skinny_bf16(x[m - 1:].contiguous(), w, torch.float32))
-
-
 @pytest.mark.parametrize("m", [1, 3, 8, 16])
 @pytest.mark.parametrize("n, k", [(37, 584), (100, 96), (4096, 4096), (50, 12288), (320, 104)])
 def test_gemm_skinny_packed_bf16(ops, m, n, k):
@@ -560,8 +544,10 @@ def test_gemm_skinny_packed_bf16(ops, m, n, k):
     want = f64(x) @ f64(w).T
     packed = ops.pack_for_mfma(w)
     close(ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32), want, 3e-6, "packed skinny product")
-    # the same sums in the same order as the unpacked kernel: bit for bit
-    assert torch.equal(ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32), ops.gemm_skinny_bf16(x, w, torch.float32))
+    # a row's result does not depend on the other rows
+    if m > 1:
+        assert torch.equal(ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32)[m - 1:],
+                           ops.gemm_skinny_packed_bf16(x[m - 1:].contiguous(), packed, n, torch.float32))
     wgu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
     y = f64(x) @ f64(wgu).T
     close(ops.gemm_skinny_packed_bf16(x, ops.pack_for_mfma(wgu, swiglu=True), n, torch.bfloat16, swiglu=True),
@@ -570,6 +556,44 @@ def test_gemm_skinny_packed_bf16(ops, m, n, k):
         got = ops.gemm_skinny_packed_bf16(x, packed, n, torch.float32, parts=parts)
         assert got.shape == (parts, m, n)
         close(got.sum(0), want, 3e-6, f"{parts} parts of K")
+
+
+@pytest.mark.parametrize("m", [1, 16, 17, 33, 40, 49, 64])
+@pytest.mark.parametrize("n, k", [(37, 72), (1000, 1024), (584, 12288), (4096, 4096), (70, 264)])
+def test_wide_packed_product(ops, m, n, k):
+    """The product for steps of 17 to 64 tokens: whole, in parts of K that add up, with the activation, from and
+    into rows in the matrix cores' order; and a row's result does not depend on how many rows there are."""
+    rng = np.random.default_rng(m + n + k)
+    x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
+    want = f64(x) @ f64(w).T
+    packed = ops.pack_for_mfma(w)
+    whole = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32)
+    close(whole, want, 3e-6, "wide product")
+    close(ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16), want, 5e-3, "wide product, bfloat16 out")
+    for parts in (2, 3, ops.wide_product_parts(n, k)):
+        got = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=parts)
+        assert got.shape == ((parts, m, n) if parts > 1 else (m, n))
+        if parts > 1:
+            close(got.sum(0), want, 3e-6, f"{parts} parts of K")
+            close(ops.sum_parts(got, torch.float32), want, 3e-6, "parts added by the kernel")
+            assert torch.equal(ops.sum_parts(got, torch.bfloat16, tiled_out=True).rows(), ops.sum_parts(got, torch.bfloat16))
+    wgu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
+    y = f64(x) @ f64(wgu).T
+    pgu = ops.pack_for_mfma(wgu, swiglu=True)
+    close(ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 5e-3,
+          "wide, with swiglu")
+    raw = ops.gemm_wide_packed_bf16(x, pgu, n, torch.float32, swiglu=True, parts=2)        # the activation after the parts
+    assert raw.shape == (2, m, 2 * n)
+    close(ops.sum_parts(raw, torch.float32, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 5e-6, "swiglu over parts")
+    assert torch.equal(ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, depth=1), whole)    # the same sums either way
+    # rows in the matrix cores' order on either side: the same bits
+    tiled = ops.sum_parts(x.float()[None].contiguous(), torch.bfloat16, tiled_out=True)
+    assert torch.equal(tiled.rows(), x)
+    assert torch.equal(ops.gemm_wide_packed_bf16(tiled, packed, n, torch.float32), whole)
+    assert torch.equal(ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16, tiled_out=True).rows(),
+                       ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16))
+    if m > 1:
+        assert torch.equal(whole[m - 1:], ops.gemm_wide_packed_bf16(x[m - 1:].contiguous(), packed, n, torch.float32))
 
 
 @pytest.mark.parametrize("packed, m", [(False, 1), (False, 2), (False, 5), (True, 1), (True, 3), (True, 16)])
@@ -737,6 +761,11 @@ def test_swiglu(ops, dtype, rel):
     for inter in (333, 232, 1000):                 # odd, and multiples of 8 (the 16-byte form)
         y = t(rng.normal(size=(5, 2 * inter)) * 3, dtype)
         close(ops.swiglu(y), P.silu(f64(y)[:, :inter]) * f64(y)[:, inter:], rel, f"swiglu, {inter}")
+        tiled = ops.swiglu(y, tiled_out=True)      # the matrix cores' order where the kernel can (16-byte form, bfloat16)
+        if dtype == torch.bfloat16 and inter % 8 == 0:
+            assert isinstance(tiled, ops.TiledRows) and torch.equal(tiled.rows(), ops.swiglu(y))
+        else:
+            assert torch.equal(tiled, ops.swiglu(y))
 
 
 def test_argmax(ops):
