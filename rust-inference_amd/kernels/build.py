@@ -164,6 +164,63 @@ def sanitizer_runtime() -> str:
     raise KernelError("the address sanitizer's runtime library was not found beside the compiler")
 
 
+PLAIN_LIB_NAME = "libri_plain.so"
+PLAIN_SRC = os.path.join(CSRC, "plain")
+_plain = None
+
+
+def _plain_hash() -> str:
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(PLAIN_SRC)):
+        if name.endswith((".cpp", ".h")):
+            with open(os.path.join(PLAIN_SRC, name), "rb") as f:
+                h.update(name.encode() + f.read())
+    return h.hexdigest()[:16]
+
+
+def build_plain(out_dir: str | None = None) -> str:
+    """The plain C++ twins of the kernels (csrc/plain) as a host library of their own; no GPU code in it."""
+    out_dir = out_dir or _HERE
+    os.makedirs(out_dir, exist_ok=True)
+    lib_path = os.path.join(out_dir, PLAIN_LIB_NAME)
+    srcs = sorted(os.path.join(PLAIN_SRC, f) for f in os.listdir(PLAIN_SRC) if f.endswith(".cpp"))
+    cxx = shutil.which("g++") or shutil.which("c++")
+    # no -march: products and sums stay separate instructions, so float32 results are those of the plain text
+    cmd = ([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off"] if cxx else
+           [_hipcc(), "--cuda-host-only", "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off"])
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())
+    proc = subprocess.run([*cmd, *srcs, "-o", lib_path + ".tmp"], capture_output=True, text=True, env=env)
+    if proc.returncode != 0:
+        raise KernelError(f"building {PLAIN_LIB_NAME} failed:\n{proc.stderr[-4000:]}")
+    os.replace(lib_path + ".tmp", lib_path)
+    with open(lib_path + ".hash", "w") as f:
+        f.write(_plain_hash())
+    return lib_path
+
+
+def load_plain() -> ctypes.CDLL:
+    """The plain C++ twins, built at the first call where the library is not there or its sources changed."""
+    global _plain
+    if _plain is None:
+        path = os.path.join(_HERE, PLAIN_LIB_NAME)
+        stamp = path + ".hash"
+        current = os.path.exists(path) and os.path.exists(stamp) and open(stamp).read().strip() == _plain_hash()
+        if not current:
+            if os.access(_HERE, os.W_OK):
+                path = build_plain(_HERE)
+            else:
+                alt = os.path.join(tempfile.gettempdir(), f"ri_plain_{os.getuid()}_{_plain_hash()}")
+                path = os.path.join(alt, PLAIN_LIB_NAME)
+                if not os.path.exists(path):
+                    path = build_plain(alt)
+        try:
+            _plain = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load {path}: {e}") from None
+    return _plain
+
+
 def load() -> ctypes.CDLL:
     """The kernel library, loaded once per process.  Raises KernelError when it
     cannot be had: there is no other implementation to fall back to.  ``RI_KERNEL_LIBRARY``

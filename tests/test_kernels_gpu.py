@@ -791,3 +791,43 @@ def test_kernels_refuse_what_they_cannot_do(ops):
                       t([[0]], torch.int32), 1, 1, 520, None, 1.0)
     with pytest.raises(ShapeError, match="contiguous"):
         ops.swiglu(torch.zeros(4, 8, device=DEV)[:, ::2])
+
+
+def test_kernels_agree_with_their_plain_cpp_twins(ops):
+    """Each kernel family beside its scalar C++ twin (csrc/plain), float32: norm with the add, q/k norm and rotation,
+    attention over pages, the product, the activation, argmax."""
+    from rust_inference_amd.kernels import plain as N
+    rng = np.random.default_rng(21)
+    res, pend, gain = rng.normal(size=(5, 104)), rng.normal(size=(5, 104)), 1 + 0.1 * rng.normal(size=104)
+    r_t = t(res)
+    out = ops.add_rmsnorm(r_t, t(pend), t(gain), 1e-5, torch.float32)
+    total, want = N.add_rms_norm(res, pend, gain, 1e-5)
+    assert np.array_equal(r_t.cpu().numpy(), total)
+    close(out, want, 1e-6, "add + norm")
+    x, w = rng.normal(size=(7, 200)), rng.normal(size=(33, 200))
+    close(ops.gemm_f32(t(x), t(w)), N.linear(x, w), 2e-6, "product")
+    y = rng.normal(size=(4, 2 * 40)) * 3
+    close(ops.swiglu(t(y)), N.swiglu(y), 1e-6, "swiglu")
+    logits = rng.normal(size=(3, 1000)).astype(np.float32)
+    logits[1, 5] = logits[1, 700] = 9.0
+    assert ops.argmax(t(logits)).tolist() == [N.argmax(r) for r in logits]
+    heads, kv_heads, dh, lens = 6, 2, 24, [40, 70]
+    _, _, kp, vp, table = paged(rng, lens, kv_heads, dh)
+    kp.zero_(); vp.zero_()
+    tokens = sum(lens)
+    qkv = rng.normal(size=(tokens, (heads + 2 * kv_heads) * dh))
+    tok_seq = [b for b, n in enumerate(lens) for _ in range(n)]
+    tok_pos = [i for n in lens for i in range(n)]
+    qg, kg = 1 + 0.2 * rng.normal(size=dh), 1 + 0.2 * rng.normal(size=dh)
+    inv = N.rope_inv_freq(dh, 1e4)
+    qkv_t = t(qkv)
+    ops.qk_norm_rope_kv_write(qkv_t, t(qg), t(kg), 1e-6, t(inv), t(tok_pos, torch.int32), t(tok_seq, torch.int32),
+                              table, kp, vp, heads, kv_heads, dh)
+    q = qkv.astype(np.float32)[:, :heads * dh].reshape(tokens, heads, dh)
+    q_want = N.rope(N.rms_norm(q, qg, 1e-6), tok_pos, inv)
+    close(qkv_t[:, :heads * dh].reshape(tokens, heads, dh), q_want, 3e-6, "q norm and rotation")
+    got = ops.attention(qkv_t, kp, vp, t(tok_pos, torch.int32), t(tok_seq, torch.int32), table, heads, kv_heads, dh, None,
+                        1 / np.sqrt(dh))
+    want = N.attention(qkv_t.cpu().numpy()[:, :heads * dh].reshape(tokens, heads, dh), kp.cpu().numpy(), vp.cpu().numpy(),
+                       tok_pos, tok_seq, table.cpu().numpy(), None, 1 / np.sqrt(dh))
+    close(got.reshape(tokens, heads, dh), want, 3e-6, "attention over the pages the kernel wrote")
