@@ -29,6 +29,14 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 // where a row has 1,024 at most, four do, and the registers of more cost a small model 1.5%.
 #define GV_PRE_FEW 4
 #define GV_PRE_MANY 16
+// Steps of 512 k whose loads a wavefront with one row of x asks for together (see the loop below), for the
+// plain product and for the gate|up pair.
+#ifndef GV_AHEAD_PLAIN
+#define GV_AHEAD_PLAIN 4
+#endif
+#ifndef GV_AHEAD_GATED
+#define GV_AHEAD_GATED 4
+#endif
 
 template <int MT, bool SWIGLU, typename TO, int KS, int GV_PRE>
 __global__ void __launch_bounds__(GV_WAVES * RI_WAVE)
@@ -69,7 +77,42 @@ gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_
 
     float acc[MT] = {}, accu[MT] = {};
     if (row_ok) {
-        for (int k = k_begin + lane * 8; k < k_end; k += RI_WAVE * 8) {
+        // GV_AHEAD steps of 512 k at a time with all their loads asked for before the first is used: a wavefront
+        // then has GV_AHEAD (twice that with the up row) kilobytes of weights in flight instead of one.  The
+        // compiler keeps loads in flight only across code without branches, so the steps of a round are
+        // unrolled by hand and the rest of K, if any, follows one step at a time.  The same sums in the same order.
+        constexpr int GV_AHEAD = MT == 1 ? (SWIGLU ? GV_AHEAD_GATED : GV_AHEAD_PLAIN) : (MT == 2 ? 2 : 1);
+        int k = k_begin + lane * 8;
+        if (GV_AHEAD > 1) {
+            for (; k + (GV_AHEAD - 1) * RI_WAVE * 8 < k_end; k += GV_AHEAD * RI_WAVE * 8) {
+                uint4 wq[GV_AHEAD], uq[GV_AHEAD], xq[GV_AHEAD][MT];
+#pragma unroll
+                for (int a = 0; a < GV_AHEAD; ++a) {
+                    wq[a] = load_stream16(wr + k + a * RI_WAVE * 8);
+                    if (SWIGLU) uq[a] = load_stream16(wu + k + a * RI_WAVE * 8);
+#pragma unroll
+                    for (int m = 0; m < MT; ++m)
+                        xq[a][m] = *reinterpret_cast<const uint4*>(x + (size_t)(m < M ? m : 0) * K + k + a * RI_WAVE * 8);
+                }
+#pragma unroll
+                for (int a = 0; a < GV_AHEAD; ++a) {
+                    float wv[8], uv[8];
+                    unpack8(wq[a], wv);
+                    if (SWIGLU) unpack8(uq[a], uv);
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) {       // (rows beyond M repeat row 0 and are never stored: no branch here)
+                        float xv[8];
+                        unpack8(xq[a][m], xv);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            acc[m] = fmaf(xv[e], wv[e], acc[m]);
+                            if (SWIGLU) accu[m] = fmaf(xv[e], uv[e], accu[m]);
+                        }
+                    }
+                }
+            }
+        }
+        for (; k < k_end; k += RI_WAVE * 8) {
             float wv[8], uv[8];
             unpack8(load_stream16(wr + k), wv);
             if (SWIGLU) unpack8(load_stream16(wu + k), uv);
@@ -162,12 +205,13 @@ gemv_bf16_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_
     }
 }
 
-// How many wavefronts share a row: measured on MI355X with one row of x (decode at batch 1).  (Alone, the
-// gate|up pair of 2 x 12288 x 4096 is faster with four wavefronts a row, 35 us against 40 us; inside the
-// model, where it also finishes the norm before it, every workgroup adds up the row's partial sums of
-// squares first, four times the workgroups do that four times as often, and it is slower: 45 against 41.)
+// How many wavefronts share a row: measured on MI355X with one row of x (decode at batch 1).  A wavefront that
+// asks for four steps' loads at a time streams a row of 4,096 elements and more fastest alone (Qwen3-8B sizes,
+// tok/s at batch 1 with four, two and one wavefront on the rows of 12,288 elements: 308.5, 312.0, 313.4; with two
+// on the gate|up rows of 4,096: 303.0); shorter rows have no such rounds, and there two wavefronts a row keep
+// more loads in flight for a small matrix.
 static int gemv_k_split(int n, int k) {
-    if (k >= 8192) return 4;
+    if (k >= 4096) return 1;
     if ((long)n * k <= 4096L * 4096L) return 2;
     return 1;
 }
