@@ -82,23 +82,27 @@ struct PageFrags {
     Frag v[DH / 16];              // head_dim / 16 tiles of 16 channels, 32 keys deep
 };
 
+// `wanted` false: the fragments will not be used (the decode kernels keep their loads out of branches and ask
+// for a page even where a wavefront has none); every lane then reads the page's first 16 bytes, which costs
+// the memory system one line instead of sixteen kilobytes.
 template <int DH>
 __device__ __forceinline__ void load_page(PageFrags<DH>& f, const bf16_t* __restrict__ k_pages,
                                           const bf16_t* __restrict__ v_pages, long phys, int kv_heads, int kvh,
-                                          int lane) {
-    const int i = lane & 15, jg = lane >> 4;
+                                          int lane, bool wanted = true) {
+    const int w = wanted ? 1 : 0;
+    const int i = (lane & 15) * w, jg = (lane >> 4) * w;
     const bf16_t* kbase = k_pages + (phys * kv_heads + kvh) * (long)(PAGE * DH);
     const bf16_t* vbase = v_pages + (phys * kv_heads + kvh) * (long)(PAGE * DH);
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
-        const int row = (i >> 2) * 8 + kt * 4 + (i & 3);
+        const int row = (i >> 2) * 8 + (kt * 4 + (i & 3)) * w;
 #pragma unroll
         for (int ks = 0; ks < DH / 32; ++ks)
-            f.k[kt][ks].u = load_stream16(kbase + row * DH + ks * 32 + jg * 8);
+            f.k[kt][ks].u = load_stream16(kbase + row * DH + (ks * 32) * w + jg * 8);
     }
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt)
-        f.v[dt].u = load_stream16(vbase + (dt * 16 + i) * PAGE + jg * 8);
+        f.v[dt].u = load_stream16(vbase + ((dt * 16) * w + i) * PAGE + jg * 8);
 }
 
 // The state of NT tiles of 16 columns.  Lane l belongs to column l % 16 of every tile.
@@ -387,23 +391,30 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     // depends on the other's value, and each is a trip to memory that the page's loads would wait for in turn.
     const int page = chunk * (DECODE_CHUNK / PAGE) + wave;   // this wavefront's page
     const int qpos = tok_pos[tok];
-    const int phys = page_table[(long)b * table_width + min(page, table_width - 1)];
+    const int phys = max(page_table[(long)b * table_width + min(page, table_width - 1)], 0);   // not mapped: page 0, unused
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
 
+    // No load sits in a branch (the compiler counts loads in flight only along code without branches): a
+    // wavefront without a page of its own fetches page `phys` all the same, a lane without a column the
+    // group's last query, and neither is used.
     const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
-    PageFrags<DH> f;
-    if (has) load_page<DH>(f, k_pages, v_pages, phys, kv_heads, kvh, lane);
-
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
     const int jg = lane >> 4, col = lane & 15;
+    {
+        const bf16_t* qp = qkv + (long)tok * q_stride + (kvh * group + min(col, group - 1)) * DH + jg * 8;
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
+    }
+    PageFrags<DH> f;
+    load_page<DH>(f, k_pages, v_pages, phys, kv_heads, kvh, lane, has);
     if (col < group) {
         c.qpos[0] = qpos;
         c.lo[0] = lo;
-        const bf16_t* qp = qkv + (long)tok * q_stride + (kvh * group + col) * DH + jg * 8;
+    } else {
 #pragma unroll
-        for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
+        for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = make_uint4(0, 0, 0, 0);
     }
     if (has) process_page<DH, 1>(c, f, page, lane, scale_log2, false);
     finish_columns<DH, 1>(c);
@@ -561,28 +572,54 @@ static void launch_join(bf16_t* out, const float* ws, const int32_t* tok_pos, in
 }
 
 // ------------------------------------------------------------------ decode: the new token's own q, k and v
+// One head of the raw projection: per-head RMSNorm (when there is a gain), rotation (when there are
+// frequencies), rounded to bfloat16 into LDS.  The loads are apart from the arithmetic, so that a kernel can ask
+// for them before it asks for its pages and take the norm while the pages are on their way: every load is
+// issued by every lane from an address inside the row, none inside a branch (the compiler counts loads in
+// flight only along code without branches; anything else makes it wait for all of them).
+__device__ float ri_zero_row[256];                           // what an absent gain or frequency table is read from
+
 template <int DH>
-__device__ __forceinline__ void norm_rotate_head(bf16_t* dst_lds, const bf16_t* __restrict__ x,
-                                                 const float* __restrict__ gain, float eps,
-                                                 const float* __restrict__ inv_freq, int pos, int lane) {
+struct HeadLoads {
+    float x1, x2, g1, g2, f;                                 // the pair (d, d + DH/2), its gains, its frequency
+};
+
+template <int DH>
+__device__ __forceinline__ HeadLoads<DH> fetch_head(const bf16_t* __restrict__ x, const float* __restrict__ gain,
+                                                    const float* __restrict__ inv_freq, int lane) {
+    static_assert(DH <= 128 && (DH & (DH - 1)) == 0, "one (d, d + DH/2) pair per lane");
     constexpr int HALF = DH / 2;
-    float x1 = 0.f, x2 = 0.f, ss = 0.f;                      // DH <= 128: one pair per lane
-    if (lane < HALF) {
-        x1 = bf16_to_f32(x[lane]);
-        x2 = bf16_to_f32(x[lane + HALF]);
-        ss = x1 * x1 + x2 * x2;
+    const int d = lane & (HALF - 1);                         // lanes beyond HALF repeat the first ones' loads
+    const float* gp = gain ? gain : ri_zero_row;
+    const float* fp = inv_freq ? inv_freq : ri_zero_row;
+    HeadLoads<DH> h;
+    h.x1 = bf16_to_f32(x[d]);
+    h.x2 = bf16_to_f32(x[d + HALF]);
+    h.g1 = gp[d];
+    h.g2 = gp[d + HALF];
+    h.f = fp[d];
+    return h;
+}
+
+template <int DH>
+__device__ __forceinline__ void finish_head(bf16_t* dst_lds, const HeadLoads<DH>& h, bool normed, bool rotated,
+                                            float eps, int pos, int lane) {
+    constexpr int HALF = DH / 2;
+    const bool mine = lane < HALF;
+    float x1 = h.x1, x2 = h.x2;
+    if (normed) {
+        const float inv = 1.0f / sqrtf(wave_sum(mine ? x1 * x1 + x2 * x2 : 0.f) / (float)DH + eps);
+        x1 = x1 * inv * h.g1;
+        x2 = x2 * inv * h.g2;
     }
-    if (gain) {
-        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)DH + eps);
-        if (lane < HALF) { x1 = x1 * inv * gain[lane]; x2 = x2 * inv * gain[lane + HALF]; }
+    if (rotated) {
+        float sn, cs;
+        sincosf((float)pos * h.f, &sn, &cs);
+        const float a = x1 * cs - x2 * sn, b = x2 * cs + x1 * sn;
+        x1 = a;
+        x2 = b;
     }
-    if (lane < HALF) {
-        if (inv_freq) {
-            float sn, cs;
-            sincosf((float)pos * inv_freq[lane], &sn, &cs);
-            const float a = x1 * cs - x2 * sn, b = x2 * cs + x1 * sn;
-            x1 = a; x2 = b;
-        }
+    if (mine) {
         dst_lds[lane] = f32_to_bf16(x1);
         dst_lds[lane + HALF] = f32_to_bf16(x2);
     }
@@ -628,15 +665,32 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     const int p_last = min(c1 * (DECODE_CHUNK / PAGE) + DECODE_CHUNK / PAGE - 1, qpos / PAGE);   // below p_first: an empty run
     const int32_t* table = page_table + (long)b * table_width;
 
-    // This wavefront's pages are p_first + wave + STREAM_WAVES * j, j = 0, 1, ...; lane l holds the table's entry for
-    // j = base + l, fetched 64 at a time, so that a page's address never waits for a trip to memory of its own.
+    // This wavefront's pages are p_first + wave + STREAM_WAVES * j, j = 0 .. n_mine - 1, taken in blocks of
+    // 64 * HELD: lane l of held[i] holds the table's entry for page j = block + 64 * i + l of the block, fetched
+    // before the block begins, so that a page's address never waits for a trip to memory of its own.  No load
+    // of the walk sits in a branch (the compiler counts loads in flight only along code without branches, and
+    // otherwise waits for the page just asked for before it works on the one it has): an index past the end
+    // is pulled back to the last page, an entry that is not mapped reads page 0, and neither is used.
+    constexpr int HELD = 4;
     const int mine = p_first + wave;
-    int held = 0;
-    {
-        const int pg = mine + STREAM_WAVES * lane;
-        held = pg <= p_last ? table[pg] : 0;
-    }
-    auto phys_of = [&](int j) -> long { return (long)__builtin_amdgcn_readlane(held, j & 63); };
+    const int n_mine = mine <= p_last ? (p_last - mine) / STREAM_WAVES + 1 : 0;
+    int held[HELD];
+    auto fetch_table = [&](int j0) {
+#pragma unroll
+        for (int i = 0; i < HELD; ++i) {
+            const int j = min(j0 + 64 * i + lane, max(n_mine - 1, 0));
+            held[i] = max(table[min(mine + STREAM_WAVES * j, table_width - 1)], 0);
+        }
+    };
+    auto phys_of = [&](int r) -> long {                      // r: the page's number inside the block
+        int v = __builtin_amdgcn_readlane(held[0], r & 63);
+#pragma unroll
+        for (int i = 1; i < HELD; ++i) {
+            const int w = __builtin_amdgcn_readlane(held[i], r & 63);
+            v = (r >> 6) == i ? w : v;
+        }
+        return (long)v;
+    };
     auto open_page = [&](int pg) -> bool { return pg * PAGE + PAGE - 1 <= qpos && pg * PAGE >= lo; };
     // The group's queries and, where the run ends at the new token, its key and value.  These go into their
     // page before the workgroup reads any page: the barrier makes them visible to the wavefront that will
@@ -644,60 +698,61 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
     const int jg = lane >> 4, col = lane & 15;
+    fetch_table(0);
     if (FUSED) {
         const bf16_t* row = qkv + (long)b * q_stride;
         const int page_new = qpos / PAGE;
-        for (int g = wave; g < group; g += STREAM_WAVES)
-            norm_rotate_head<DH>(q_lds[g], row + (kvh * group + g) * DH, q_gain, eps, inv_freq, qpos, lane);
+        HeadLoads<DH> hq[4];                                 // up to 16 query heads a kv head: four a wavefront
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            hq[i] = fetch_head<DH>(row + (kvh * group + min(wave + STREAM_WAVES * i, group - 1)) * DH, q_gain, inv_freq, lane);
+        const HeadLoads<DH> hk = fetch_head<DH>(row + (heads + kvh) * DH, k_gain, inv_freq, lane);
+        const bf16_t* v_row = row + (heads + kv_heads + kvh) * DH;
+        const bf16_t v0 = v_row[lane & (DH - 1)], v1 = v_row[(lane + 64) & (DH - 1)];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (wave + STREAM_WAVES * i < group)
+                finish_head<DH>(q_lds[wave + STREAM_WAVES * i], hq[i], q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
         if (p_first <= p_last && p_last == page_new) {       // this run holds the new token's position
             const int slot = qpos % PAGE;
             const long head_base = ((long)table[page_new] * kv_heads + kvh) * (long)(PAGE * DH);
             if (wave == STREAM_WAVES - 1) {                  // the key: norm, rotation, into its page
-                norm_rotate_head<DH>(knew, row + (heads + kvh) * DH, k_gain, eps, inv_freq, qpos, lane);
+                finish_head<DH>(knew, hk, k_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
                 __builtin_amdgcn_wave_barrier();
                 for (int d = lane; d < DH; d += 64) k_pages[head_base + (long)slot * DH + d] = knew[d];
             } else if (wave == STREAM_WAVES - 2) {           // the value: a copy, transposed inside the page
-                for (int d = lane; d < DH; d += 64)
-                    v_pages[head_base + (long)d * PAGE + slot] = row[(heads + kv_heads + kvh) * DH + d];
+                if (lane < DH) v_pages[head_base + (long)lane * PAGE + slot] = v0;
+                if (lane + 64 < DH) v_pages[head_base + (long)(lane + 64) * PAGE + slot] = v1;
             }
         }
         __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks)
+            c.q[0][ks].u = *reinterpret_cast<const uint4*>(&q_lds[min(col, group - 1)][ks * 32 + jg * 8]);
+    } else {
+        const bf16_t* qp = qkv + (long)b * q_stride + (kvh * group + min(col, group - 1)) * DH + jg * 8;
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
     }
     if (col < group) {
         c.qpos[0] = qpos;
         c.lo[0] = lo;
-        if (FUSED) {
+    } else {
 #pragma unroll
-            for (int ks = 0; ks < DH / 32; ++ks)
-                c.q[0][ks].u = *reinterpret_cast<const uint4*>(&q_lds[col][ks * 32 + jg * 8]);
-        } else {
-            const bf16_t* qp = qkv + (long)b * q_stride + (kvh * group + col) * DH + jg * 8;
-#pragma unroll
-            for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
-        }
+        for (int ks = 0; ks < DH / 32; ++ks) c.q[0][ks].u = make_uint4(0, 0, 0, 0);
     }
     PageFrags<DH> fa, fb;
-    bool ha = mine <= p_last;
-    if (ha) load_page<DH>(fa, k_pages, v_pages, phys_of(0), kv_heads, kvh, lane);
-    for (int j = 0;; j += 2) {
-        const int pa = mine + STREAM_WAVES * j, pb = pa + STREAM_WAVES;
-        const bool hb = pb <= p_last;
-        if (hb) {
-            load_page<DH>(fb, k_pages, v_pages, phys_of(j + 1), kv_heads, kvh, lane);
+    for (int j0 = 0; j0 < n_mine; j0 += 64 * HELD) {
+        if (j0 > 0) fetch_table(j0);
+        const int n_blk = min(n_mine - j0, 64 * HELD);
+        load_page<DH>(fa, k_pages, v_pages, phys_of(0), kv_heads, kvh, lane);
+        for (int r = 0; r < n_blk; r += 2) {
+            const int pa = mine + STREAM_WAVES * (j0 + r), pb = pa + STREAM_WAVES;
+            load_page<DH>(fb, k_pages, v_pages, phys_of(min(r + 1, n_blk - 1)), kv_heads, kvh, lane, r + 1 < n_blk);
+            process_page<DH, 1>(c, fa, pa, lane, scale_log2, open_page(pa));
+            load_page<DH>(fa, k_pages, v_pages, phys_of(min(r + 2, n_blk - 1)), kv_heads, kvh, lane, r + 2 < n_blk);
+            if (r + 1 < n_blk) process_page<DH, 1>(c, fb, pb, lane, scale_log2, open_page(pb));
         }
-        if (ha) process_page<DH, 1>(c, fa, pa, lane, scale_log2, open_page(pa));
-        if (!hb) break;
-        const int pa2 = pb + STREAM_WAVES;
-        ha = pa2 <= p_last;
-        if (ha) {
-            if (((j + 2) & 63) == 0) {                       // the next 64 entries of the table
-                const int pg = pa2 + STREAM_WAVES * lane;
-                held = pg <= p_last ? table[pg] : 0;
-            }
-            load_page<DH>(fa, k_pages, v_pages, phys_of(j + 2), kv_heads, kvh, lane);
-        }
-        process_page<DH, 1>(c, fb, pb, lane, scale_log2, open_page(pb));
-        if (!ha) break;
     }
     finish_columns<DH, 1>(c);
 
@@ -790,42 +845,55 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;      // chunks last: the empty ones start last
     const int group = heads / kv_heads;
-    // the position and this wavefront's entry of the page table are asked for together (see above)
+    // 1. What needs nothing but the workgroup's indices is asked for first: the heads this wavefront will norm
+    // (two of the group's queries at most, and the new key), the new value, the position and this wavefront's
+    // entry of the page table.  An entry that is not mapped reads page 0, which is never used then.
+    const bf16_t* row = qkv + (long)b * q_stride;
+    const int g0 = min(wave, group - 1), g1 = min(wave + DECODE_WAVES, group - 1);
+    const HeadLoads<DH> hq0 = fetch_head<DH>(row + (kvh * group + g0) * DH, q_gain, inv_freq, lane);
+    const HeadLoads<DH> hq1 = fetch_head<DH>(row + (kvh * group + g1) * DH, q_gain, inv_freq, lane);
+    const HeadLoads<DH> hk = fetch_head<DH>(row + (heads + kvh) * DH, k_gain, inv_freq, lane);
+    const bf16_t* v_row = row + (heads + kv_heads + kvh) * DH;
+    const bf16_t v0 = v_row[lane & (DH - 1)], v1 = v_row[(lane + 64) & (DH - 1)];
     const int page = chunk * (DECODE_CHUNK / PAGE) + wave;
     const int qpos = tok_pos[b];                             // token b is sequence b's one new token
-    const int phys = page_table[(long)b * table_width + min(page, table_width - 1)];
+    const int phys = max(page_table[(long)b * table_width + min(page, table_width - 1)], 0);
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
     const bool owner = chunk == qpos / DECODE_CHUNK;         // this chunk holds the new token's position
 
-    // 1. this wavefront's page is on its way while the queries are made
+    // 2. this wavefront's page is on its way while the queries are made (a wavefront without a page of its own
+    // fetches page `phys` all the same and leaves it unused)
     const bool has = page * PAGE <= qpos && page * PAGE + PAGE - 1 >= lo;
     PageFrags<DH> f;
-    if (has) load_page<DH>(f, k_pages, v_pages, phys, kv_heads, kvh, lane);
-    const long phys_new = page_table[(long)b * table_width + qpos / PAGE];
+    load_page<DH>(f, k_pages, v_pages, phys, kv_heads, kvh, lane, has);
+    const long phys_new = owner ? page_table[(long)b * table_width + qpos / PAGE] : 0;
 
-    // 2. queries of the group; in the owner also the new key and value
-    const bf16_t* row = qkv + (long)b * q_stride;
-    for (int g = wave; g < group; g += DECODE_WAVES)
-        norm_rotate_head<DH>(q_lds[g], row + (kvh * group + g) * DH, q_gain, eps, inv_freq, qpos, lane);
+    // 3. queries of the group; in the owner also the new key and value
+    if (wave < group) finish_head<DH>(q_lds[wave], hq0, q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
+    if (wave + DECODE_WAVES < group)
+        finish_head<DH>(q_lds[wave + DECODE_WAVES], hq1, q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
     if (owner) {
         const int slot = qpos % PAGE;
         const long head_base = (phys_new * kv_heads + kvh) * (long)(PAGE * DH);
         if (wave == DECODE_WAVES - 1) {                      // the key: norm, rotation, into LDS and into its page
-            norm_rotate_head<DH>(knew, row + (heads + kvh) * DH, k_gain, eps, inv_freq, qpos, lane);
+            finish_head<DH>(knew, hk, k_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
             __builtin_amdgcn_wave_barrier();
             for (int d = lane; d < DH; d += 64) k_pages[head_base + (long)slot * DH + d] = knew[d];
         } else if (wave == DECODE_WAVES - 2) {               // the value: a copy, transposed inside the page
-            for (int d = lane; d < DH; d += 64) {
-                const bf16_t v = row[(heads + kv_heads + kvh) * DH + d];
-                vnew[d] = v;
-                v_pages[head_base + (long)d * PAGE + slot] = v;
+            if (lane < DH) {
+                vnew[lane] = v0;
+                v_pages[head_base + (long)lane * PAGE + slot] = v0;
+            }
+            if (lane + 64 < DH) {
+                vnew[lane + 64] = v1;
+                v_pages[head_base + (long)(lane + 64) * PAGE + slot] = v1;
             }
         }
     }
     __syncthreads();
 
-    // 3. this wavefront's page against the group's queries
+    // 4. this wavefront's page against the group's queries
     Columns<DH, 1> c;
     init_columns<DH, 1>(c);
     const int jg = lane >> 4, col = lane & 15;

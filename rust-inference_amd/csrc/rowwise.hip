@@ -78,7 +78,11 @@ __device__ __forceinline__ void store4(bf16_t* p, float4 v) {
     *reinterpret_cast<uint2*>(p) = w;
 }
 
-template <typename TP, typename TO, int VPT>
+// Every load is issued whatever the indices are, from an address pulled back inside the row, and a value from
+// outside is dropped afterwards: a load inside a branch or inside a loop of unknown length makes the compiler
+// wait for each one before the next is asked for (a norm over four parts of a split product took sixteen
+// trips to memory in turn that way).  PQ parts are fetched together; the sum is taken in the order of the parts.
+template <typename TP, typename TO, int VPT, int PQ>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const TP* __restrict__ pending,
                        int parts, size_t part_stride, const float* __restrict__ gain, float eps,
@@ -88,17 +92,34 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
     const size_t src = (size_t)(rows ? rows[row] : row) * dim;
     const bool write_back = rows == nullptr && pending != nullptr;
     float4 v[VPT], g[VPT];
+    int at[VPT];
+    bool ok[VPT];
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
         const int d = (i * 256 + threadIdx.x) * 4;
-        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (d < dim) {
-            v[i] = load4(residual + src + d);
-            g[i] = load4(gain + d);
-            if (pending) {
-                for (int q = 0; q < parts; ++q) {            // the parts of a split product, always in this order
-                    const float4 p = load4(pending + q * part_stride + src + d);
-                    v[i].x += p.x; v[i].y += p.y; v[i].z += p.z; v[i].w += p.w;
+        ok[i] = d < dim;
+        at[i] = ok[i] ? d : 0;
+        v[i] = load4(residual + src + at[i]);
+        g[i] = load4(gain + at[i]);
+    }
+    if (pending) {
+        for (int q0 = 0; q0 < parts; q0 += PQ) {                 // the parts of a split product, always in this order
+            float4 p[PQ][VPT];
+#pragma unroll
+            for (int j = 0; j < PQ; ++j) {
+                const size_t base = (size_t)min(q0 + j, parts - 1) * part_stride + src;
+#pragma unroll
+                for (int i = 0; i < VPT; ++i) p[j][i] = load4(pending + base + at[i]);
+            }
+#pragma unroll
+            for (int j = 0; j < PQ; ++j) {
+                const bool live = q0 + j < parts;
+#pragma unroll
+                for (int i = 0; i < VPT; ++i) {
+                    v[i].x = live ? v[i].x + p[j][i].x : v[i].x;
+                    v[i].y = live ? v[i].y + p[j][i].y : v[i].y;
+                    v[i].z = live ? v[i].z + p[j][i].z : v[i].z;
+                    v[i].w = live ? v[i].w + p[j][i].w : v[i].w;
                 }
             }
         }
@@ -106,9 +127,8 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int d = (i * 256 + threadIdx.x) * 4;
-        if (d < dim) {
-            if (write_back) store4(residual + src + d, v[i]);
+        if (ok[i]) {
+            if (write_back) store4(residual + src + at[i], v[i]);
             ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
         }
     }
@@ -116,11 +136,20 @@ add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ residual, const
     TO* o = out + (size_t)row * dim;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int d = (i * 256 + threadIdx.x) * 4;
-        if (d < dim)                                         // four columns of one chunk of eight either way
-            store4(tiled ? out + tiled_at(row, d, (dim + 31) / 32) : o + d, make_float4(v[i].x * inv * g[i].x, v[i].y * inv * g[i].y, v[i].z * inv * g[i].z,
-                                      v[i].w * inv * g[i].w));
+        if (ok[i])                                           // four columns of one chunk of eight either way
+            store4(tiled ? out + tiled_at(row, at[i], (dim + 31) / 32) : o + at[i],
+                   make_float4(v[i].x * inv * g[i].x, v[i].y * inv * g[i].y, v[i].z * inv * g[i].z,
+                               v[i].w * inv * g[i].w));
     }
+}
+
+template <typename TP, typename TO, int VPT>
+static void launch_add_rmsnorm_vec(TO* out, float* residual, const TP* pending, int parts, size_t ps, const float* gain,
+                                   float eps, const int32_t* rows, int n_rows, int dim, int tiled, hipStream_t s) {
+    if (parts > 1)
+        add_rmsnorm_vec_kernel<TP, TO, VPT, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
+    else
+        add_rmsnorm_vec_kernel<TP, TO, VPT, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
 }
 
 template <typename TP, typename TO>
@@ -128,13 +157,13 @@ static void launch_add_rmsnorm_typed(TO* out, float* residual, const TP* pending
                                      const float* gain, float eps, const int32_t* rows, int n_rows, int dim,
                                      int tiled, hipStream_t s) {
     if (dim % 4 == 0 && dim <= 1024)
-        add_rmsnorm_vec_kernel<TP, TO, 1><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
+        launch_add_rmsnorm_vec<TP, TO, 1>(out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, tiled, s);
     else if (dim % 4 == 0 && dim <= 2048)
-        add_rmsnorm_vec_kernel<TP, TO, 2><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
+        launch_add_rmsnorm_vec<TP, TO, 2>(out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, tiled, s);
     else if (dim % 4 == 0 && dim <= 4096)
-        add_rmsnorm_vec_kernel<TP, TO, 4><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
+        launch_add_rmsnorm_vec<TP, TO, 4>(out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, tiled, s);
     else if (dim % 4 == 0 && dim <= 8192)
-        add_rmsnorm_vec_kernel<TP, TO, 8><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim, tiled);
+        launch_add_rmsnorm_vec<TP, TO, 8>(out, residual, pending, parts, ps, gain, eps, rows, n_rows, dim, tiled, s);
     else
         add_rmsnorm_kernel<TP, TO><<<n_rows, 256, 0, s>>>(out, residual, pending, parts, ps, gain, eps, rows, dim);
 }
