@@ -133,13 +133,13 @@ int ri_gemm_skinny_packed_bf16_linked(void* out, int out_dtype, const void* x, c
 int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float eps, int dim, int rows, int x_tiled,
                    void* stream);
 
-// The packed product for 17 to 64 rows of x: four wavefronts a workgroup on four neighbouring row tiles share
-// the tiles of x through LDS.  parts > 1 cuts K into that many stretches whose float32 sums go to
-// out[parts][m][n]; ri_gemm_wide_packed_bf16_parts says how many parts fill the machine
-// for a matrix.  tiled as in ri_gemm_skinny_packed_bf16.
-int ri_gemm_wide_packed_bf16_parts(int n, int k);
+// The packed product for 17 to 64 rows of x: the three or four wavefronts of a workgroup, on as many
+// neighbouring row tiles, share the tiles of x through LDS.  parts > 1 cuts K into that many stretches whose
+// float32 sums go to out[parts][m][n]; ri_gemm_wide_packed_bf16_plan says how many wavefronts and parts fill
+// the machine most evenly for a matrix (with swiglu: never parts).  tiled as in ri_gemm_skinny_packed_bf16.
+int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts);
 int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
-                             int swiglu, int parts, int tiled, int depth, void* stream);
+                             int swiglu, int parts, int tiled, int depth, int waves, void* stream);
 // (depth: 1 or 2 slices of eight weight fragments that a wavefront keeps in flight.  With parts > 1 and swiglu
 // the parts are [parts][m][2 n]: gate sums then up sums, the activation left to ri_sum_parts.)
 // out[m, i] = sum over p, in order, of parts[p][m][i] (float32 parts; out float32 or bfloat16, in rows or, for

@@ -4,15 +4,19 @@
 // At this many rows the weights are still the traffic from memory (a step of 64 sequences reads every
 // weight once for 64 tokens), but every kilobyte of them meets RT kilobytes of x (RT tiles of 16 rows).  A
 // wavefront that fetches those for itself from the L2 cache asks that cache for four times what memory
-// delivers.  Here the four wavefronts of a workgroup work on four neighbouring row tiles of the matrix over
-// the same stretch of K and share the tiles of x through LDS: a slice of WD_SLICE steps (of 32 k) is copied
+// delivers.  Here the W wavefronts of a workgroup (three or four) work on W neighbouring row tiles of the
+// matrix over the same stretch of K and share the tiles of x through LDS: a slice of WD_SLICE steps (of 32 k) is copied
 // in once for all of them, in two buffers that take turns, so that there is one barrier a slice and the
 // copy of the next slice is in registers while this one is multiplied.  A wavefront keeps WD_SLICE weight
 // fragments in flight as a ring: a register asks for its step of the next slice as soon as the matrix
 // cores have taken the one it held.
 //
-// A matrix of a few thousand rows has too few groups of four row tiles to give every compute unit work,
-// so K is cut into `parts` stretches (blockIdx.y) whose float32 sums go to out[part][M][N] for a reader
+// A compute unit streams from memory at a rate of its own (about 30 GB/s here, an eighth of a thousandth of
+// the machine's), so the product is as fast as the fullest compute unit: the workgroups should be a multiple
+// of the compute units, all alike.  Three wavefronts instead of four do that for a matrix whose row tiles are
+// a multiple of three times the compute units (768 pairs of gate|up tiles: 256 workgroups of three, where
+// groups of four make 192 and leave a quarter of the machine idle).  A matrix of a few thousand rows has too
+// few groups of row tiles to give every compute unit work, so K is cut into `parts` stretches (blockIdx.y) whose float32 sums go to out[part][M][N] for a reader
 // that adds them in order (the residual stream's norm, or ri_sum_parts below).  A row's result does not
 // depend on the number of rows: rows beyond M are zero columns, every tile of x has accumulators of its own.
 #include "api.h"
@@ -26,22 +30,21 @@ union FragW {
     uint4 u;
 };
 
-#define WD_WAVES 4        // wavefronts of a workgroup: one row tile of the matrix each
 #define WD_SLICE 8        // MFMA steps (of 32 k) per slice of x in LDS
 
 __device__ __forceinline__ float silu_wd(float z) { return z / (1.0f + expf(-z)); }
 
-template <int RT, bool SWIGLU, typename TO, int NS>
-__global__ void __launch_bounds__(WD_WAVES * 64)
+// W: wavefronts of a workgroup, one row tile of the matrix each
+template <int RT, bool SWIGLU, typename TO, int NS, int W>
+__global__ void __launch_bounds__(W * 64)
 gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked, int M,
                         int N, int K, int k_tiles, int part_tiles, int row_tiles, int tiled) {
-    constexpr int PIECES = RT * WD_SLICE * 64;               // 16-byte pieces of x in a slice
-    constexpr int PER_THREAD = PIECES / (WD_WAVES * 64);     // of which a thread copies this many
-    static_assert(PIECES % (WD_WAVES * 64) == 0, "the copy divides evenly");
+    constexpr int FRAGS = RT * WD_SLICE;                     // fragments of x (64 pieces of 16 bytes) in a slice
+    constexpr int PER_THREAD = (FRAGS + W - 1) / W;          // of which a wavefront copies this many
     __shared__ uint4 xs[2][RT][WD_SLICE][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nt = blockIdx.x * WD_WAVES + wave;
+    const int nt = blockIdx.x * W + wave;
     const bool live_tile = nt < row_tiles;                    // past the edge: works on tile 0 again and stores nothing
     const int kt_begin = blockIdx.y * part_tiles, kt_end = min(k_tiles, kt_begin + part_tiles);
     const int slices = (kt_end - kt_begin + WD_SLICE - 1) / WD_SLICE;
@@ -57,9 +60,10 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
     // a slice of x that is zero there).  A load inside a branch would end the pipelining: the compiler cannot
     // count the loads in flight across a branch that may not have issued one, and waits for all of them.
     // piece j of this thread's share of a slice: (tile of x, step) = q / WD_SLICE, q % WD_SLICE with
-    // q = wave + j * WD_WAVES; the 64 lanes of a wavefront copy one fragment (64 x 16 bytes)
+    // q = wave + j * W; the 64 lanes of a wavefront copy one fragment (64 x 16 bytes).  Where the fragments do
+    // not divide among the wavefronts, the last one is copied twice (the same values to the same place).
     auto fetch = [&](int j, int slice) -> uint4 {
-        const int q = wave + j * WD_WAVES;
+        const int q = min(wave + j * W, FRAGS - 1);
         const int step = q % WD_SLICE, rt = q / WD_SLICE;
         const int row = rt * 16 + (lane & 15);
         const int kt = kt_begin + slice * WD_SLICE + step;
@@ -76,7 +80,7 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
         return v;
     };
     auto stash = [&](int j, int buf, const uint4& v) {
-        const int q = wave + j * WD_WAVES;
+        const int q = min(wave + j * W, FRAGS - 1);
         xs[buf][q / WD_SLICE][q % WD_SLICE][lane] = v;
     };
 
@@ -160,34 +164,52 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
     }
 }
 
-// Into how many stretches K is cut: enough workgroups for every compute unit to have one, whole slices each
-// (measured on 4096 x 12288 at 64 rows: 66, 38, 26 and 26 us with 1, 2, 4 and 8 stretches; every stretch more is
-// another float32 copy of the result for the reader to add).
-extern "C" int ri_gemm_wide_packed_bf16_parts(int n, int k) {
-    const int groups = ((n + 15) / 16 + WD_WAVES - 1) / WD_WAVES;
-    const int k_tiles = (k + 31) / 32;
+// How many wavefronts a workgroup has (row tiles it takes) and into how many stretches K is cut: of three and
+// four wavefronts the choice whose workgroups fill the compute units more evenly (four on a tie), with K cut
+// until every compute unit has a workgroup, whole slices each, and not at all with the activation (its parts
+// would have to be added by a kernel of their own).
+// (Measured on 4096 x 12288 at 64 rows with four wavefronts: 66, 38, 26 and 26 us with 1, 2, 4 and 8 stretches;
+// every stretch more is another float32 copy of the result for the reader to add.)
+static int wide_parts(int groups, int k_tiles, bool swiglu) {
     int parts = 1;
-    while (parts < 16 && groups * parts < 256 && k_tiles / (parts * 2) >= 2 * WD_SLICE) parts *= 2;
+    while (!swiglu && parts < 16 && groups * parts < 256 && k_tiles / (parts * 2) >= 2 * WD_SLICE) parts *= 2;
     return parts;
 }
 
-template <int RT, bool SWIGLU, int NS>
+extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts) {
+    const int row_tiles = (n + 15) / 16, k_tiles = (k + 31) / 32;
+    double best = -1.0;
+    for (int w = 4; w >= 3; --w) {
+        const int groups = (row_tiles + w - 1) / w;
+        const int p = wide_parts(groups, k_tiles, swiglu != 0);
+        const long wgs = (long)groups * p;
+        const double fill = (double)wgs / (double)((wgs + 255) / 256 * 256);
+        if (fill > best + 1e-9) {
+            best = fill;
+            *waves = w;
+            *parts = p;
+        }
+    }
+    return 0;
+}
+
+template <int RT, bool SWIGLU, int NS, int W>
 static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts,
                         int tiled, hipStream_t s) {
     const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
     const int part_tiles = ((k_tiles + parts - 1) / parts + WD_SLICE - 1) / WD_SLICE * WD_SLICE;
-    dim3 grid((row_tiles + WD_WAVES - 1) / WD_WAVES, parts);
+    dim3 grid((row_tiles + W - 1) / W, parts);
     if (out_dtype == RI_F32)
-        gemm_wide_packed_kernel<RT, SWIGLU, float, NS><<<grid, WD_WAVES * 64, 0, s>>>(
+        gemm_wide_packed_kernel<RT, SWIGLU, float, NS, W><<<grid, W * 64, 0, s>>>(
             (float*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
     else
-        gemm_wide_packed_kernel<RT, SWIGLU, bf16_t, NS><<<grid, WD_WAVES * 64, 0, s>>>(
+        gemm_wide_packed_kernel<RT, SWIGLU, bf16_t, NS, W><<<grid, W * 64, 0, s>>>(
             (bf16_t*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
 }
 
-// depth: slices of weights a wavefront keeps in flight (1 or 2)
+// depth: slices of weights a wavefront keeps in flight (1 or 2); waves: wavefronts (row tiles) a workgroup (3 or 4)
 extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
-                                        int k, int swiglu, int parts, int tiled, int depth, void* stream) {
+                                        int k, int swiglu, int parts, int tiled, int depth, int waves, void* stream) {
     RI_REQUIRE(m > 0 && m <= 64, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 64", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_wide_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_wide_packed_bf16: out dtype %d", out_dtype);
@@ -196,10 +218,15 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
     RI_REQUIRE(!(tiled & ~(TILED_X | TILED_OUT)) && (!(tiled & TILED_OUT) || (out_dtype == RI_BF16 && parts == 1)),
                "gemm_wide_packed_bf16: layout flags %d (a tiled result is bfloat16 and whole)", tiled);
     RI_REQUIRE(depth == 1 || depth == 2, "gemm_wide_packed_bf16: depth %d", depth);
+    RI_REQUIRE(waves == 3 || waves == 4, "gemm_wide_packed_bf16: %d wavefronts a workgroup (3 or 4)", waves);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)wpacked;
-#define RI_WIDE_GO(RT, SG, NS) launch_wide<RT, SG, NS>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s)
+#define RI_WIDE_GO(RT, SG, NS)                                                                       \
+    do {                                                                                             \
+        if (waves == 3) launch_wide<RT, SG, NS, 3>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s); \
+        else            launch_wide<RT, SG, NS, 4>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s); \
+    } while (0)
 #define RI_WIDE_CASE(RT)                                                                  \
     if (swiglu) { if (depth == 2) RI_WIDE_GO(RT, true, 2); else RI_WIDE_GO(RT, true, 1); } \
     else        { if (depth == 2) RI_WIDE_GO(RT, false, 2); else RI_WIDE_GO(RT, false, 1); }

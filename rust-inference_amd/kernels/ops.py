@@ -45,8 +45,8 @@ _SIGNATURES = {
     "ri_gemm_skinny_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_mid_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_gemm_wide_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                 c_void_p],
-    "ri_gemm_wide_packed_bf16_parts": [c_int, c_int],
+                                 c_int, c_void_p],
+    "ri_gemm_wide_packed_bf16_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
     "ri_sum_parts": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_attention_decode_streams": [c_int, c_int, c_int],
@@ -507,19 +507,23 @@ def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloa
     return out
 
 
-def wide_product_parts(n: int, k: int) -> int:
-    """Into how many stretches of K ``gemm_wide_packed_bf16`` cuts a product with an ``n x k`` matrix so
-    that the machine is full (host code only)."""
-    return _get("ri_gemm_wide_packed_bf16_parts")(int(n), int(k))
+def wide_product_plan(n: int, k: int, swiglu: bool = False) -> tuple[int, int]:
+    """``(waves, parts)``: how many wavefronts a workgroup of ``gemm_wide_packed_bf16`` should have and into how
+    many stretches of K it should cut a product with an ``n x k`` matrix so that the compute units are filled
+    evenly (host code only)."""
+    waves, parts = ctypes.c_int(0), ctypes.c_int(0)
+    _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), int(swiglu), ctypes.addressof(waves), ctypes.addressof(parts))
+    return waves.value, parts.value
 
 
 def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloat16, swiglu: bool = False,
-                          parts: int = 1, tiled_out: bool = False, depth: int = 2):
+                          parts: int = 1, tiled_out: bool = False, depth: int = 2, waves: int = 4):
     """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by ``pack_for_mfma``,
     the tiles of x shared by a workgroup's wavefronts through LDS: the product for steps of 17 to 64 tokens.
     ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
     that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
-    ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``."""
+    ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``.  ``waves``: wavefronts (row tiles) a
+    workgroup, 3 or 4 (``wide_product_plan``); the sums do not depend on it."""
     m, k = x.shape
     row_tiles = -(-n // 16)
     want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
@@ -536,7 +540,8 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
         out = torch.empty((m, n) if parts == 1 else (parts, m, 2 * n if swiglu else n), dtype=out_dtype, device=x.device)
     _call("ri_gemm_wide_packed_bf16", _dev(out.data if tiled_out else out, "out"), code(out_dtype),
           _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
-          int(swiglu), int(parts), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), int(depth), _stream())
+          int(swiglu), int(parts), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), int(depth),
+          int(waves), _stream())
     return out
 
 

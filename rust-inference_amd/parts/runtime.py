@@ -2,10 +2,18 @@
 dtype, and the matrix product that fits both."""
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from ..errors import KernelError, ShapeError
 from ..kernels import ops
+
+
+@functools.lru_cache(maxsize=None)
+def _wide_plan(n: int, k: int, swiglu: bool) -> tuple[int, int]:
+    """``ops.wide_product_plan``, asked once per matrix size."""
+    return ops.wide_product_plan(n, k, swiglu)
 
 # Which product kernel runs, by the number of rows of x (measured on MI355X at Qwen3-8B sizes with the
 # weights streamed from HBM through non-temporal loads, every variant replayed as a graph):
@@ -46,6 +54,13 @@ MID_TILED_ROWS = 32
 # reach 3.9 TB/s on gate|up at 64 rows and 5 TB/s at 32, whatever they do with x: more weights in flight (a
 # ring of sixteen steps instead of eight) or more workgroups (K in stretches) change nothing there.
 WIDE_MIN_K = 8192
+# The gate|up pair at 33 to 64 rows goes to the wide kernel where workgroups of three or four wavefronts with K
+# whole fill at least this share of the compute units' rounds (12288 pairs of rows: 256 workgroups of three,
+# at 64 rows 45 us against the library's 48 + 5 for the activation, at 48 rows 40 against 50; with groups of
+# four, 192 workgroups, it only drew level).  What bounds it then is what a compute unit can pull through its
+# vector memory path, about 30 GB/s whether the bytes come from memory or from the L2 cache: its share of the
+# weights plus all of x once.
+WIDE_GATED_FILL = 0.9
 SPLIT_K = 4096
 # Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation
 # rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
@@ -153,6 +168,17 @@ class Runtime:
             return True
         return tiled and m <= MID_TILED_ROWS
 
+    @staticmethod
+    def _wide_gated(pw: PackedWeight) -> bool:
+        """Whether the wide kernel takes a gate|up pair at 33 to 64 rows: where its workgroups (of three or
+        four wavefronts, K whole) fill the compute units evenly; else a quarter of the machine idles and the
+        library with its activation kernel is as fast."""
+        if pw.packed is None:
+            return False
+        waves, parts = _wide_plan(pw.n, pw.k, True)
+        groups = -(-(-(-pw.n // 16)) // waves) * parts
+        return groups / (-(-groups // 256) * 256) >= WIDE_GATED_FILL
+
     def takes_tiled(self, pw: PackedWeight, m: int) -> bool:
         """Whether the product of ``m`` rows with this weight runs on a packed kernel: whoever makes its
         rows then makes them as ``ops.TiledRows``."""
@@ -160,7 +186,7 @@ class Runtime:
             return False
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
-        if MID_TILED_ROWS < m <= MID_MAX_ROWS and not pw.swiglu and pw.k >= WIDE_MIN_K:
+        if MID_TILED_ROWS < m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu else pw.k >= WIDE_MIN_K):
             return True                                          # the wide kernel (where the reader adds its parts)
         return SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and self._mid_pays(pw, m, True)
 
@@ -205,8 +231,13 @@ class Runtime:
                 # a long K at 33 to 64 rows: K in stretches, every stretch a workgroup that shares the tiles of x
                 # through LDS; the stream's next norm adds the stretches' sums
                 x = self.normed_now(x) if later else x
-                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=ops.wide_product_parts(pw.n, pw.k),
-                                                 depth=1)
+                waves, parts = _wide_plan(pw.n, pw.k, False)
+                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
+            if MID_TILED_ROWS < m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw):
+                x = self.normed_now(x) if later else x
+                waves, _ = _wide_plan(pw.n, pw.k, True)
+                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=True, depth=1, waves=waves,
+                                                 tiled_out=tiled_out and out_dtype == torch.bfloat16)
             if (SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and pw.packed is not None
                     and self._mid_pays(pw, m, isinstance(x, ops.TiledRows))):
                 x = self.normed_now(x) if later else x

@@ -570,7 +570,7 @@ def test_wide_packed_product(ops, m, n, k):
     whole = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32)
     close(whole, want, 3e-6, "wide product")
     close(ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16), want, 5e-3, "wide product, bfloat16 out")
-    for parts in (2, 3, ops.wide_product_parts(n, k)):
+    for parts in (2, 3, ops.wide_product_plan(n, k)[1]):
         got = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=parts)
         assert got.shape == ((parts, m, n) if parts > 1 else (m, n))
         if parts > 1:
@@ -586,6 +586,14 @@ def test_wide_packed_product(ops, m, n, k):
     assert raw.shape == (2, m, 2 * n)
     close(ops.sum_parts(raw, torch.float32, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 5e-6, "swiglu over parts")
     assert torch.equal(ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, depth=1), whole)    # the same sums either way
+    # three row tiles a workgroup instead of four: the same sums again, whole, in parts and with the activation
+    assert torch.equal(ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, waves=3), whole)
+    assert torch.equal(ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=3, waves=3, depth=1),
+                       ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=3))
+    assert torch.equal(ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, waves=3, tiled_out=True).rows(),
+                       ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True))
+    waves, parts = ops.wide_product_plan(n, k, True)
+    assert waves in (3, 4) and parts == 1                   # the activation is never left to a second kernel
     # rows in the matrix cores' order on either side: the same bits
     tiled = ops.sum_parts(x.float()[None].contiguous(), torch.bfloat16, tiled_out=True)
     assert torch.equal(tiled.rows(), x)
