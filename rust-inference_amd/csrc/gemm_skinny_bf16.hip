@@ -65,14 +65,21 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     // latency hides behind the stream.  Partial sums of squares: wavefront w has the rows w, w + SK_WAVES, ...,
     // each lane SK_PRE of a row's partial sums (more are fetched afterwards).  And the element of the
     // residual stream and the gain that this thread's result meets.
+    // (None of these loads sits in a branch either: each is issued from an address inside its array, or inside
+    // the weights where there is no such array, and a value from outside is dropped.  In branches the compiler
+    // had every row's first load wait for the one before it: four trips to the L2 cache in turn before the
+    // first weight was asked for.)
     float pre[SK_ROWS][SK_PRE];
-    if (link.ssq_in) {
+    {
+        const float* sp = link.ssq_in ? link.ssq_in : reinterpret_cast<const float*>(wpacked);
 #pragma unroll
         for (int j = 0; j < SK_ROWS; ++j)
 #pragma unroll
             for (int q = 0; q < SK_PRE; ++q) {
                 const int m = wave + j * SK_WAVES, p = lane + q * 64;
-                pre[j][q] = (m < M && p < link.n_in) ? link.ssq_in[(size_t)m * link.n_in + p] : 0.f;
+                const bool have = link.ssq_in && m < M && p < link.n_in;
+                const float v = sp[have ? (size_t)m * link.n_in + p : 0];
+                pre[j][q] = have ? v : 0.f;
             }
     }
     const int t = threadIdx.x;
@@ -80,9 +87,12 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
     const int nl = 4 * (ln >> 4) + r, n = nt * 16 + nl, m = ln & 15;      // D[row n, column m]
     const bool ok = m < M && n < N;
     float res_pre = 0.f, gain_pre = 0.f;
-    if (link.residual && t < 256 && ok) {
-        res_pre = link.residual[(size_t)m * N + n];
-        gain_pre = link.next_gain[n];
+    {
+        const bool have = link.residual && t < 256 && ok;
+        const float* rp = link.residual ? link.residual : reinterpret_cast<const float*>(wpacked);
+        const float* gp = link.residual ? link.next_gain : reinterpret_cast<const float*>(wpacked);
+        res_pre = rp[have ? (size_t)m * N + n : 0];
+        gain_pre = gp[have ? n : 0];
     }
 
     floatx4 acc = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
@@ -196,6 +206,12 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
 // gate|up matrix against 4.6 with eight); a long K with few row tiles wants the eight (K = 12288, 256 tiles).
 // (Two wavefronts for that gate|up pair are 5% faster alone at 8 and 16 rows of x and 1 to 2% slower inside
 // the model, where each wavefront then adds up eight rows' sums of squares for the norm before it.)
+// (A matrix of 384 row tiles leaves half of 256 compute units with two workgroups and the others with one, and a
+// compute unit streams at a rate of its own: the launch takes as long as 512 tiles would.  Workgroups of three
+// half tiles (8 rows, two wavefronts each on half of K, a load fetching the rows for two steps of K at once) make
+// 256 equal workgroups of it and were slower all the same, 15.0 against 13.7 us at 8 rows: every step of K then
+// needs its rows of x for 8 rows of weights instead of 16, and a compute unit's vector memory path counts those
+// bytes from the L2 cache like the ones from memory.)
 static int skinny_waves(int n, int k) { return k >= 8192 ? 8 : 4; }
 
 template <int WAVES, bool SWIGLU>

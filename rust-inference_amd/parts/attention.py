@@ -121,7 +121,7 @@ class GroupedQueryAttention(Mixer):
                 o = ops.attention_decode_fused_bf16(qkv, self.q_gain, self.k_gain, self.eps, table, store.k_pages,
                                                     store.v_pages, ctx.tok_pos, page_table, ctx.B, ctx.max_len,
                                                     self.heads, self.kv_heads, self.head_dim, self.window, self.scale,
-                                                    tiled_out=rt.takes_tiled(self.w_o, ctx.B))
+                                                    tiled_out=rt.takes_tiled(self.w_o, ctx.B, self.b_o is None))
             return self.project_out(o, link)
         with profiler.section(profiler.QK_NORM_ROPE_APPEND):
             shape = (self.heads, self.kv_heads, self.head_dim)
@@ -143,7 +143,7 @@ class GroupedQueryAttention(Mixer):
     def project_out(self, o, link):
         with profiler.section(profiler.OUT_PROJECTION):
             if self.b_o is None:
-                return self.rt.linear_packed(o, self.w_o, link=link)
+                return self.rt.linear_packed(o, self.w_o, parts_ok=True, link=link)
             return ops.add_bias(self.rt.linear_packed(o, self.w_o), self.b_o)
 
     def attend(self, qkv, ctx, store, page_table):
@@ -155,7 +155,7 @@ class GroupedQueryAttention(Mixer):
             if ctx.is_decode:
                 return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                                  page_table, ctx.B, ctx.max_len, *args,
-                                                 tiled_out=self.rt.takes_tiled(self.w_o, ctx.B))
+                                                 tiled_out=self.rt.takes_tiled(self.w_o, ctx.B, self.b_o is None))
             return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                               page_table, ctx.B, ctx.max_new, *args)
         return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args)

@@ -44,6 +44,6 @@ class SwiGLU(FeedForward):
         # the activation is in the epilogue of the decode-size kernels, which hand the down product its rows
         # in the order it loads fastest when that product is a packed one too
         with profiler.section(profiler.MLP):
-            a = rt.linear_packed(x, self.w_gate_up, tiled_out=rt.takes_tiled(self.w_down, x.shape[0]))
+            a = rt.linear_packed(x, self.w_gate_up, tiled_out=rt.takes_tiled(self.w_down, x.shape[0], True))
             # may come in parts: the stream's next norm adds them
             return rt.linear_packed(a, self.w_down, parts_ok=True, link=link)

@@ -43,17 +43,17 @@ SKINNY_MAX_ROWS = 16
 MID_MAX_ROWS = 64
 MID_MAX_BYTES = 20_000_000
 MID_TILED_ROWS = 32
-# 33 to 64 rows against a matrix with long rows whose result goes into the residual stream (`down`): the wide
-# kernel (ops.gemm_wide_packed_bf16: four row tiles a workgroup, the tiles of x shared through LDS) with K cut
+# 33 to 64 rows against a matrix whose result goes into the residual stream (`o`, `down`): the wide kernel
+# (ops.gemm_wide_packed_bf16: three or four row tiles a workgroup, the tiles of x shared through LDS) with K cut
 # into stretches that the next norm adds up.  Measured at Qwen3-8B sizes as graphs, in us, against the library
 # and the kernel above: 4096 x 12288 at 64 rows 26.0 : 38.8 : 38.6, at 32 rows 23.0 : 29.0 : 29.2; in the model
-# (where the norm that adds the stretches takes 3 us longer) decode at 64 sequences went from 7,150 to 7,340
-# tok/s and at 48 from 5,910 to 6,160, and at 24 and 32 it lost 1 to 3% to the kernel above.  On the
-# other matrices it only draws level (6144 x 4096 at 64 rows, with the kernel that adds its four stretches:
-# 21.7 : 18.3 : 24.4; 4096 x 4096 17.2 : 12.5 : 17.2; gate|up 51.0 : 52.1 : 52.4) and is not used.  All three
-# reach 3.9 TB/s on gate|up at 64 rows and 5 TB/s at 32, whatever they do with x: more weights in flight (a
-# ring of sixteen steps instead of eight) or more workgroups (K in stretches) change nothing there.
-WIDE_MIN_K = 8192
+# decode at 64 sequences went from 7,150 to 7,340 tok/s and at 48 from 5,910 to 6,160, and at 24 and 32 it
+# lost 1 to 3% to the kernel above.  4096 x 4096 takes 14 us against the library's 18 inside the model (alone,
+# over a few copies of the matrix that the memory-side cache holds, the library needs 12.5: such small
+# matrices have to be timed in the model), worth 1% of the step at 40 and 48 sequences.  A product whose reader
+# cannot add stretches (q|k|v: 6144 x 4096, with a kernel of its own to add them 22 us against 15 to 18) stays
+# with the library.
+WIDE_MIN_K = 4096
 # The gate|up pair at 33 to 64 rows goes to the wide kernel where workgroups of three or four wavefronts with K
 # whole fill at least this share of the compute units' rounds (12288 pairs of rows: 256 workgroups of three,
 # at 64 rows 45 us against the library's 48 + 5 for the activation, at 48 rows 40 against 50; with groups of
@@ -179,14 +179,15 @@ class Runtime:
         groups = -(-(-(-pw.n // 16)) // waves) * parts
         return groups / (-(-groups // 256) * 256) >= WIDE_GATED_FILL
 
-    def takes_tiled(self, pw: PackedWeight, m: int) -> bool:
-        """Whether the product of ``m`` rows with this weight runs on a packed kernel: whoever makes its
-        rows then makes them as ``ops.TiledRows``."""
+    def takes_tiled(self, pw: PackedWeight, m: int, parts_ok: bool = False) -> bool:
+        """Whether the product of ``m`` rows with this weight (called with this ``parts_ok``) runs on a packed
+        kernel: whoever makes its rows then makes them as ``ops.TiledRows``."""
         if self.dtype != torch.bfloat16 or pw.packed is None or pw.k % 8:
             return False
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
-        if MID_TILED_ROWS < m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu else pw.k >= WIDE_MIN_K):
+        if MID_TILED_ROWS < m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu
+                                                   else parts_ok and pw.k >= WIDE_MIN_K):
             return True                                          # the wide kernel (where the reader adds its parts)
         return SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and self._mid_pays(pw, m, True)
 
