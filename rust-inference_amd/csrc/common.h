@@ -40,6 +40,12 @@ __device__ __forceinline__ size_t tiled_at(int m, int n, int k_tiles) {
     return (((size_t)(m >> 4) * k_tiles + (n >> 5)) * 64 + (m & 15) + 16 * ((n & 31) >> 3)) * 8 + (n & 7);
 }
 
+// One kilobyte of zeros: what a lane reads in place of a fragment piece that lies outside its matrix (rows beyond
+// M, columns beyond K), lane l at ri_zero_fragment + 8 * l.  The kernels keep their loads out of branches (the
+// compiler counts loads in flight only along code without branches) and choose the address instead; dropping a
+// loaded value afterwards works too, but makes the compiler wait for the load where the value is dropped.
+static __device__ bf16_t ri_zero_fragment[512];             // (never written; not const, which would move it to another address space and make every such load a flat one)
+
 // A 16-byte load of data that is read once (a weight matrix streaming through): marked non-temporal, so
 // that it does not displace what the caches hold to be used again.
 __device__ __forceinline__ uint4 load_stream16(const void* p) {

@@ -300,20 +300,61 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
     const int kt_begin = wave * tiles_per_wave, kt_end = min(k_tiles, kt_begin + tiles_per_wave);
     const bf16_t* wp = wpacked + ((size_t)nt * k_tiles * 64 + lane) * 8;
     const bf16_t* up = SWIGLU ? wpacked + ((size_t)(up_tile_offset + nt) * k_tiles * 64 + lane) * 8 : nullptr;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
     const bf16_t* xp[RT];
     bool x_ok[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         x_ok[rt] = rt * 16 + i < M;
-        xp[rt] = (tiled & TILED_X) ? x + ((size_t)rt * k_tiles * 64 + lane) * 8
+        // (RT may be more tiles than x has: 33 to 48 rows are three tiles and run with RT = 4.  A tile beyond
+        // the last is never read: the loop that asks for every fragment reads the last tile again instead.)
+        xp[rt] = (tiled & TILED_X) ? x + ((size_t)min(rt, (M - 1) >> 4) * k_tiles * 64 + lane) * 8
                                    : x + (size_t)(x_ok[rt] ? rt * 16 + i : 0) * K + jg * 8;
     }
     const int x_step = (tiled & TILED_X) ? 512 : 32;         // elements from one step's fragment to the next
     floatx4 acc[RT], accu[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = accu[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // the same in every wavefront of the launch: K in whole steps, every wavefront's share whole rounds of CH
+    const bool ring = K % 32 == 0 && tiles_per_wave % CH == 0 && k_tiles == tiles_per_wave * SK_WAVES;
+    if (ring) {
+        // The fragments are a ring: a register asks for the step CH further on as soon as the matrix cores have
+        // taken the one it held, and no load sits in a branch (see the kernel above).  Rows of x beyond M read
+        // row 0, the unused rows of a tile or the last tile once more: their columns are never stored.
+        Frag wf[CH], uf[CH], xf[RT][CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            wf[c].u = load_stream16(wp + (size_t)(kt_begin + c) * 512);
+            if (SWIGLU) uf[c].u = load_stream16(up + (size_t)(kt_begin + c) * 512);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                xf[rt][c].u = *reinterpret_cast<const uint4*>(xp[rt] + (size_t)(kt_begin + c) * x_step);
+        }
+        int kt = kt_begin;
+        for (; kt + CH < kt_end; kt += CH) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt], 0, 0, 0);
+                    if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt], 0, 0, 0);
+                }
+                const size_t next = (size_t)(kt + c + CH);
+                wf[c].u = load_stream16(wp + next * 512);
+                if (SWIGLU) uf[c].u = load_stream16(up + next * 512);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) xf[rt][c].u = *reinterpret_cast<const uint4*>(xp[rt] + next * x_step);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt], 0, 0, 0);
+                if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt], 0, 0, 0);
+            }
+    } else
     for (int kt = kt_begin; kt < kt_end; kt += CH) {
+        const uint4 zero = make_uint4(0, 0, 0, 0);
         Frag wf[CH], uf[CH], xf[RT][CH];
 #pragma unroll
         for (int c = 0; c < CH; ++c) {

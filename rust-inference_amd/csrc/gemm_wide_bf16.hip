@@ -51,13 +51,12 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
     const int ntc = live_tile ? nt : 0;
     const bf16_t* wp = wpacked + ((size_t)ntc * k_tiles * 64 + lane) * 8;
     const bf16_t* up = SWIGLU ? wpacked + ((size_t)(row_tiles + ntc) * k_tiles * 64 + lane) * 8 : nullptr;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
     const bool x_tiled = tiled & TILED_X;
     const int jg = lane >> 4;
 
-    // Every load below is issued whatever the indices are, from an address pulled back inside the data, and
-    // what lies outside is replaced by zero afterwards (x) or meets zeros (weights past the stretch's end meet
-    // a slice of x that is zero there).  A load inside a branch would end the pipelining: the compiler cannot
+    // Every load below is issued whatever the indices are: what lies outside x is read from a kilobyte of zeros
+    // instead, and weights past the stretch's end (pulled back to its last tile) meet a slice of x that is zero
+    // there.  A load inside a branch would end the pipelining: the compiler cannot
     // count the loads in flight across a branch that may not have issued one, and waits for all of them.
     // piece j of this thread's share of a slice: (tile of x, step) = q / WD_SLICE, q % WD_SLICE with
     // q = wave + j * W; the 64 lanes of a wavefront copy one fragment (64 x 16 bytes).  Where the fragments do
@@ -72,12 +71,7 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
         const bool ok = row < M && kt < kt_end && kt * 32 + jg * 8 < K;
         const bf16_t* p = x_tiled ? x + (((size_t)rt * k_tiles + ktc) * 64 + lane) * 8
                                   : x + (size_t)min(row, M - 1) * K + min(ktc * 32 + jg * 8, K - 8);
-        uint4 v = *reinterpret_cast<const uint4*>(p);
-        v.x = ok ? v.x : 0u;
-        v.y = ok ? v.y : 0u;
-        v.z = ok ? v.z : 0u;
-        v.w = ok ? v.w : 0u;
-        return v;
+        return *reinterpret_cast<const uint4*>(ok ? p : ri_zero_fragment + lane * 8);
     };
     auto stash = [&](int j, int buf, const uint4& v) {
         const int q = min(wave + j * W, FRAGS - 1);

@@ -39,22 +39,27 @@ SKINNY_MAX_ROWS = 16
 # ones too up to 32 rows (Qwen3-8B sizes at 32 rows, us: q|k|v 16.6 : 16.1, o 10.9 : 13.0, gate|up 40.2 : 51.0
 # + 5 for the activation, down 28.3 : 28.5; 5120 x 25600: 97 : 146; the model's decode step at 24 and 32
 # sequences is 5% and 7% shorter).  From 33 rows on it is not: q|k|v 23.2 : 18.0, and gate|up, level alone
-# with the activation counted (51.8 : 51.8 + 5), made the step at 48 sequences 1% longer.
+# with the activation counted (51.8 : 51.8 + 5), made the step at 48 sequences 1% longer.  (These figures are
+# from before the kernel kept its loads in flight as a ring; with the ring the step at 17, 24 and 32 sequences
+# became 9, 4 and 3% shorter again, and q|k|v on it at 33, 48 and 64 rows still makes the step 2 to 3% longer
+# than the library does.)
 MID_MAX_ROWS = 64
 MID_MAX_BYTES = 20_000_000
 MID_TILED_ROWS = 32
-# 33 to 64 rows against a matrix whose result goes into the residual stream (`o`, `down`): the wide kernel
+# 17 to 64 rows against a matrix whose result goes into the residual stream (`o`, `down`): the wide kernel
 # (ops.gemm_wide_packed_bf16: three or four row tiles a workgroup, the tiles of x shared through LDS) with K cut
 # into stretches that the next norm adds up.  Measured at Qwen3-8B sizes as graphs, in us, against the library
-# and the kernel above: 4096 x 12288 at 64 rows 26.0 : 38.8 : 38.6, at 32 rows 23.0 : 29.0 : 29.2; in the model
-# decode at 64 sequences went from 7,150 to 7,340 tok/s and at 48 from 5,910 to 6,160, and at 24 and 32 it
-# lost 1 to 3% to the kernel above.  4096 x 4096 takes 14 us against the library's 18 inside the model (alone,
-# over a few copies of the matrix that the memory-side cache holds, the library needs 12.5: such small
-# matrices have to be timed in the model), worth 1% of the step at 40 and 48 sequences.  A product whose reader
-# cannot add stretches (q|k|v: 6144 x 4096, with a kernel of its own to add them 22 us against 15 to 18) stays
-# with the library.
+# and the kernel above: 4096 x 12288 at 64 rows 26.0 : 38.8 : 38.6, at 32 rows 23.0 : 29.0 : 29.2.  4096 x 4096
+# takes 14 us against the library's 18 inside the model (alone, over a few copies of the matrix that the
+# memory-side cache holds, the library needs 12.5: such small matrices have to be timed in the model).  In the
+# model, with gate|up on it too (below) and the kernel above for q|k|v up to 32 rows, a decode step of 17, 24,
+# 32, 48 and 64 sequences takes 4.90, 5.31, 5.79, 7.23 and 8.10 ms, where the kernel above alone (to 32 rows)
+# and the library (beyond) took 5.10, 5.50, 5.98, 7.76 and 8.53.  A product whose reader cannot add stretches
+# (q|k|v: 6144 x 4096, with a kernel of its own to add them 22 us against 15 to 18) stays with the kernel above
+# or the library.
 WIDE_MIN_K = 4096
-# The gate|up pair at 33 to 64 rows goes to the wide kernel where workgroups of three or four wavefronts with K
+WIDE_MIN_ROWS = 17
+# The gate|up pair at 17 to 64 rows goes to the wide kernel where workgroups of three or four wavefronts with K
 # whole fill at least this share of the compute units' rounds (12288 pairs of rows: 256 workgroups of three,
 # at 64 rows 45 us against the library's 48 + 5 for the activation, at 48 rows 40 against 50; with groups of
 # four, 192 workgroups, it only drew level).  What bounds it then is what a compute unit can pull through its
@@ -170,7 +175,7 @@ class Runtime:
 
     @staticmethod
     def _wide_gated(pw: PackedWeight) -> bool:
-        """Whether the wide kernel takes a gate|up pair at 33 to 64 rows: where its workgroups (of three or
+        """Whether the wide kernel takes a gate|up pair at 17 to 64 rows: where its workgroups (of three or
         four wavefronts, K whole) fill the compute units evenly; else a quarter of the machine idles and the
         library with its activation kernel is as fast."""
         if pw.packed is None:
@@ -186,7 +191,7 @@ class Runtime:
             return False
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
-        if MID_TILED_ROWS < m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu
+        if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu
                                                    else parts_ok and pw.k >= WIDE_MIN_K):
             return True                                          # the wide kernel (where the reader adds its parts)
         return SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and self._mid_pays(pw, m, True)
@@ -227,14 +232,14 @@ class Runtime:
                 if not mine[1]:
                     return ops.gemv_bf16(ops.as_rows(x), pw.w, out_dtype, swiglu=pw.swiglu)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
-            if (MID_TILED_ROWS < m <= MID_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
+            if (WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
                     and pw.k >= WIDE_MIN_K):
-                # a long K at 33 to 64 rows: K in stretches, every stretch a workgroup that shares the tiles of x
+                # 17 to 64 rows into the residual stream: K in stretches, every stretch a workgroup that shares the tiles of x
                 # through LDS; the stream's next norm adds the stretches' sums
                 x = self.normed_now(x) if later else x
                 waves, parts = _wide_plan(pw.n, pw.k, False)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
-            if MID_TILED_ROWS < m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw):
+            if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw):
                 x = self.normed_now(x) if later else x
                 waves, _ = _wide_plan(pw.n, pw.k, True)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=True, depth=1, waves=waves,
