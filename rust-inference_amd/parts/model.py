@@ -61,8 +61,15 @@ class OutputHead(Part):
             self.weight = embedding.table           # the same device tensor: tying costs no memory
         else:
             self.weight = rt.place_matrix(weights[self.name])
+        # A second copy in the matrix cores' tile order for steps that want 2 to 16 rows of logits (a decode step
+        # of as many sequences): at 151,936 x 4,096 the packed kernel takes 0.21 ms where the library's product
+        # takes 0.26 (1% of such a step), for 1.2 GB more memory.  One row goes to the one-row kernel, more than
+        # 16 to the library, both on the row-major matrix.
+        self.packed = rt.pack(self.weight, always=True)
 
     def forward(self, x):
+        if self.packed.packed is not None and 2 <= x.shape[0] <= 16:
+            return self.rt.linear_packed(x, self.packed, out_dtype=torch.float32)
         return self.rt.linear(x, self.weight, out_dtype=torch.float32)
 
 

@@ -156,11 +156,11 @@ class Runtime:
             return ops.as_rows(x)
         return ops.finish_norm(x)
 
-    def pack(self, w: torch.Tensor, swiglu: bool = False) -> PackedWeight:
+    def pack(self, w: torch.Tensor, swiglu: bool = False, always: bool = False) -> PackedWeight:
         """A placed weight, with a packed copy where the packed kernel is the faster one for 2 to 16
-        rows (bfloat16 compute only)."""
+        rows (bfloat16 compute only), or wherever it can be used when the caller says ``always``."""
         n, k = w.shape
-        pays = swiglu or _packed_pays(n, k)
+        pays = always or swiglu or _packed_pays(n, k)
         if self.dtype != torch.bfloat16 or k % 8 or not pays:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)

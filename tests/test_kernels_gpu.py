@@ -83,6 +83,24 @@ def test_add_rmsnorm_adds_the_parts_of_a_split_product(ops):
     close(ops.add_rmsnorm(res2, p2, g2, 1e-6, torch.float32, rows), want, 2e-6, "gathered rows over parts")
 
 
+@pytest.mark.parametrize("n_parts", [2, 4, 5, 8, 9])
+@pytest.mark.parametrize("dim", [72, 1000, 4096, 5120])
+def test_the_norm_adds_any_number_of_parts_in_their_order(ops, n_parts, dim):
+    """The parts are fetched four at a time; the sum is residual + part 0 + part 1 + ... in float32, bit for bit,
+    whatever their number, and a row shorter than the threads' reach is not read beyond its end."""
+    rng = np.random.default_rng(n_parts * dim)
+    res = t(rng.normal(size=(5, dim)))
+    parts = t(rng.normal(size=(n_parts, 5, dim)))
+    gain = t(1 + 0.1 * rng.normal(size=dim))
+    want_sum = res.clone()
+    for q in range(n_parts):
+        want_sum += parts[q]
+    got = res.clone()
+    out = ops.add_rmsnorm(got, parts, gain, 1e-6, torch.float32)
+    assert torch.equal(got, want_sum)
+    close(out, P.rms_norm(f64(want_sum), f64(gain), 1e-6), 2e-6, "norm over parts")
+
+
 @pytest.mark.parametrize("pending_dtype", [torch.float32, torch.bfloat16])
 def test_add_rows_in_place_and_bias(ops, pending_dtype):
     rng = np.random.default_rng(12)
