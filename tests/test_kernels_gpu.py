@@ -711,6 +711,46 @@ def test_every_maker_of_rows_can_tile_them(ops, m, dim, n):
         ops.add_rmsnorm(t(rng.normal(size=(65, dim))), None, gain, 1e-5, torch.bfloat16, tiled=True)
 
 
+def test_streaming_attention_walks_a_run_of_more_pages_than_it_holds_table_entries_for(ops):
+    """A wavefront of the streaming kernel fetches the page table's entries for 256 of its pages at a time; a run
+    of more than 1,024 pages (32,768 keys) goes round that loop again.  64 sequences of one kv head each side of
+    that length, eight kv heads (512 runs: one a sequence and kv head), against the generic kernel on the same
+    pages; the sequences are of unequal length and one key far back in one of them gets a score that stands out."""
+    heads, kv_heads, dh, B = 8, 8, 32, 64
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    lens = [33_000 + 37 * b for b in range(B)]
+    lens[5] = 40_000
+    pages_per = [-(-n // 32) for n in lens]
+    width = max(pages_per)
+    num_pages = sum(pages_per)
+    assert ops.decode_attention_runs(B, kv_heads, max(lens)) == 1
+    kp = torch.randn((num_pages, kv_heads, 32, dh), device="cuda", generator=gen).to(torch.bfloat16)
+    vp = torch.randn((num_pages, kv_heads, dh, 32), device="cuda", generator=gen).to(torch.bfloat16)
+    order = torch.randperm(num_pages, device="cuda", generator=gen).to(torch.int32)
+    table = torch.zeros((B, width), dtype=torch.int32, device="cuda")
+    at = 0
+    for b, n in enumerate(pages_per):
+        table[b, :n] = order[at:at + n]
+        at += n
+    qkv = torch.randn((B, (heads + 2 * kv_heads) * dh), device="cuda", generator=gen).to(torch.bfloat16)
+    # Queries that are a multiple of one far key, so that the output is that key's value: a key among a
+    # wavefront's first 256 pages (position 9,000 of sequence 5) and keys among its later ones (pages from 1,024
+    # on: position 39,990 of sequence 5, a key of sequence 9's last pages and one of sequence 20's page 1,024)
+    for b, far, head in ((5, 9_000, 2), (5, 39_990, 3), (9, lens[9] - 100, 1), (20, 32_768 + 10, 4)):
+        key = kp[table[b, far // 32].item(), head, far % 32].float()
+        qkv[b, head * dh:(head + 1) * dh] = (6.0 * key / key.norm() * dh ** 0.25).to(torch.bfloat16)
+    pos = t([n - 1 for n in lens], torch.int32)
+    cu = t(np.arange(B + 1), torch.int32)
+    seq = t(np.arange(B), torch.int32)
+    got = ops.attention_decode_bf16(qkv, kp, vp, cu, pos, table, B, max(lens), heads, kv_heads, dh, None, dh ** -0.5)
+    want = ops.attention(qkv, kp, vp, pos, seq, table, heads, kv_heads, dh, None, dh ** -0.5)
+    close(got, f64(want), 1e-2, "a run of more than 1,024 pages")
+    for b, head in ((5, 2), (5, 3), (9, 1), (20, 4)):       # and these rows are not drowned by the others' size
+        row = slice(head * dh, (head + 1) * dh)
+        assert want[b, row].float().abs().max() > 0.5
+        close(got[b, row], f64(want[b, row]), 1e-2, f"sequence {b}, head {head}")
+
+
 @pytest.mark.parametrize("fused", [False, True])
 def test_decode_attention_writes_tiled_rows(ops, fused):
     rng = np.random.default_rng(77)
