@@ -34,11 +34,20 @@ __device__ __forceinline__ float silu_sk(float z) { return z / (1.0f + expf(-z))
 #define SK_ROWS (16 / SK_WAVES)   // rows of x whose sums of squares one wavefront adds up
 #define SK_PRE 4                  // partial sums of squares a lane fetches ahead of the weights
 
-template <int SK_WAVES, bool SWIGLU, typename TO>
+// A wavefront's sum over its share of K is kept in two halves, the steps of the same parity as its first one
+// and the others, each added up in order and the two added at the end.  That makes two chains of matrix
+// instructions that do not wait for one another, and it is the order in which PAIRED gets its sums:
+// PAIRED (up to 8 rows of x, the ring's conditions): a lane's piece of x is a row's 8 elements of one step for
+// lanes 0-7 of every 16 and of the next step for lanes 8-15, so one load of x serves two steps of K (the rows
+// of x that a workgroup pulls from the L2 cache count against what its compute unit can pull like the weights
+// do).  The fragment goes through the matrix cores with either step's weights: columns 0-7 of the first
+// product and columns 8-15 of the second are the rows' sums over the even and over the odd steps, the other
+// columns pair one step's weights with the other step's x and are dropped.  The same bits as without.
+template <int SK_WAVES, bool SWIGLU, typename TO, bool PAIRED>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked,
                           int M, int N, int K, int k_tiles, int tiles_per_wave, int up_tile_offset, NormLink link, int tiled) {
-    __shared__ float red[SWIGLU ? 2 : 1][SK_WAVES][4][64];
+    __shared__ float red[SWIGLU ? 2 : 1][PAIRED ? 2 : 1][SK_WAVES][4][64];
     __shared__ float inv_lds[16];
     __shared__ float sq_lds[16][17];
     const int lane = threadIdx.x & 63;
@@ -95,8 +104,55 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
         gain_pre = gp[have ? n : 0];
     }
 
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
-    if (ring) {
+    floatx4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, accu[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if (PAIRED) {
+        // (the host launches this form only where the ring's conditions hold)
+        constexpr int PC = SK_CHUNK / 2;                     // pairs of steps in flight: as many weights as the ring below
+        const int sub = i >> 3;                              // which step of a pair this lane's piece of x belongs to
+        const bf16_t* xq = x_tiled ? x + (size_t)(jg * 16 + (i & 7)) * 8 + (size_t)sub * 512
+                                   : x + (size_t)((i & 7) < M ? (i & 7) : 0) * K + jg * 8 + sub * 32;
+        Frag wa[PC], wb[PC], ua[PC], ub[PC], xf[PC];
+#pragma unroll
+        for (int c = 0; c < PC; ++c) {
+            const size_t at = (size_t)(kt_begin + 2 * c);
+            wa[c].u = load_stream16(wp + at * 512);
+            wb[c].u = load_stream16(wp + (at + 1) * 512);
+            if (SWIGLU) {
+                ua[c].u = load_stream16(up + at * 512);
+                ub[c].u = load_stream16(up + (at + 1) * 512);
+            }
+            xf[c].u = *reinterpret_cast<const uint4*>(xq + at * x_step);
+        }
+        int kt = kt_begin;
+        for (; kt + SK_CHUNK < kt_end; kt += SK_CHUNK) {
+#pragma unroll
+            for (int c = 0; c < PC; ++c) {
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[c].v, xf[c].v, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[c].v, xf[c].v, acc[1], 0, 0, 0);
+                if (SWIGLU) {
+                    accu[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ua[c].v, xf[c].v, accu[0], 0, 0, 0);
+                    accu[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ub[c].v, xf[c].v, accu[1], 0, 0, 0);
+                }
+                const size_t next = (size_t)(kt + 2 * c + SK_CHUNK);
+                wa[c].u = load_stream16(wp + next * 512);
+                wb[c].u = load_stream16(wp + (next + 1) * 512);
+                if (SWIGLU) {
+                    ua[c].u = load_stream16(up + next * 512);
+                    ub[c].u = load_stream16(up + (next + 1) * 512);
+                }
+                xf[c].u = *reinterpret_cast<const uint4*>(xq + next * x_step);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < PC; ++c) {
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[c].v, xf[c].v, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[c].v, xf[c].v, acc[1], 0, 0, 0);
+            if (SWIGLU) {
+                accu[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ua[c].v, xf[c].v, accu[0], 0, 0, 0);
+                accu[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ub[c].v, xf[c].v, accu[1], 0, 0, 0);
+            }
+        }
+    } else if (ring) {
         // Every wavefront's share is a whole number of rounds of SK_CHUNK steps and K a multiple of 32: the
         // fragments are a ring, and a register asks for the step SK_CHUNK further on as soon as the matrix
         // cores have taken the one it held, so that SK_CHUNK steps' loads stay in flight all the way instead
@@ -115,8 +171,8 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
         for (; kt + SK_CHUNK < kt_end; kt += SK_CHUNK) {
 #pragma unroll
             for (int c = 0; c < SK_CHUNK; ++c) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
-                if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
+                acc[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc[c & 1], 0, 0, 0);
+                if (SWIGLU) accu[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu[c & 1], 0, 0, 0);
                 const size_t next = (size_t)(kt + c + SK_CHUNK);
                 wf[c].u = load_stream16(wp + next * 512);
                 if (SWIGLU) uf[c].u = load_stream16(up + next * 512);
@@ -125,8 +181,8 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
         }
 #pragma unroll
         for (int c = 0; c < SK_CHUNK; ++c) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
-            if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
+            acc[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc[c & 1], 0, 0, 0);
+            if (SWIGLU) accu[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu[c & 1], 0, 0, 0);
         }
     } else
     for (int kt = kt_begin; kt < kt_end; kt += SK_CHUNK) {
@@ -141,15 +197,25 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
                           ? *reinterpret_cast<const uint4*>(xp + (size_t)(kt + c) * x_step) : zero;
         }
 #pragma unroll
-        for (int c = 0; c < SK_CHUNK; ++c) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc, 0, 0, 0);
-            if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu, 0, 0, 0);
+        for (int c = 0; c < SK_CHUNK; ++c) {               // SK_CHUNK is even: c's parity is the step's, counted from kt_begin
+            acc[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc[c & 1], 0, 0, 0);
+            if (SWIGLU) accu[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu[c & 1], 0, 0, 0);
         }
     }
+    if (PAIRED) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        red[0][wave][e][lane] = acc[e];
-        if (SWIGLU) red[1][wave][e][lane] = accu[e];
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                red[0][PAIRED ? h : 0][wave][e][lane] = acc[h][e];
+                if (SWIGLU) red[SWIGLU ? 1 : 0][PAIRED ? h : 0][wave][e][lane] = accu[h][e];
+            }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            red[0][0][wave][e][lane] = acc[0][e] + acc[1][e];
+            if (SWIGLU) red[SWIGLU ? 1 : 0][0][wave][e][lane] = accu[0][e] + accu[1][e];
+        }
     }
     // rows of x that still want their 1 / rms: the lanes' shares in the order of wave_sum, the same in every
     // workgroup
@@ -172,8 +238,9 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
         float g = 0.f, u = 0.f;
 #pragma unroll
         for (int wv = 0; wv < SK_WAVES; ++wv) {
-            g += red[0][wv][r][ln];
-            if (SWIGLU) u += red[1][wv][r][ln];
+            // PAIRED: column m of the even steps' product plus column m + 8 of the odd steps' (m < 8 is all that is stored)
+            g += PAIRED ? red[0][0][wv][r][ln] + red[0][PAIRED ? 1 : 0][wv][r][(ln + 8) & 63] : red[0][0][wv][r][ln];
+            if (SWIGLU) u += PAIRED ? red[SWIGLU ? 1 : 0][0][wv][r][ln] + red[SWIGLU ? 1 : 0][PAIRED ? 1 : 0][wv][r][(ln + 8) & 63] : red[SWIGLU ? 1 : 0][0][wv][r][ln];
         }
         if (link.ssq_in && m < M) {
             g *= inv_lds[m];
@@ -221,12 +288,18 @@ static void launch_packed(void* out, int out_dtype, const bf16_t* x, const bf16_
     const int part_tiles = (k_tiles + parts - 1) / parts;
     const int tiles_per_wave = (part_tiles + WAVES - 1) / WAVES;
     dim3 grid(row_tiles, parts);
-    if (out_dtype == RI_F32)
-        gemm_skinny_packed_kernel<WAVES, SWIGLU, float><<<grid, WAVES * 64, 0, s>>>(
-            (float*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link, tiled);
-    else
-        gemm_skinny_packed_kernel<WAVES, SWIGLU, bf16_t><<<grid, WAVES * 64, 0, s>>>(
-            (bf16_t*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link, tiled);
+    // the ring's conditions (the kernel works them out the same way) and at most 8 rows: two steps to a load of x
+    const bool paired = m <= 8 && k % 32 == 0 && tiles_per_wave % SK_CHUNK == 0 && part_tiles == tiles_per_wave * WAVES &&
+                        k_tiles % part_tiles == 0;
+#define RI_SKINNY_GO(TO, PAIRED)                                                        \
+    gemm_skinny_packed_kernel<WAVES, SWIGLU, TO, PAIRED><<<grid, WAVES * 64, 0, s>>>(   \
+        (TO*)out, x, w, m, n, k, k_tiles, tiles_per_wave, row_tiles, link, tiled)
+    if (out_dtype == RI_F32) {
+        if (paired) RI_SKINNY_GO(float, true); else RI_SKINNY_GO(float, false);
+    } else {
+        if (paired) RI_SKINNY_GO(bf16_t, true); else RI_SKINNY_GO(bf16_t, false);
+    }
+#undef RI_SKINNY_GO
 }
 
 static int packed_run(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k, int swiglu,
@@ -311,9 +384,11 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
                                    : x + (size_t)(x_ok[rt] ? rt * 16 + i : 0) * K + jg * 8;
     }
     const int x_step = (tiled & TILED_X) ? 512 : 32;         // elements from one step's fragment to the next
-    floatx4 acc[RT], accu[RT];
+    // two halves of every sum, by the parity of the step counted from the wavefront's first, added at the end:
+    // the order of the kernel above, so that a row's bits are the same from either
+    floatx4 acc[RT][2], accu[RT][2];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt] = accu[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = acc[rt][1] = accu[rt][0] = accu[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
     // the same in every wavefront of the launch: K in whole steps, every wavefront's share whole rounds of CH
     const bool ring = K % 32 == 0 && tiles_per_wave % CH == 0 && k_tiles == tiles_per_wave * SK_WAVES;
     if (ring) {
@@ -335,8 +410,8 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
             for (int c = 0; c < CH; ++c) {
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt], 0, 0, 0);
-                    if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt], 0, 0, 0);
+                    acc[rt][c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt][c & 1], 0, 0, 0);
+                    if (SWIGLU) accu[rt][c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt][c & 1], 0, 0, 0);
                 }
                 const size_t next = (size_t)(kt + c + CH);
                 wf[c].u = load_stream16(wp + next * 512);
@@ -349,8 +424,8 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
         for (int c = 0; c < CH; ++c)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt], 0, 0, 0);
-                if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt], 0, 0, 0);
+                acc[rt][c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt][c & 1], 0, 0, 0);
+                if (SWIGLU) accu[rt][c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt][c & 1], 0, 0, 0);
             }
     } else
     for (int kt = kt_begin; kt < kt_end; kt += CH) {
@@ -370,16 +445,16 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
         for (int c = 0; c < CH; ++c)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt], 0, 0, 0);
-                if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt], 0, 0, 0);
+                acc[rt][c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[rt][c].v, acc[rt][c & 1], 0, 0, 0);
+                if (SWIGLU) accu[rt][c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[rt][c].v, accu[rt][c & 1], 0, 0, 0);
             }
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            red[0][wave][rt * 4 + e][lane] = acc[rt][e];
-            if (SWIGLU) red[1][wave][rt * 4 + e][lane] = accu[rt][e];
+            red[0][wave][rt * 4 + e][lane] = acc[rt][0][e] + acc[rt][1][e];
+            if (SWIGLU) red[1][wave][rt * 4 + e][lane] = accu[rt][0][e] + accu[rt][1][e];
         }
     __syncthreads();
     // D[row n, column m] of a tile: lane ln of register r holds n = 4 * (ln / 16) + r, m = ln % 16
