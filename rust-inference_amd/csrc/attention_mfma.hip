@@ -20,15 +20,17 @@
 // second product rounded to bfloat16, the running sum is taken of them before the rounding.  (Letting
 // the reference point of the exponents lag behind the running maximum, so that the accumulators are
 // rescaled only rarely, was tried and changed no timing: the rescaling is not what the kernel waits for.)
-// (Also tried with two tiles a wavefront: all scores first, then one tile's value product interleaved with
-// the other tile's exponentials by scheduling hints.  The instructions came out in that order and the
-// kernel gained 1%: the two wavefronts of a SIMD already fill each other's gaps.)
 //
 // Prefill: one wavefront per tile of tokens, walking the sequence's pages in order; the four
-// wavefronts of a workgroup share the pages through LDS.  Decode (one new
+// wavefronts of a workgroup share the pages through LDS.  The walk is one page ahead with the scores: the
+// matrix cores take the next page's scores while the vector unit turns this page's into weights, and this
+// page's value product while it finds the next page's maxima (3 to 6% over one page at a time at 2,048 to
+// 32,768 tokens; the same bits).  Decode (one new
 // token per sequence): the keys are cut into chunks of 256 at fixed places, one workgroup per chunk
 // (its eight wavefronts take one page each), partial results go to a workspace and a second kernel
 // joins them in chunk order.  Neither order depends on the batch or on how tokens were cut.
+#include <type_traits>
+
 #include "api.h"
 #include "common.h"
 
@@ -206,6 +208,86 @@ __device__ __forceinline__ void init_columns(Columns<DH, NT>& c) {
     }
 }
 
+// The same work in four pieces, for a loop that takes the scores of the next page while it weighs this one
+// (the prefill's): the results are those of scores_and_weights and weighted_values bit for bit.
+template <int DH, int NT>
+__device__ __forceinline__ void scores_of(const Columns<DH, NT>& c, const Frag (&kf)[2][DH / 32], float (&s)[NT][8]) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < DH / 32; ++ks) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][ks].v, c.q[j][ks].v, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][ks].v, c.q[j][ks].v, s1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            s[j][e] = s0[e];
+            s[j][4 + e] = s1[e];
+        }
+    }
+}
+
+template <int DH, int NT>
+__device__ __forceinline__ void mask_scores(const Columns<DH, NT>& c, float (&s)[NT][8], int page, int lane) {
+    const int key0 = page * PAGE + (lane >> 4) * 8;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int key = key0 + e;
+            if (key > c.qpos[j] || key < c.lo[j]) s[j][e] = -INFINITY;
+        }
+}
+
+// The columns' running maxima with a page's scores taken in (c.m itself stays as it is).
+template <int DH, int NT>
+__device__ __forceinline__ void maxima_with(const Columns<DH, NT>& c, const float (&s)[NT][8], float (&m_new)[NT],
+                                            float scale_log2) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        float mx = fmaxf(fmaxf(fmaxf(s[j][0], s[j][1]), fmaxf(s[j][2], s[j][3])),
+                         fmaxf(fmaxf(s[j][4], s[j][5]), fmaxf(s[j][6], s[j][7])));
+        mx = column_max<(NT >= 2 || DH < 128)>(mx);
+        m_new[j] = fmaxf(c.m[j], mx * scale_log2);
+    }
+}
+
+// Moves the reference point of the exponents to the new maxima (sums and accumulators are rescaled where a
+// maximum rose anywhere in the wavefront) and returns in ref what the next weights subtract.
+template <int DH, int NT>
+__device__ __forceinline__ void move_reference(Columns<DH, NT>& c, const float (&m_new)[NT], float (&ref)[NT]) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        ref[j] = m_new[j] == -INFINITY ? 0.f : m_new[j];           // a column that has seen no key yet
+        if (__any(m_new[j] != c.m[j])) {
+            const float corr = __builtin_amdgcn_exp2f(c.m[j] - ref[j]);      // 0 while m is -inf
+            c.l[j] *= corr;
+#pragma unroll
+            for (int dt = 0; dt < DH / 16; ++dt) c.o[j][dt] *= corr;
+            c.m[j] = m_new[j];
+        }
+    }
+}
+
+// A page's weights from its scores and the reference point that already holds its maximum.
+template <int DH, int NT>
+__device__ __forceinline__ void weights_of(Columns<DH, NT>& c, const float (&s)[NT][8], const float (&ref)[NT],
+                                           Frag (&p)[NT], float scale_log2) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        float ps[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float a = __builtin_amdgcn_exp2f(fmaf(s[j][2 * e], scale_log2, -ref[j]));
+            const float b = __builtin_amdgcn_exp2f(fmaf(s[j][2 * e + 1], scale_log2, -ref[j]));
+            p[j].w[e] = pack_bf16x2(a, b);
+            ps[e] = a + b;
+        }
+        c.l[j] += (ps[0] + ps[1]) + (ps[2] + ps[3]);
+    }
+}
+
 // ------------------------------------------------------------------ prefill
 // A workgroup of four wavefronts takes 4 * (16 NT / group) consecutive tokens of one sequence and one kv
 // head.  The pages of keys and values go through LDS, fetched once for all four wavefronts and
@@ -225,11 +307,15 @@ struct LdsPage {
 };
 
 template <int DH>
-__device__ __forceinline__ void stage_store_one(bf16_t* k_lds, bf16_t* v_lds, int c, const uint4& k, const uint4& v) {
+__device__ __forceinline__ void stage_store_key(bf16_t* k_lds, int c, const uint4& k) {
     const int krow = c / (DH / 8), kcol = c % (DH / 8);                  // key row 0..31, 16-byte column
     const int w = krow & 7;
     const int lrow = (w >= 4 ? 16 : 0) + (krow >> 3) * 4 + (w & 3);
     *reinterpret_cast<uint4*>(k_lds + lrow * LdsPage<DH>::KS + kcol * 8) = k;
+}
+
+template <int DH>
+__device__ __forceinline__ void stage_store_value(bf16_t* v_lds, int c, const uint4& v) {
     const int vrow = c / 4, vcol = c % 4;                                // channel 0..DH-1, 16-byte column
     *reinterpret_cast<uint4*>(v_lds + vrow * LdsPage<DH>::VS + vcol * 8) = v;
 }
@@ -291,12 +377,10 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
             for (int ks = 0; ks < DH / 32; ++ks) c.q[j][ks].u = *reinterpret_cast<const uint4*>(qp + ks * 32);
         }
     }
-    // pages the workgroup walks, and the part of them this wavefront's tokens can see
+    // pages the workgroup walks (every wavefront takes them all)
     const int wg_first = tok_pos[t_wg], wg_last = tok_pos[min(t_end, t_wg + 4 * tile_tokens) - 1];
     const int p_lo = window > 0 ? max(0, wg_first - window + 1) / PAGE : 0;
     const int p_hi = wg_last / PAGE;
-    const int my_hi = nt > 0 ? tok_pos[t0 + nt - 1] / PAGE : -1;
-    const int my_lo = (nt > 0 && window > 0) ? max(0, tok_pos[t0] - window + 1) / PAGE : 0;
     // a page is open to the whole wavefront when its last key is at or before the first token's position
     // and its first key inside the last token's window; wavefronts with unused columns mask always
     const bool full = nt * group == 16 * NT;
@@ -311,48 +395,91 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
     const int c0 = threadIdx.x;
     const bool has0 = c0 < LdsPage<DH>::CHUNKS;
     uint4 sk0 = make_uint4(0, 0, 0, 0), sk1 = sk0, sv0 = sk0, sv1 = sk0;
-#define RI_STAGE_LOAD(PHYS)                                                                          \
+#define RI_STAGE_LOAD(PAGES, R0, R1, PHYS)                                                           \
     {                                                                                                \
         const long base_ = ((long)(PHYS) * kv_heads + kvh) * (long)(PAGE * DH);                      \
-        if (has0) {                                                                                  \
-            sk0 = *reinterpret_cast<const uint4*>(k_pages + base_ + c0 * 8);                         \
-            sv0 = *reinterpret_cast<const uint4*>(v_pages + base_ + c0 * 8);                         \
-        }                                                                                            \
-        if (TWO) {                                                                                   \
-            sk1 = *reinterpret_cast<const uint4*>(k_pages + base_ + (c0 + 256) * 8);                 \
-            sv1 = *reinterpret_cast<const uint4*>(v_pages + base_ + (c0 + 256) * 8);                 \
-        }                                                                                            \
+        if (has0) R0 = *reinterpret_cast<const uint4*>(PAGES + base_ + c0 * 8);                      \
+        if (TWO) R1 = *reinterpret_cast<const uint4*>(PAGES + base_ + (c0 + 256) * 8);               \
     }
-#define RI_STAGE_STORE(BUF)                                                                          \
+    // The loop is one page ahead with the scores: a turn takes the scores of page p + 1 while it turns the
+    // scores of page p into weights (the matrix cores work on the one while the vector unit works on the
+    // other), then the value product of page p while it finds the maxima of page p + 1.  Keys are staged
+    // two pages ahead and values one; in turn i the keys read lie in buffer i % 2 and the values in the other,
+    // and the pages that arrive are written to the buffers that are not read, so one barrier a turn is enough.
+    // Every wavefront takes every page of the workgroup (those outside its own tokens' sight are masked
+    // whole and add nothing), and the page numbers of the loads are clamped: no branch in a turn but the mask
+    // and the move of the reference point, so that each half of a turn is one stretch of code to schedule.
+#define RI_TURN_LOADS(P)                                                                             \
+    RI_STAGE_LOAD(k_pages, sk0, sk1, table[min((P) + 2, p_hi)]);                                     \
+    RI_STAGE_LOAD(v_pages, sv0, sv1, table[min((P) + 1, p_hi)]);
+#define RI_TURN_STORES(I)                                                                            \
     {                                                                                                \
-        if (has0) stage_store_one<DH>(k_lds[BUF], v_lds[BUF], c0, sk0, sv0);                         \
-        if (TWO) stage_store_one<DH>(k_lds[BUF], v_lds[BUF], c0 + 256, sk1, sv1);                    \
+        if (has0) stage_store_key<DH>(k_lds[((I) & 1) ^ 1], c0, sk0);                                \
+        if (TWO) stage_store_key<DH>(k_lds[((I) & 1) ^ 1], c0 + 256, sk1);                           \
+        if (has0) stage_store_value<DH>(v_lds[(I) & 1], c0, sv0);                                    \
+        if (TWO) stage_store_value<DH>(v_lds[(I) & 1], c0 + 256, sv1);                               \
+        __syncthreads();                /* what arrived is in place; what was read may be overwritten */ \
     }
-    RI_STAGE_LOAD(table[p_lo]);
-    RI_STAGE_STORE(0);
+#define RI_PAGE_OPEN(Q) ((Q) * PAGE + PAGE - 1 <= min_qpos && (Q) * PAGE >= max_lo)
+    RI_STAGE_LOAD(k_pages, sk0, sk1, table[p_lo]);
+    {
+        if (has0) stage_store_key<DH>(k_lds[0], c0, sk0);
+        if (TWO) stage_store_key<DH>(k_lds[0], c0 + 256, sk1);
+    }
     __syncthreads();
-    for (int p = p_lo; p <= p_hi; ++p) {
-        const int buf = (p - p_lo) & 1;
-        if (p < p_hi) RI_STAGE_LOAD(table[p + 1]);
-        if (p >= my_lo && p <= my_hi) {
-            const bool open = p * PAGE + PAGE - 1 <= min_qpos && p * PAGE >= max_lo;
-            Frag w[NT];
-            {
-                Frag kf[2][DH / 32];
-                key_frags_from_lds<DH>(kf, k_lds[buf], lane);
-                scores_and_weights<DH, NT>(c, kf, w, p, lane, scale_log2, open);
-            }
-            {
-                Frag vf[DH / 16];
-                value_frags_from_lds<DH>(vf, v_lds[buf], lane);
-                weighted_values<DH, NT>(c, vf, w);
-            }
-        }
-        if (p < p_hi) RI_STAGE_STORE(buf ^ 1);
-        __syncthreads();                                     // the next page is in place; this one may be overwritten
+    float s_cur[NT][8], ref[NT], m_new[NT];
+    {                                                        // turn 0: the first page's scores and maxima
+        RI_TURN_LOADS(p_lo - 1);
+        Frag kf[2][DH / 32];
+        key_frags_from_lds<DH>(kf, k_lds[0], lane);
+        scores_of<DH, NT>(c, kf, s_cur);
+        if (!RI_PAGE_OPEN(p_lo)) mask_scores<DH, NT>(c, s_cur, p_lo, lane);
+        maxima_with<DH, NT>(c, s_cur, m_new, scale_log2);
+        move_reference<DH, NT>(c, m_new, ref);
+        RI_TURN_STORES(0);
     }
+    // A turn with the next page open to every column of the wavefront has no mask in it; pages are open in
+    // one stretch (behind the window's edge, before the diagonal), so the turns come as three loops.
+    auto turn = [&](int p, auto masked) {
+        const int i = p - p_lo + 1;
+        RI_TURN_LOADS(p);
+        Frag w[NT];
+        float s_next[NT][8];
+        {
+            Frag kf[2][DH / 32];
+            key_frags_from_lds<DH>(kf, k_lds[i & 1], lane);
+            scores_of<DH, NT>(c, kf, s_next);
+            weights_of<DH, NT>(c, s_cur, ref, w, scale_log2);
+        }
+        if (decltype(masked)::value) mask_scores<DH, NT>(c, s_next, p + 1, lane);
+        {
+            Frag vf[DH / 16];
+            value_frags_from_lds<DH>(vf, v_lds[(i & 1) ^ 1], lane);
+            weighted_values<DH, NT>(c, vf, w);
+            maxima_with<DH, NT>(c, s_next, m_new, scale_log2);
+        }
+        move_reference<DH, NT>(c, m_new, ref);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s_cur[j][e] = s_next[j][e];
+        RI_TURN_STORES(i);
+    };
+    int p = p_lo;
+    for (; p < p_hi && !RI_PAGE_OPEN(p + 1); ++p) turn(p, std::true_type());
+    for (; p < p_hi && RI_PAGE_OPEN(p + 1); ++p) turn(p, std::false_type());
+    for (; p < p_hi; ++p) turn(p, std::true_type());
+    {                                                        // the last page's weights and value product
+        const int i = p_hi - p_lo + 1;
+        Frag w[NT], vf[DH / 16];
+        weights_of<DH, NT>(c, s_cur, ref, w, scale_log2);
+        value_frags_from_lds<DH>(vf, v_lds[(i & 1) ^ 1], lane);
+        weighted_values<DH, NT>(c, vf, w);
+    }
+#undef RI_TURN_LOADS
+#undef RI_TURN_STORES
+#undef RI_PAGE_OPEN
 #undef RI_STAGE_LOAD
-#undef RI_STAGE_STORE
     finish_columns<DH, NT>(c);
 
 #pragma unroll
@@ -980,12 +1107,16 @@ static int check_common(const char* name, int heads, int kv_heads, int head_dim,
 // prompt of a few thousand tokens: at 32 query and 8 kv heads of 128, 2,048 tokens take 81 us with 1,024
 // workgroups of half the columns against 95 us with 512; from 4,096 tokens on the full tiles win).  A
 // column's arithmetic does not depend on the tile it sits in, only the grid does.
+// Tiles are halved while the launch has fewer workgroups than this: three for each of the 256 compute units
+// (a prompt of 3,072 tokens at Qwen3-8B sizes: 105 us with two tiles a wavefront in 768 workgroups, 126 us with
+// one tile in 1,536; at 2,048 tokens one tile in 1,024 workgroups takes 57 us, two in 512 take 67).
+#define PREFILL_MIN_WGS 768
 static int prefill_tiles(int head_dim, int group, int max_new, int seqs, int kv_heads) {
     int nt = head_dim <= 64 ? 4 : 2;
     while (nt > 1 && group <= 16 * (nt / 2)) {
         const int tile_tokens = (16 * nt) / group;
         const long wgs = (long)((max_new + 4 * tile_tokens - 1) / (4 * tile_tokens)) * seqs * kv_heads;
-        if (wgs >= 1024) break;
+        if (wgs >= PREFILL_MIN_WGS) break;
         nt /= 2;
     }
     return nt;
