@@ -18,7 +18,8 @@ def _wide_plan(n: int, k: int, swiglu: bool) -> tuple[int, int]:
 # Which product kernel runs, by the number of rows of x (measured on MI355X at Qwen3-8B sizes with the
 # weights streamed from HBM through non-temporal loads, every variant replayed as a graph):
 #   1 row      one wavefront per weight row (gemv_bf16): 5.6 to 5.7 TB/s on the large matrices, 7.0 on the
-#              output head.  (At two rows the packed kernel is ahead: 471 against 438 tok/s for the model.)
+#              output head.  (At two rows the packed kernel is ahead: 471 against 438 tok/s for the model;
+#              at one row it is behind, a decode step of 3.19 ms against 3.12.)
 #   2-16 rows  the matrix-core kernel on weights packed into MFMA tiles ahead of time, where a part asked for
 #              the packed copy; it hands its rows to the next packed product in the operand's order
 #              (ops.TiledRows) and does the norms around it.  Where there is no packed copy the vendor
