@@ -124,21 +124,47 @@ def main() -> int:
     prefill_s = min(times[1:])
     del engine
 
-    # ---- decoding
+    # ---- decoding: the generation loop's steady state (engine/generate.py).  A step is launched with the ids
+    # the step before picked, still on the device, and the host reads every step's ids while the next step runs;
+    # where there is no captured graph for the step yet (or --no-graphs) the host reads them first.
     def decode_run(batch, steps, warmup):
         engine = fresh_engine(batch)
         slots = [engine.cache.acquire() for _ in range(batch)]
         logits = engine.step([StepEntry(s, q, "last") for s, q in zip(slots, prompts(batch, args.prompt))])
-        nxt = ops.argmax(logits).tolist()
-        for _ in range(warmup):
-            nxt = ops.argmax(engine.step([StepEntry(s, [t], "last") for s, t in zip(slots, nxt)])).tolist()
+        ids = ops.argmax(logits)
+        pinned = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+
+        def one_step(ids):
+            out = engine.decode_on_device(slots, ids)
+            if out is None:
+                out = engine.step([StepEntry(s, [t], "last") for s, t in zip(slots, ids.tolist())])
+            return ops.argmax(out)
+
+        def run(n):
+            nonlocal ids
+            unread, read = None, 0
+            for i in range(n):
+                ids = one_step(ids)
+                if unread is not None:
+                    unread[0].synchronize()
+                    read += len(unread[1].tolist())
+                pinned[i & 1].copy_(ids, non_blocking=True)
+                ev = torch.cuda.Event()
+                ev.record()
+                unread = (ev, pinned[i & 1])
+            if unread is not None:
+                unread[0].synchronize()
+                read += len(unread[1].tolist())
+            return read
+
+        run(warmup)
         sync()
         first_context = sum(engine.cache.length(s) for s in slots) / batch + 1
         t0 = time.perf_counter()
-        for _ in range(steps):
-            nxt = ops.argmax(engine.step([StepEntry(s, [t], "last") for s, t in zip(slots, nxt)])).tolist()
+        read = run(steps)
         sync()
         dt = time.perf_counter() - t0
+        assert read == batch * steps
         mean_context = first_context + (steps - 1) / 2.0
         for s in slots:
             engine.cache.release(s)

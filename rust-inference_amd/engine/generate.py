@@ -10,6 +10,13 @@ Per sequence the loop is the reference's (src/bin/runner.rs:287-313): the first
 token comes from the prompt's logits and counts toward ``max_new_tokens``; a stop
 token is tested before it is put out, is not part of the output and is never fed
 back; the last token allowed is put out but not fed.
+
+Where the engine can take a step's tokens from the device (``decode_on_device``: captured graphs) and no
+repetition penalty needs them on the host first, the loop runs one step ahead of what it has read: it
+launches step n + 1 with the ids step n picked, still on the device, and reads step n's ids while step n + 1
+runs, so that the host's share of a step (the rules below, the step's layout, the launch) hides behind the
+GPU's.  A sequence whose token then turns out to be a stop token has been carried through one step too many:
+that step's result for it is dropped, its slot goes back as it would have, and nobody's tokens change.
 """
 from __future__ import annotations
 
@@ -19,7 +26,9 @@ from typing import Sequence
 
 from .. import profiler
 from ..errors import CacheError, ShapeError
-from ..sampling import DeviceHistory, SamplingParams, SequenceSampler, sample_batch
+import torch
+
+from ..sampling import DeviceHistory, SamplingParams, SequenceSampler, pick_batch, sample_batch
 from .step import StepEntry
 
 
@@ -90,6 +99,27 @@ class _Live:
         self.reason = None
 
 
+class _Flight:
+    """A step that has been launched and sampled but whose picks the host has not read: its sequences, the
+    ids on the device, and their copy on its way into a pinned buffer."""
+
+    def __init__(self, members, ids, pinned, turn):
+        self.members, self.ids, self.event, self.host = members, ids, None, None
+        if ids.is_cuda:
+            if pinned[turn] is None or pinned[turn].numel() < ids.numel():
+                pinned[turn] = torch.empty(max(ids.numel(), 64), dtype=torch.int32, pin_memory=True)
+            self.host = pinned[turn][:ids.numel()]
+            self.host.copy_(ids, non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record()
+
+    def read(self) -> list:
+        if self.event is None:
+            return self.ids.tolist()
+        self.event.synchronize()
+        return self.host.tolist()
+
+
 def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sampling: SamplingParams,
               stop: frozenset, ignore_eos: bool, stats: GenerationStats, on_token=None) -> dict:
     """Serve one batch to the end; returns request -> (tokens, reason)."""
@@ -117,38 +147,77 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
         for s, tok in zip(live, picks):
             s.next_token, s.generated = int(tok), 1
         t0 = time.perf_counter()
-        while live:
-            going = []
-            for s in live:
-                if not ignore_eos and s.next_token in stop:
-                    s.reason = "stop"                           # tested before output; not part of it
+
+        def settle(s) -> bool:
+            """The rules for a token that has just become known; whether the sequence goes on."""
+            if not ignore_eos and s.next_token in stop:
+                s.reason = "stop"                               # tested before output; not part of it
+            else:
+                s.out.append(s.next_token)
+                if on_token is not None:
+                    on_token(s.request, s.next_token)
+                if s.generated >= max_new_tokens:
+                    s.reason = "length"                         # put out but never fed
+            if s.reason is None:
+                return True
+            done[s.request] = (s.out, s.reason)
+            cache.release(s.slot)                               # slot and pages go back at once
+            held.discard(s.slot)
+            return False
+
+        ahead = sampling.repetition_penalty == 1.0 and hasattr(engine, "decode_on_device")
+        pinned = [None, None]
+        flight = None                                           # the step whose picks the host has not read yet
+        while True:
+            if flight is None:
+                # every sequence of `live` has a token that is known and not yet settled
+                live = [s for s in live if settle(s)]
+                if not live:
+                    break
+                logits = engine.step([StepEntry(s.slot, [s.next_token], "last") for s in live])
+                for s in live:
+                    s.sampler.history.append(s.next_token)
+                if history is not None:
+                    history.mark([s.sampler.seen_row for s in live], [s.next_token for s in live])
+                with profiler.section(profiler.SAMPLING):
+                    picks = pick_batch(logits, [s.sampler for s in live], history)
+                for s in live:
+                    s.generated += 1
+                stats.decode_tokens += len(live)
+                stats.decode_steps += 1
+                if ahead:
+                    flight = _Flight(live, picks, pinned, stats.decode_steps & 1)
                 else:
-                    s.out.append(s.next_token)
-                    if on_token is not None:
-                        on_token(s.request, s.next_token)
-                    if s.generated >= max_new_tokens:
-                        s.reason = "length"                     # put out but never fed
+                    for s, tok in zip(live, picks.tolist()):
+                        s.next_token = int(tok)
+                continue
+            # A step is in flight.  Whoever took part in it and may have another token goes into the next step
+            # with the id it picked, before the host knows that id; then the host reads the picks in flight.
+            members = flight.members
+            going = [i for i, s in enumerate(members) if s.reason is None and s.generated < max_new_tokens]
+            logits = None
+            if going:
+                ids = flight.ids if len(going) == len(members) else flight.ids[torch.tensor(going, device=flight.ids.device)]
+                logits = engine.decode_on_device([members[i].slot for i in going], ids)
+            for s, tok in zip(members, flight.read()):
                 if s.reason is None:
-                    going.append(s)
-                else:
-                    done[s.request] = (s.out, s.reason)
-                    cache.release(s.slot)                       # slot and pages go back at once
-                    held.discard(s.slot)
-            live = going
-            if not live:
-                break
-            logits = engine.step([StepEntry(s.slot, [s.next_token], "last") for s in live])
-            for s in live:
-                s.sampler.history.append(s.next_token)
-            if history is not None:
-                history.mark([s.sampler.seen_row for s in live], [s.next_token for s in live])
+                    s.next_token = int(tok)
+            if logits is None:                                  # nothing launched: on with the tokens themselves
+                live, flight = [s for s in members if s.reason is None], None
+                continue
+            carried = [members[i] for i in going]
             with profiler.section(profiler.SAMPLING):
-                picks = sample_batch(logits, [s.sampler for s in live], history)
-            for s, tok in zip(live, picks):
-                s.next_token = int(tok)
+                picks = pick_batch(logits, [s.sampler for s in carried], None)
+            for s in members:
+                if s.reason is None:
+                    settle(s)
+            fed = [s for s in carried if s.reason is None]      # the others were carried a step too far
+            for s in fed:
+                s.sampler.history.append(s.next_token)
                 s.generated += 1
-            stats.decode_tokens += len(live)
-            stats.decode_steps += 1
+            stats.decode_tokens += len(fed)
+            stats.decode_steps += 1 if fed else 0
+            flight = _Flight(carried, picks, pinned, stats.decode_steps & 1)
         stats.decode_seconds += time.perf_counter() - t0
     finally:
         for slot in held:

@@ -244,17 +244,25 @@ class Engine:
         self.cache.commit(ctx.slot_list, ctx.new_counts)
         return dg.logits
 
-    def _replay(self, dg: _DecodeGraph, entries: Sequence[StepEntry], slots: np.ndarray) -> torch.Tensor:
+    def _replay(self, dg: _DecodeGraph, entries: Sequence[StepEntry] | None, slots: np.ndarray,
+                ids_dev: torch.Tensor | None = None) -> torch.Tensor:
         """A decode step whose graph exists: reserve the pages, write the step's layout into the buffers the
         graph reads, replay.  The same layout as ``build_context`` makes, without the objects a first run
-        needs (at 64 sequences the host's share of a step is a few per cent of it)."""
+        needs (at 64 sequences the host's share of a step is a few per cent of it).  With ``ids_dev`` the
+        tokens are int32 ids already on the device (what the step before picked): they are copied into the
+        layout there, after its other pieces have come from the host."""
         cache, batch = self.cache, dg.batch
-        tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=batch)
         vocab = self.model.spec.vocab_size
-        if tokens.min() < 0 or tokens.max() >= vocab:
-            bad = int(tokens[(tokens < 0) | (tokens >= vocab)][0])
-            raise ShapeError(f"token id {bad} is outside the vocabulary of {vocab}")
-        tokens = tokens.astype(np.int32)
+        if ids_dev is None:
+            tokens = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=batch)
+            if tokens.min() < 0 or tokens.max() >= vocab:
+                bad = int(tokens[(tokens < 0) | (tokens >= vocab)][0])
+                raise ShapeError(f"token id {bad} is outside the vocabulary of {vocab}")
+            tokens = tokens.astype(np.int32)
+        else:
+            if ids_dev.dtype != torch.int32 or ids_dev.shape != (batch,) or ids_dev.device != dg.ctx.tokens.device:
+                raise ShapeError(f"the ids of {batch} sequences on the device: got {tuple(ids_dev.shape)} {ids_dev.dtype}")
+            tokens = np.zeros(batch, dtype=np.int32)         # their place in the layout; the ids follow on the device
         ones = np.ones(batch, dtype=np.int32)
         want = np.arange(batch, dtype=np.int32)
         cache.reserve(slots, ones)
@@ -268,6 +276,23 @@ class Engine:
         if used < 0:
             raise ShapeError(cache_native.lib().ri_last_error().decode())
         dg.staging.upload(used)
+        if ids_dev is not None:
+            dg.ctx.tokens.copy_(ids_dev)                     # in stream order: after the layout, before the graph
         dg.graph.replay()
         cache.commit(slots, ones)
         return dg.logits
+
+    def decode_on_device(self, slots: Sequence[int], ids_dev: torch.Tensor) -> torch.Tensor | None:
+        """A decode step (one token per sequence, logits of every one) whose tokens are int32 ids on the device,
+        so that the host need not have read them: the generation loop launches a step with what the step
+        before picked and reads those picks while it runs.  Returns None where there is no captured graph for
+        this step's size yet (or no graphs at all): the caller then takes ``step`` with the tokens themselves."""
+        if not self.use_graphs or profiler.enabled() or len(slots) == 0:
+            return None
+        slots = np.asarray(slots, dtype=np.int32)
+        key = (len(slots), _decode_bound(self.cache, self.cache.longest(slots) + 1))
+        dg = self._graphs.get(key)
+        if dg is None or dg.graph is None:
+            return None
+        self._graphs[key] = self._graphs.pop(key)            # the most recently used sits last
+        return self._replay(dg, None, slots, ids_dev)

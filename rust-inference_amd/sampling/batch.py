@@ -40,18 +40,19 @@ class DeviceHistory:
                           torch.tensor(tokens, dtype=torch.int32, device=dev))
 
 
-def sample_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> list[int]:
-    """One token per row of float32 ``logits [B, vocab]``; appends nothing to the histories."""
+def pick_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> torch.Tensor:
+    """One token per row of float32 ``logits [B, vocab]`` as int32 ids where the logits are (on the GPU nothing
+    waits for them); appends nothing to the histories."""
     if logits.shape[0] != len(samplers):
         raise ValueError(f"{logits.shape[0]} rows of logits for {len(samplers)} sequences")
     if not logits.is_cuda:          # logits that never were on a GPU (tests of the loop): the host sampler
         rows = logits.detach().to(torch.float32).numpy()
-        return [s.host.sample(rows[i], s.history) for i, s in enumerate(samplers)]
+        return torch.tensor([s.host.sample(rows[i], s.history) for i, s in enumerate(samplers)], dtype=torch.int32)
     p = samplers[0].params
     if any(s.params != p for s in samplers):
         raise ValueError("the sequences of one batch share their sampling parameters")
     if p.greedy and p.repetition_penalty == 1.0:
-        return ops.argmax(logits).tolist()
+        return ops.argmax(logits)
     dev = logits.device
     uniform = None
     if not p.greedy:
@@ -62,4 +63,10 @@ def sample_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history:
             raise ValueError("a repetition penalty needs the device history of the batch")
         seen = history.seen
         seen_rows = torch.tensor([s.seen_row for s in samplers], dtype=torch.int32, device=dev)
-    return ops.sample(logits, uniform, p.temperature, p.top_k, p.top_p, p.repetition_penalty, seen, seen_rows).tolist()
+    return ops.sample(logits, uniform, p.temperature, p.top_k, p.top_p, p.repetition_penalty, seen, seen_rows)
+
+
+def sample_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> list[int]:
+    """One token per row of float32 ``logits [B, vocab]``, read back to the host; appends nothing to the
+    histories."""
+    return pick_batch(logits, samplers, history).tolist()

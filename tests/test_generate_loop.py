@@ -109,6 +109,101 @@ def test_more_requests_than_slots_run_as_batches_one_after_another():
     assert eng.cache.slots.free_count == 2
 
 
+class AheadEngine(ScriptedEngine):
+    """The scripted engine with steps that take their tokens as ids "on the device" (here: a tensor the loop
+    has not read), as the real engine's captured graphs do; like it, it has no such step for a batch size
+    until a step with the tokens themselves has run at that size."""
+
+    def __init__(self, *a, **k):
+        super().__init__(*a, **k)
+        self.known_sizes, self.on_device = set(), []
+
+    def step(self, entries):
+        if all(len(e.tokens) == 1 for e in entries):
+            self.known_sizes.add(len(entries))
+        return super().step(entries)
+
+    def decode_on_device(self, slots, ids):
+        if len(slots) not in self.known_sizes:
+            return None
+        assert ids.dtype == torch.int32 and ids.shape == (len(slots),)
+        self.on_device.append(list(slots))
+        return ScriptedEngine.step(self, [StepEntry(s, [int(t)], "last") for s, t in zip(slots, ids.tolist())])
+
+
+def test_one_step_ahead_gives_the_same_tokens_and_carries_an_ended_sequence_one_step_at_most():
+    prompts = [[1, 2, 3], [9, 9], [5], [4, 4, 4, 4]]
+    full = [expected(p, 12)[0] for p in prompts]
+    others = set(full[0]) | set(full[2])
+    stop = {next(t for t in full[1][2:] if t not in others), next(t for t in full[3][5:] if t not in others)}
+    plain = generate(ScriptedEngine(), prompts, max_new_tokens=12, stop_token_ids=stop)
+    eng = AheadEngine()
+    res = generate(eng, prompts, max_new_tokens=12, stop_token_ids=stop)
+    assert res.tokens == plain.tokens and res.finish_reasons == plain.finish_reasons
+    for p, toks, why in zip(prompts, res.tokens, res.finish_reasons):
+        assert (toks, why) == expected(p, 12, stop)
+    assert "stop" in res.finish_reasons and "length" in res.finish_reasons
+    assert eng.on_device, "steps did run with ids the loop had not read"
+    # what the statistics count is what the plain loop counts: steps and tokens that were asked for
+    assert res.stats.decode_tokens == plain.stats.decode_tokens and res.stats.decode_steps == plain.stats.decode_steps
+    # a sequence is fed at most one token more than the plain loop feeds it (the step that was launched before
+    # its stop token was read), and never more than its pages were planned for
+    fed = {r: 0 for r in range(len(prompts))}
+    for slots, counts in eng.steps[1:]:
+        for sl in slots:
+            fed[sl] += 1
+    for r, toks in enumerate(res.tokens):
+        wanted = len(toks) if res.finish_reasons[r] == "stop" else len(toks) - 1
+        assert wanted <= fed[r] <= wanted + 1 and fed[r] <= 11
+    eng.cache.check_consistent()
+    assert eng.cache.slots.free_count == 4 and eng.cache.free_pages() == [32]
+
+
+def test_one_step_ahead_with_a_stop_token_first_and_batches_one_after_another():
+    p = [3, 4]
+    first = expected(p, 1)[0][0]
+    res = generate(AheadEngine(), [p, [8]], max_new_tokens=5, stop_token_ids=[first])
+    assert res.tokens[0] == [] and res.finish_reasons[0] == "stop"
+    assert (res.tokens[1], res.finish_reasons[1]) == expected([8], 5, {first})
+    eng = AheadEngine(slots=2)
+    prompts = [[i + 1] * (i + 1) for i in range(5)]
+    res = generate(eng, prompts, max_new_tokens=4)
+    assert res.tokens == [expected(q, 4)[0] for q in prompts] and res.stats.batches == 3
+    eng.cache.check_consistent()
+    assert eng.cache.slots.free_count == 2
+    one = generate(AheadEngine(), [[4, 5, 6]], max_new_tokens=1)
+    assert one.tokens == [expected([4, 5, 6], 1)[0]] and one.finish_reasons == ["length"]
+    # everything stops at once: the step launched ahead was for nobody, and is not counted
+    q = [[7], [7]]
+    second = expected([7], 2)[0][1]
+    both = generate(AheadEngine(), q, max_new_tokens=9, stop_token_ids=[second])
+    assert both.tokens == [expected([7], 9, {second})[0]] * 2 and both.finish_reasons == ["stop", "stop"]
+    assert both.stats.decode_steps == 1 and both.stats.decode_tokens == 2
+
+
+def test_one_step_ahead_draws_the_same_numbers_as_the_plain_loop():
+    class Flat(AheadEngine):
+        def step(self, entries):
+            super().step(entries)
+            return torch.zeros(len(entries), VOCAB)
+
+        def decode_on_device(self, slots, ids):
+            out = super().decode_on_device(slots, ids)
+            return None if out is None else torch.zeros(len(slots), VOCAB)
+
+    class FlatPlain(ScriptedEngine):
+        def step(self, entries):
+            super().step(entries)
+            return torch.zeros(len(entries), VOCAB)
+    prompts = [[1], [2], [3]]
+    p = SamplingParams(temperature=1.0, seed=11)
+    assert generate(Flat(), prompts, 9, p).tokens == generate(FlatPlain(), prompts, 9, p).tokens
+    # with a repetition penalty the tokens are needed on the host before the next step: no step runs ahead
+    eng = AheadEngine()
+    generate(eng, prompts, 5, SamplingParams(repetition_penalty=1.2))
+    assert not eng.on_device
+
+
 def test_batches_are_cut_to_fit_the_pages():
     # pages of 32: each request of 40 + 30 - 1 = 69 tokens needs 3 pages; 7 pages hold two of them
     assert plan_batches([40, 40, 40], 30, 32, 7, 8, 256) == [range(0, 2), range(2, 3)]
