@@ -20,10 +20,15 @@ def read_model_f64(model_dir):
 
 
 def reference_fixture(name):
-    """The folder `tests/fixtures/<name>` of the reference, or None when it is not at hand: the folder the
-    environment variable RI_REFERENCE_FIXTURES names, else `reference/tests/fixtures` beside this checkout."""
-    here = os.path.dirname(os.path.dirname(os.path.realpath(__file__)))
-    for base in (os.environ.get("RI_REFERENCE_FIXTURES"), os.path.join(os.path.dirname(here), "reference", "tests", "fixtures")):
+    """A fixture that the reference's own tests hold (`tests/fixtures/<name>` there: a model folder with the
+    logits and tokens its authors recorded).  `tiny-qwen3` lies beside these tests as a copy of those data files,
+    so that the comparison runs wherever the tests do; others are looked for in the folder the environment
+    variable RI_REFERENCE_FIXTURES names, else in `reference/tests/fixtures` beside this checkout, and None is
+    returned where they are not at hand."""
+    tests = os.path.dirname(os.path.realpath(__file__))
+    here = os.path.dirname(tests)
+    for base in (os.path.join(tests, "fixtures"), os.environ.get("RI_REFERENCE_FIXTURES"),
+                 os.path.join(os.path.dirname(here), "reference", "tests", "fixtures")):
         if base and os.path.isfile(os.path.join(base, name, "config.json")):
             return os.path.join(base, name)
     return None
