@@ -10,6 +10,7 @@ from typing import Sequence
 
 import torch
 
+from .cache import PAGE_SIZE
 from .engine import Engine, GenerationResult, StepEntry, generate as _generate
 from .parts import load_model, random_model
 from .sampling import DEFAULT_SEED, SamplingParams
@@ -34,8 +35,7 @@ class Model:
                  use_graphs: bool = True):
         self.decoder = decoder
         self.config = getattr(decoder, "config", None)
-        page = 32
-        per_seq = -(-max_seq_len // page) * page
+        per_seq = -(-max_seq_len // PAGE_SIZE) * PAGE_SIZE
         self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
         self.engine = Engine(decoder, self.cache, use_graphs=use_graphs)
 
@@ -51,8 +51,10 @@ class Model:
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 600, temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 1.0, repetition_penalty: float = 1.0, seed: int = DEFAULT_SEED,
                  stop_token_ids: Sequence[int] = (), ignore_eos: bool = False, max_batch: int | None = None,
-                 on_token=None) -> GenerationResult:
-        params = SamplingParams(temperature, top_k, top_p, repetition_penalty, seed)
+                 on_token=None, sampling: Sequence[SamplingParams] | None = None) -> GenerationResult:
+        """The options are the reference runner's (src/bin/runner.rs:78-96) and hold for every prompt;
+        ``sampling`` instead gives every prompt its own ``SamplingParams``."""
+        params = sampling if sampling is not None else SamplingParams(temperature, top_k, top_p, repetition_penalty, seed)
         return _generate(self.engine, prompts, max_new_tokens, params, stop_token_ids, ignore_eos, max_batch, on_token)
 
     def step(self, entries) -> torch.Tensor:

@@ -11,6 +11,8 @@ extern "C" {
 
 const char* ri_last_error(void);
 int ri_abi_version(void);
+// Compute units of the current device (256 where there is none): what the launch-sizing rules count against.
+int ri_compute_units(void);
 
 // out[t, :] = table[ids[t], :] as float32.  ids are int32 and must be < vocab (checked by the caller).
 int ri_embed_gather(float* out, const void* table, int table_dtype, const int32_t* ids,

@@ -930,15 +930,19 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 // do not keep the memory busy (one sequence of 131,000 keys in 16 runs: 12% longer; runs of four chunks: no
 // gain), and runs that need a join lose at a few thousand keys (2 runs at 48 sequences of 2,080 keys: -2.5%;
 // 4 runs at 16 sequences of 4,100: -1.5%; 32 sequences of 4,100 gain 2.5% and are left to the chunks with them).
-#define STREAM_WORKGROUPS 1024
+// (The counts of workgroups above were measured on 256 compute units and are kept per compute unit: two of
+// them for each to stream at all, four for each where runs are joined.)
+#define STREAM_WORKGROUPS_PER_CU 4
+#define STREAM_MIN_PER_CU 2
 #define STREAM_MIN_CHUNKS 8
 #define STREAM_JOINED_FROM 64
 static int stream_splits(int seqs, int kv_heads, int max_chunks) {
     const long rows = (long)seqs * kv_heads;
-    if (rows >= 512) return 1;
+    const long cus = ri_compute_units();
+    if (rows >= STREAM_MIN_PER_CU * cus) return 1;
     if (max_chunks < STREAM_JOINED_FROM) return 0;
-    const long splits = min((STREAM_WORKGROUPS + rows - 1) / rows, (long)max_chunks / STREAM_MIN_CHUNKS);
-    if (splits < 2 || rows * splits < 512) return 0;
+    const long splits = min((STREAM_WORKGROUPS_PER_CU * cus + rows - 1) / rows, (long)max_chunks / STREAM_MIN_CHUNKS);
+    if (splits < 2 || rows * splits < STREAM_MIN_PER_CU * cus) return 0;
     return (int)splits;
 }
 
@@ -1107,16 +1111,17 @@ static int check_common(const char* name, int heads, int kv_heads, int head_dim,
 // prompt of a few thousand tokens: at 32 query and 8 kv heads of 128, 2,048 tokens take 81 us with 1,024
 // workgroups of half the columns against 95 us with 512; from 4,096 tokens on the full tiles win).  A
 // column's arithmetic does not depend on the tile it sits in, only the grid does.
-// Tiles are halved while the launch has fewer workgroups than this: three for each of the 256 compute units
-// (a prompt of 3,072 tokens at Qwen3-8B sizes: 105 us with two tiles a wavefront in 768 workgroups, 126 us with
-// one tile in 1,536; at 2,048 tokens one tile in 1,024 workgroups takes 57 us, two in 512 take 67).
-#define PREFILL_MIN_WGS 768
+// Tiles are halved while the launch has fewer workgroups than this many for each compute unit (measured with
+// 256 of them: a prompt of 3,072 tokens at Qwen3-8B sizes takes 105 us with two tiles a wavefront in 768
+// workgroups, 126 us with one tile in 1,536; at 2,048 tokens one tile in 1,024 workgroups takes 57 us, two in
+// 512 take 67).
+#define PREFILL_MIN_WGS_PER_CU 3
 static int prefill_tiles(int head_dim, int group, int max_new, int seqs, int kv_heads) {
     int nt = head_dim <= 64 ? 4 : 2;
     while (nt > 1 && group <= 16 * (nt / 2)) {
         const int tile_tokens = (16 * nt) / group;
         const long wgs = (long)((max_new + 4 * tile_tokens - 1) / (4 * tile_tokens)) * seqs * kv_heads;
-        if (wgs >= PREFILL_MIN_WGS) break;
+        if (wgs >= (long)PREFILL_MIN_WGS_PER_CU * ri_compute_units()) break;
         nt /= 2;
     }
     return nt;

@@ -164,20 +164,21 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
 // would have to be added by a kernel of their own).
 // (Measured on 4096 x 12288 at 64 rows with four wavefronts: 66, 38, 26 and 26 us with 1, 2, 4 and 8 stretches;
 // every stretch more is another float32 copy of the result for the reader to add.)
-static int wide_parts(int groups, int k_tiles, bool swiglu) {
+static int wide_parts(int groups, int k_tiles, bool swiglu, int cus) {
     int parts = 1;
-    while (!swiglu && parts < 16 && groups * parts < 256 && k_tiles / (parts * 2) >= 2 * WD_SLICE) parts *= 2;
+    while (!swiglu && parts < 16 && groups * parts < cus && k_tiles / (parts * 2) >= 2 * WD_SLICE) parts *= 2;
     return parts;
 }
 
 extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts) {
     const int row_tiles = (n + 15) / 16, k_tiles = (k + 31) / 32;
+    const int cus = ri_compute_units();
     double best = -1.0;
     for (int w = 4; w >= 3; --w) {
         const int groups = (row_tiles + w - 1) / w;
-        const int p = wide_parts(groups, k_tiles, swiglu != 0);
+        const int p = wide_parts(groups, k_tiles, swiglu != 0, cus);
         const long wgs = (long)groups * p;
-        const double fill = (double)wgs / (double)((wgs + 255) / 256 * 256);
+        const double fill = (double)wgs / (double)((wgs + cus - 1) / cus * cus);
         if (fill > best + 1e-9) {
             best = fill;
             *waves = w;

@@ -120,14 +120,17 @@ class _Flight:
         return self.host.tolist()
 
 
-def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sampling: SamplingParams,
+def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sampling,
               stop: frozenset, ignore_eos: bool, stats: GenerationStats, on_token=None) -> dict:
-    """Serve one batch to the end; returns request -> (tokens, reason)."""
+    """Serve one batch to the end; returns request -> (tokens, reason).  ``sampling`` is one ``SamplingParams``
+    for every request, or one per request (indexed like ``prompts``)."""
     cache = engine.cache
     live = []
+    of = (lambda r: sampling) if isinstance(sampling, SamplingParams) else (lambda r: sampling[r])
+    penalised = any(of(r).repetition_penalty != 1.0 for r in requests)
     try:
         for r in requests:
-            live.append(_Live(r, cache.acquire(), list(prompts[r]), SequenceSampler(sampling, r, prompts[r])))
+            live.append(_Live(r, cache.acquire(), list(prompts[r]), SequenceSampler(of(r), r, prompts[r])))
     except Exception:
         for s in live:
             cache.release(s.slot)
@@ -138,7 +141,7 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
         t0 = time.perf_counter()
         logits = engine.step([StepEntry(s.slot, s.prompt, "last") for s in live])
         history = None
-        if sampling.repetition_penalty != 1.0 and logits.is_cuda:
+        if penalised and logits.is_cuda:
             history = DeviceHistory([s.sampler for s in live], logits.shape[1], logits.device)
         with profiler.section(profiler.SAMPLING):
             picks = sample_batch(logits, [s.sampler for s in live], history)
@@ -165,7 +168,7 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
             held.discard(s.slot)
             return False
 
-        ahead = sampling.repetition_penalty == 1.0 and hasattr(engine, "decode_on_device")
+        ahead = not penalised and hasattr(engine, "decode_on_device")
         pinned = [None, None]
         flight = None                                           # the step whose picks the host has not read yet
         while True:
@@ -226,10 +229,15 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
 
 
 def generate(engine, prompts: Sequence[Sequence[int]], max_new_tokens: int = 600,
-             sampling: SamplingParams | None = None, stop_token_ids: Sequence[int] = (), ignore_eos: bool = False,
+             sampling: SamplingParams | Sequence[SamplingParams] | None = None, stop_token_ids: Sequence[int] = (), ignore_eos: bool = False,
              max_batch: int | None = None, on_token=None) -> GenerationResult:
-    """Generate for every prompt; results in the order of the prompts."""
+    """Generate for every prompt; results in the order of the prompts.  ``sampling``: one ``SamplingParams``
+    for all of them, or a list with one per prompt."""
     sampling = sampling or SamplingParams()
+    if not isinstance(sampling, SamplingParams):
+        sampling = list(sampling)
+        if len(sampling) != len(prompts):
+            raise ShapeError(f"{len(sampling)} sampling parameters for {len(prompts)} prompts")
     if max_new_tokens < 1:
         raise ShapeError("max_new_tokens must be at least 1")
     cache = engine.cache

@@ -16,6 +16,7 @@ import sys
 
 import torch
 
+from ..cache import PAGE_SIZE
 from ..errors import InferenceError
 from ..parts import load_model
 from .step import Engine, StepEntry
@@ -49,10 +50,11 @@ class Replayer:
 
 def engine_for_trace(model, max_tokens: int) -> Engine:
     """An engine whose cache holds ``max_tokens`` tokens of live requests, each request's count
-    rounded up to a multiple of 64 by the caller (two pages of 32)."""
-    page = 32
-    max_tokens = max(max_tokens, page)
-    cache = model.new_cache(max_tokens=max_tokens, num_slots=max(1, -(-max_tokens // 64)),
+    rounded up to a multiple of 64 by the caller (whole pages, where a page divides 64; else the cache
+    rounds every request up to its own pages, and the trace's bound is read as that many pages' worth)."""
+    max_tokens = max(max_tokens, PAGE_SIZE)
+    unit = max(64, PAGE_SIZE)                     # the smallest request the bound counts
+    cache = model.new_cache(max_tokens=max_tokens, num_slots=max(1, -(-max_tokens // unit)),
                             max_seq_len=max_tokens)
     return Engine(model, cache)
 

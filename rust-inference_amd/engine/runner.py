@@ -31,7 +31,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--think", action="store_true", help="with --chat, leave thinking mode enabled")
     ap.add_argument("--ignore-eos", action="store_true", help="keep generating past end-of-sequence tokens")
     ap.add_argument("--tokenizer", help="directory holding tokenizer.json, if not the model directory")
-    ap.add_argument("--max-pages", type=int, default=256, help="KV cache pages per layer (32 tokens each)")
+    ap.add_argument("--max-pages", type=int, default=256, help="KV cache pages per layer (a page holds 32 tokens, as the reference's: src/kvcache.rs:12)")
     ap.add_argument("--pages-per-seq", type=int, default=128, help="maximum KV pages per sequence")
     ap.add_argument("-t", "--threads", type=int, default=None, help="host worker threads (defaults to all cores)")
     ap.add_argument("--profile", action="store_true", help="print a per-step timing summary at the end")
@@ -145,12 +145,13 @@ def main(argv=None) -> int:
 
     from .. import profiler
     from ..api import Model
+    from ..cache import PAGE_SIZE
     from ..errors import InferenceError
     profiler.enable(args.profile)                                      # src/bin/runner.rs:207
     t0 = time.perf_counter()
     try:
-        per_seq = args.pages_per_seq * 32
-        options = dict(max_batch=min(len(prompts), 64), max_seq_len=per_seq, max_tokens=args.max_pages * 32,
+        per_seq = args.pages_per_seq * PAGE_SIZE
+        options = dict(max_batch=min(len(prompts), 64), max_seq_len=per_seq, max_tokens=args.max_pages * PAGE_SIZE,
                        use_graphs=not args.no_graphs)
         if args.random:
             path = args.model_dir if os.path.isfile(args.model_dir) else os.path.join(args.model_dir, "config.json")

@@ -47,6 +47,7 @@ _SIGNATURES = {
     "ri_gemm_wide_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_int, c_void_p],
     "ri_gemm_wide_packed_bf16_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
+    "ri_compute_units": [],
     "ri_sum_parts": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_attention_decode_streams": [c_int, c_int, c_int],
@@ -505,6 +506,12 @@ def gemm_mid_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bfloa
           _dev(x.data if x_tiled else x, "x", torch.bfloat16), _dev(wpacked, "wpacked", torch.bfloat16), m, n, k,
           int(swiglu), (TILED_X if x_tiled else 0) | (TILED_OUT if tiled_out else 0), _stream())
     return out
+
+
+def compute_units() -> int:
+    """Compute units of the current device (256 where there is none): what the rules that size launches
+    count workgroups against."""
+    return int(_get("ri_compute_units")())
 
 
 def wide_product_plan(n: int, k: int, swiglu: bool = False) -> tuple[int, int]:

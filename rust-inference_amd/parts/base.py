@@ -19,6 +19,27 @@ class Part:
         """Take the weights (host tensors, as stored) and put what is needed on the device."""
         self.rt = rt
 
+    def connect(self, parts: dict) -> None:
+        """Called once after every part of the model is bound, with the model's own parts by name
+        (``"embedding"``, ``"final_norm"``, ``"head"``, ``"layers"``): for a part that shares something with
+        another one (an output matrix tied to the embedding table).  Most parts need nothing here."""
+
+
+class Embedding(Part):
+    """``forward(ctx) -> [T, hidden]`` float32: what the residual stream starts from.  The part gets the whole
+    step's context, so one that adds something by position (``ctx.tok_pos``) or by sequence (``ctx.tok_seq``,
+    ``ctx.slots``) to the rows of its table needs nothing from the model."""
+
+    def forward(self, ctx):
+        raise NotImplementedError
+
+
+class Head(Part):
+    """``forward(x) -> [rows, vocab]`` float32 logits of the final norm's rows."""
+
+    def forward(self, x):
+        raise NotImplementedError
+
 
 class Norm(Part):
     """``apply(residual, pending, out_dtype, rows=None)``: adds ``pending`` into the

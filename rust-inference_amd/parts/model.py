@@ -13,7 +13,7 @@ from .. import profiler
 from ..kernels import ops
 from ..weights.loader import MATRIX, TensorSpec, load_checked
 from ..weights.random_init import random_tensors
-from .base import Part
+from .base import Embedding, Head
 from .block import ResidualStream
 from .registry import build_part, part_class, register_part
 from .runtime import Runtime
@@ -21,7 +21,7 @@ from .spec import ModelSpec
 
 
 @register_part("embedding", "table")
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     """``h[t, :] = E[id_t, :]`` without scaling (the reference: src/ops/embedding.rs:10-42)."""
 
     def __init__(self, vocab: int, dim: int, name: str):
@@ -34,12 +34,12 @@ class TokenEmbedding(Part):
         self.rt = rt
         self.table = rt.place_matrix(weights[self.name])
 
-    def forward(self, ids):
-        return ops.embed_gather(self.table, ids)
+    def forward(self, ctx):
+        return ops.embed_gather(self.table, ctx.tokens)
 
 
 @register_part("head", "linear")
-class OutputHead(Part):
+class OutputHead(Head):
     """``logits = x W^T`` in float32, no scaling or cap.  The matrix is the embedding
     table when the configuration ties them or the checkpoint has no tensor of this
     name (the reference: src/models/qwen3.rs:167-171, :286)."""
@@ -53,23 +53,35 @@ class OutputHead(Part):
     def written_when_random(self) -> bool:
         return not self.tied
 
-    def bind(self, weights, rt, embedding: TokenEmbedding | None = None):
+    def bind(self, weights, rt):
         self.rt = rt
-        if self.tied or self.name not in weights:
-            if embedding is None:
-                raise ConfigError(f"{self.name} is absent and there is no embedding to tie it to")
-            self.weight = embedding.table           # the same device tensor: tying costs no memory
-        else:
+        self.weight = self.packed = None
+        if not self.tied and self.name in weights:
             self.weight = rt.place_matrix(weights[self.name])
-        # A second copy in the matrix cores' tile order for steps that want 2 to 16 rows of logits (a decode step
-        # of as many sequences): at 151,936 x 4,096 the packed kernel takes 0.21 ms where the library's product
-        # takes 0.26 (1% of such a step), for 1.2 GB more memory.  One row goes to the one-row kernel, more than
-        # 16 to the library, both on the row-major matrix.
-        self.packed = rt.pack(self.weight, always=True)
+
+    def connect(self, parts):
+        if self.weight is None:
+            table = getattr(parts.get("embedding"), "table", None)
+            if table is None or tuple(table.shape) != (self.vocab, self.dim):
+                raise ConfigError(f"{self.name} is absent and there is no embedding table of {self.vocab} x {self.dim} "
+                                  "to tie it to")
+            self.weight = table                     # the same device tensor: tying costs no memory
+
+    def _packed_copy(self):
+        """A second copy of the matrix in the matrix cores' tile order, for steps that want 2 to 16 rows of
+        logits (a decode step of as many sequences): at 151,936 x 4,096 the packed kernel takes 0.21 ms where
+        the library's product takes 0.26 (1% of such a step), for 1.2 GB more memory.  It is made at the first
+        such step, so that a model which never runs one (a single slot, or only larger batches) does not pay
+        for it; never while a graph is being captured (the engine runs every step once before it captures it)."""
+        if self.packed is None and not torch.cuda.is_current_stream_capturing():
+            self.packed = self.rt.pack(self.weight, always=True)
+        return self.packed
 
     def forward(self, x):
-        if self.packed.packed is not None and 2 <= x.shape[0] <= 16:
-            return self.rt.linear_packed(x, self.packed, out_dtype=torch.float32)
+        if 2 <= x.shape[0] <= 16:
+            packed = self._packed_copy()
+            if packed is not None and packed.packed is not None:
+                return self.rt.linear_packed(x, packed, out_dtype=torch.float32)
         return self.rt.linear(x, self.weight, out_dtype=torch.float32)
 
 
@@ -112,7 +124,12 @@ class DecoderModel:
             for part in layer.parts():
                 part.bind(weights, rt)
         self.final_norm.bind(weights, rt)
-        self.head.bind(weights, rt, self.embedding)
+        self.head.bind(weights, rt)
+        named = {"embedding": self.embedding, "layers": self.layers, "final_norm": self.final_norm, "head": self.head}
+        for part in self.parts():
+            connect = getattr(part, "connect", None)
+            if connect is not None:
+                connect(named)
         return self
 
     # ---- cache
@@ -149,7 +166,7 @@ class DecoderModel:
         """float32 logits ``[n_want, vocab]`` for the wanted rows of this step's tokens."""
         rt = self.rt
         with profiler.section(profiler.EMBEDDING):
-            stream = ResidualStream(self.embedding.forward(ctx.tokens))
+            stream = ResidualStream(self.embedding.forward(ctx))
         for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]
             follower = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None

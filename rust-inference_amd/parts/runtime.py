@@ -82,15 +82,20 @@ SPLIT_K = 4096
 # cannot add themselves into the residual stream, so only rows of 16,384 elements and more are cut.
 PACKED_MAX_BYTES = 101_000_000
 PACKED_LONG_K = 16384
-COMPUTE_UNITS = 256
+
+
+@functools.lru_cache(maxsize=None)
+def _compute_units() -> int:
+    return ops.compute_units()
 
 
 def _packed_pays(n: int, k: int) -> bool:
     if k >= PACKED_LONG_K or n * k * 2 <= 40_000_000:
         return True
     tiles = -(-n // 16)
-    last_round = tiles % COMPUTE_UNITS
-    return n * k * 2 <= PACKED_MAX_BYTES and not (tiles > COMPUTE_UNITS and 0 < last_round < COMPUTE_UNITS // 2)
+    cus = _compute_units()
+    last_round = tiles % cus
+    return n * k * 2 <= PACKED_MAX_BYTES and not (tiles > cus and 0 < last_round < cus // 2)
 
 
 class PackedWeight:
@@ -183,7 +188,8 @@ class Runtime:
             return False
         waves, parts = _wide_plan(pw.n, pw.k, True)
         groups = -(-(-(-pw.n // 16)) // waves) * parts
-        return groups / (-(-groups // 256) * 256) >= WIDE_GATED_FILL
+        cus = _compute_units()
+        return groups / (-(-groups // cus) * cus) >= WIDE_GATED_FILL
 
     def takes_tiled(self, pw: PackedWeight, m: int, parts_ok: bool = False) -> bool:
         """Whether the product of ``m`` rows with this weight (called with this ``parts_ok``) runs on a packed

@@ -40,17 +40,9 @@ class DeviceHistory:
                           torch.tensor(tokens, dtype=torch.int32, device=dev))
 
 
-def pick_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> torch.Tensor:
-    """One token per row of float32 ``logits [B, vocab]`` as int32 ids where the logits are (on the GPU nothing
-    waits for them); appends nothing to the histories."""
-    if logits.shape[0] != len(samplers):
-        raise ValueError(f"{logits.shape[0]} rows of logits for {len(samplers)} sequences")
-    if not logits.is_cuda:          # logits that never were on a GPU (tests of the loop): the host sampler
-        rows = logits.detach().to(torch.float32).numpy()
-        return torch.tensor([s.host.sample(rows[i], s.history) for i, s in enumerate(samplers)], dtype=torch.int32)
+def _pick_alike(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None) -> torch.Tensor:
+    """The rows of a batch whose sequences sample alike: one launch."""
     p = samplers[0].params
-    if any(s.params != p for s in samplers):
-        raise ValueError("the sequences of one batch share their sampling parameters")
     if p.greedy and p.repetition_penalty == 1.0:
         return ops.argmax(logits)
     dev = logits.device
@@ -64,6 +56,33 @@ def pick_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: D
         seen = history.seen
         seen_rows = torch.tensor([s.seen_row for s in samplers], dtype=torch.int32, device=dev)
     return ops.sample(logits, uniform, p.temperature, p.top_k, p.top_p, p.repetition_penalty, seen, seen_rows)
+
+
+def _alike(p: SamplingParams) -> tuple:
+    """What two sequences must share to be picked in one launch (each draws from its own generator anyway)."""
+    return (max(p.temperature, 0.0), p.top_k, p.top_p, p.repetition_penalty)
+
+
+def pick_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> torch.Tensor:
+    """One token per row of float32 ``logits [B, vocab]`` as int32 ids where the logits are (on the GPU nothing
+    waits for them); appends nothing to the histories.  Sequences may sample each in its own way: the rows are
+    grouped by their parameters and every group is one launch (a batch that samples alike, the usual case, is one
+    group and its logits are not copied)."""
+    if logits.shape[0] != len(samplers):
+        raise ValueError(f"{logits.shape[0]} rows of logits for {len(samplers)} sequences")
+    if not logits.is_cuda:          # logits that never were on a GPU (tests of the loop): the host sampler
+        rows = logits.detach().to(torch.float32).numpy()
+        return torch.tensor([s.host.sample(rows[i], s.history) for i, s in enumerate(samplers)], dtype=torch.int32)
+    groups: dict[tuple, list[int]] = {}
+    for i, s in enumerate(samplers):
+        groups.setdefault(_alike(s.params), []).append(i)
+    if len(groups) == 1:
+        return _pick_alike(logits, samplers, history)
+    out = torch.empty(len(samplers), dtype=torch.int32, device=logits.device)
+    for members in groups.values():
+        at = torch.tensor(members, dtype=torch.int64, device=logits.device)
+        out.index_copy_(0, at, _pick_alike(logits.index_select(0, at), [samplers[i] for i in members], history))
+    return out
 
 
 def sample_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None = None) -> list[int]:

@@ -355,3 +355,24 @@ def test_which_decode_steps_the_attention_walks_in_runs():
     assert runs(1, 8, 32896) == 0                      # 16 runs of eight chunks would be 128 workgroups
     assert runs(16, 8, 4200) == 0 and runs(48, 8, 2100) == 0 and runs(32, 8, 8192) == 0
     assert runs(8, 8, 16384) == 8 and runs(8, 8, 16000) == 0
+
+
+def test_every_request_may_sample_in_its_own_way():
+    """A list of sampling parameters, one per prompt: a request's tokens are those it gets when all requests
+    share its parameters (its generator is seeded by its index either way), and a list of the wrong length is
+    refused."""
+    class Peaked(ScriptedEngine):
+        def step(self, entries):
+            logits = super().step(entries)
+            return logits + 0.5 * torch.sin(torch.arange(VOCAB) * 0.7)[None, :]      # a few plausible tokens each
+
+    prompts = [[1, 2, 3], [4, 5], [6], [7, 8, 9, 10]]
+    kinds = [SamplingParams(), SamplingParams(temperature=5.0, seed=11), SamplingParams(temperature=5.0, top_k=3, seed=11),
+             SamplingParams(temperature=2.0, top_p=0.5, repetition_penalty=1.3, seed=11)]
+    mixed = generate(Peaked(), prompts, max_new_tokens=6, sampling=kinds).tokens
+    for i, kind in enumerate(kinds):
+        alone = generate(Peaked(), prompts, max_new_tokens=6, sampling=kind).tokens
+        assert mixed[i] == alone[i], f"request {i}"
+    assert len({tuple(t) for t in mixed}) > 1
+    with pytest.raises(ShapeError, match="sampling parameters"):
+        generate(Peaked(), prompts, max_new_tokens=2, sampling=kinds[:2])

@@ -1097,3 +1097,131 @@ def test_a_layer_of_six_parts_that_keeps_two_things_per_sequence(tmp_path, dtype
         got = plans.collect(steps, lambda i: outs[i], SANDWICH["vocab_size"])
         for rid, toks in reqs.items():
             assert_logits_close(got[rid], sandwich_plain(w, toks), dtype_name, f"sandwich, {what}, {rid}")
+
+
+# ------------------------------------------------------------------------------------------------ positions at the embedding
+LEARNED = {"architectures": ["ToyLearnedPositionsForCausalLM"], "vocab_size": 83, "hidden_size": 48, "inter": 80, "heads": 3,
+           "kv_heads": 1, "head_dim": 16, "eps": 1e-5, "positions": 96}
+
+
+def register_learned_positions():
+    """An embedding of another kind, registered from here: the token's row plus a learned row for its position
+    (absolute positions enter the model here and nowhere else: the attention has no rotation).  The output
+    matrix is tied to this embedding's table, which the head finds among the model's parts by name."""
+    from rust_inference_amd.config import ModelConfig, register_architecture
+    from rust_inference_amd.kernels import ops
+    from rust_inference_amd.parts import Embedding, LayerSpec, ModelSpec, PartSpec, Run, register_part
+    from rust_inference_amd.weights import MATRIX, TensorSpec
+
+    @register_part("embedding", "toy_table_and_positions")
+    class TableAndPositions(Embedding):
+        def __init__(self, vocab, dim, positions, name, positions_name):
+            self.vocab, self.dim, self.positions, self.name, self.positions_name = vocab, dim, positions, name, positions_name
+
+        def tensors(self):
+            return {self.name: TensorSpec((self.vocab, self.dim), MATRIX),
+                    self.positions_name: TensorSpec((self.positions, self.dim), MATRIX)}
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.table = rt.place_matrix(weights[self.name])
+            self.where = rt.place_matrix(weights[self.positions_name])
+
+        def forward(self, ctx):
+            # both gathers by the library's kernel; the positions are the step's own (the cache lengths)
+            return ops.embed_gather(self.table, ctx.tokens) + ops.embed_gather(self.where, ctx.tok_pos)
+
+    @dataclass(frozen=True)
+    class LearnedConfig(ModelConfig):
+        vocab_size: int = 0
+        hidden_size: int = 0
+        inter: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        eps: float = 1e-5
+        positions: int = 0
+        ARCHITECTURE: ClassVar[str] = "ToyLearnedPositionsForCausalLM"
+        MODEL_TYPE: ClassVar[str] = "toy_learned_positions"
+
+        @classmethod
+        def from_dict(cls, raw):
+            import dataclasses
+            return cls(**{f.name: raw[f.name] for f in dataclasses.fields(cls)})
+
+    def spec(c):
+        d = c.hidden_size
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"dim": d, "eps": c.eps, "name": name})
+
+        def layer(p):
+            return LayerSpec(
+                mixer_norm=norm(p + "n1.weight"), feed_forward_norm=norm(p + "n2.weight"),
+                feed_forward=PartSpec("swiglu", {"hidden": d, "inter": c.inter, "prefix": p + "ff."}),
+                mixer=PartSpec("attention", {"hidden": d, "heads": c.heads, "kv_heads": c.kv_heads, "head_dim": c.head_dim,
+                                             "prefix": p + "attn.", "qk_norm": False, "eps": c.eps, "window": None,
+                                             "position": PartSpec("none")}))
+        return ModelSpec(
+            architecture="ToyLearnedPositionsForCausalLM", vocab_size=c.vocab_size, hidden_size=d,
+            embedding=PartSpec("toy_table_and_positions", {"vocab": c.vocab_size, "dim": d, "positions": c.positions,
+                                                           "name": "embed.weight", "positions_name": "embed.positions"}),
+            layers=(layer("l0."), layer("l1.")), schedule=(Run(0, 0), Run(1, 1)),
+            final_norm=norm("final.weight"),
+            head=PartSpec("linear", {"vocab": c.vocab_size, "dim": d, "name": "head.weight", "tied": True}),
+            max_positions=c.positions)
+
+    register_architecture("ToyLearnedPositionsForCausalLM", LearnedConfig, spec, model_types=("toy_learned_positions",))
+
+
+def learned_plain(w, ids):
+    c = LEARNED
+    s = len(ids)
+    h = P.embedding(w["embed.weight"], ids) + w["embed.positions"][:s]
+    for p in ("l0.", "l1."):
+        x = P.rms_norm(h, w[p + "n1.weight"], c["eps"])
+        q = (x @ w[p + "attn.q_proj.weight"].T).reshape(s, c["heads"], c["head_dim"])
+        k = (x @ w[p + "attn.k_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        v = (x @ w[p + "attn.v_proj.weight"].T).reshape(s, c["kv_heads"], c["head_dim"])
+        r = h + P.attention(q, k, v).reshape(s, -1) @ w[p + "attn.o_proj.weight"].T
+        h = r + P.swiglu_mlp(P.rms_norm(r, w[p + "n2.weight"], c["eps"]), w[p + "ff.gate_proj.weight"],
+                             w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+    return P.rms_norm(h, w["final.weight"], c["eps"]) @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_an_embedding_that_adds_learned_positions(tmp_path, dtype_name):
+    """The embedding part gets the step's context: one that adds a learned row per position (and ties the output
+    matrix to its table) is registered here and runs through the unchanged model, whole prompts, their tails
+    token by token and unequal batches on reused slots alike; without the positions the logits would not
+    depend on the order of the earlier tokens' positions at all, so a cut that got them wrong would show."""
+    register_learned_positions()
+    from rust_inference_amd.engine.replay import Replayer, engine_for_trace
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    from safetensors import safe_open
+    folder = write_random_model(str(tmp_path / "m"), LEARNED, seed=41, dtype=torch.float32, matrix_std=0.15)
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        w = {k: f.get_tensor(k).to(torch.float64).numpy() for k in f.keys()}
+    assert "embed.positions" in w and "head.weight" not in w
+    model = load_model(folder, {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name])
+    assert model.head.weight is model.embedding.table
+    rng = np.random.default_rng(42)
+    reqs = {f"r{i}": [int(x) for x in rng.integers(0, LEARNED["vocab_size"], n)] for i, n in enumerate([40, 5, 66, 33])}
+    # the positions matter: the same tokens one place later give other logits
+    moved = learned_plain(w, [reqs["r0"][0]] + reqs["r0"])[1:]
+    assert np.abs(moved - learned_plain(w, reqs["r0"])).max() > 1e-2
+    for what, steps in (("whole", plans.whole(reqs)), ("tail", plans.tail_one_by_one(reqs, 24)),
+                        ("batches", plans.unequal_batches([
+                            {k: (v, max(1, len(v) - 20)) for k, v in list(reqs.items())[:2]},
+                            {k: (v, max(1, len(v) - 30)) for k, v in list(reqs.items())[2:]}]))):
+        engine = engine_for_trace(model, plans.max_live_tokens(steps))
+        player, outs = Replayer(engine), {}
+        for s in steps:
+            logits = player.feed(s)
+            if logits is not None:
+                outs[s["step"]] = logits.cpu().numpy()
+        engine.cache.check_consistent()
+        got = plans.collect(steps, lambda i: outs[i], LEARNED["vocab_size"])
+        for rid, toks in reqs.items():
+            assert_logits_close(got[rid], learned_plain(w, toks), dtype_name, f"learned positions, {what}, {rid}")

@@ -124,3 +124,20 @@ def test_generation_with_penalty_and_temperature_is_seeded(model_dirs):
     b = model.generate(prompts, seed=3, **kw).tokens
     alone = model.generate(prompts[:1], seed=3, **kw).tokens
     assert a == b and alone[0] == a[0] and a != model.generate(prompts, seed=4, **kw).tokens
+
+
+def test_sequences_of_one_batch_sample_each_in_their_own_way(model_dirs):
+    """Per-request sampling parameters through the entry point: greedy, temperature, top-k with a penalty side
+    by side in one batch give each request the tokens it gets when the whole batch samples its way (float32:
+    a request's logits do not depend on its neighbours; its generator is seeded by its index either way)."""
+    from rust_inference_amd import Model
+    from rust_inference_amd.sampling import SamplingParams
+    model = Model.load(model_dirs["A"], dtype="float32", max_batch=4, max_seq_len=64)
+    prompts = [[1, 2, 3, 4], [9, 8], [5], [7, 7, 7]]
+    kinds = [SamplingParams(), SamplingParams(temperature=0.9, seed=3), SamplingParams(temperature=1.2, top_k=20, seed=3),
+             SamplingParams(temperature=0.9, top_p=0.9, repetition_penalty=1.3, seed=3)]
+    mixed = model.generate(prompts, max_new_tokens=8, sampling=kinds).tokens
+    for i, kind in enumerate(kinds):
+        alike = model.generate(prompts, max_new_tokens=8, sampling=[kind] * 4).tokens
+        assert mixed[i] == alike[i], f"request {i}"
+    assert mixed[0] == model.generate(prompts, max_new_tokens=8).tokens[0]
