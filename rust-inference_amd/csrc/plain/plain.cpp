@@ -158,8 +158,19 @@ extern "C" int ri_plain_sample(const float* logits, int vocab, const int32_t* hi
     struct Cand { int id; float v; };
     std::vector<Cand> cand((size_t)vocab);
     for (int i = 0; i < vocab; ++i) cand[i] = {i, row[i] / temperature};
-    // falling value, rising id among equals; the k largest by that order are the first k of the sorted list
-    std::sort(cand.begin(), cand.end(), [](const Cand& a, const Cand& b) { return a.v > b.v || (a.v == b.v && a.id < b.id); });
+    // falling value, rising id among equals; the k largest by that order are the first k of the sorted list.
+    // Values are compared as the reference compares them (f32::total_cmp, src/sampling.rs:96-101): by a key that
+    // orders every bit pattern, NaNs included (a positive NaN above +inf, a negative one below -inf, -0 below +0),
+    // so that the comparison is a strict weak ordering whatever the logits hold.
+    auto key = [](float v) {
+        int32_t b;
+        memcpy(&b, &v, sizeof b);
+        return b ^ (int32_t)((uint32_t)(b >> 31) >> 1);
+    };
+    std::sort(cand.begin(), cand.end(), [&key](const Cand& a, const Cand& b) {
+        const int32_t ka = key(a.v), kb = key(b.v);
+        return ka > kb || (ka == kb && a.id < b.id);
+    });
     if (top_k > 0 && top_k < vocab) cand.resize((size_t)top_k);
     std::vector<float> probs(cand.size());
     float total = 0.f;

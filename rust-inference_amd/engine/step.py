@@ -125,6 +125,7 @@ class Engine:
         self._staging = None
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}       # in order of last use
         self.max_graphs = MAX_GRAPHS
+        self.keep_graphs = False     # keep what was captured beside what is replayed, so that its nodes can be counted
 
     def _stage(self, n: int) -> _Staging:
         if self._staging is None or self._staging.capacity < n:
@@ -236,7 +237,7 @@ class Engine:
         self.model.forward(ctx, self.cache)
         self.cache.restore_state(saved)
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
+        graph = torch.cuda.CUDAGraph(keep_graph=True) if self.keep_graphs else torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             dg.logits = self.model.forward(ctx, self.cache)
         dg.graph, dg.ctx = graph, ctx
@@ -281,6 +282,33 @@ class Engine:
         dg.graph.replay()
         cache.commit(slots, ones)
         return dg.logits
+
+    def graph_launches(self) -> dict:
+        """``{(batch, bound): kernel nodes}`` of the captured decode steps: the launches a step of that size
+        costs.  Only for graphs captured while ``keep_graphs`` was set (measurement)."""
+        import ctypes
+        hip = ctypes.CDLL("libamdhip64.so")
+        out = {}
+        for key, dg in self._graphs.items():
+            raw = getattr(dg.graph, "raw_cuda_graph", None) if dg.graph is not None else None
+            try:
+                handle = ctypes.c_void_p(raw()) if raw else None
+            except RuntimeError:                 # captured without keep_graphs
+                handle = None
+            if not handle:
+                continue
+            n = ctypes.c_size_t(0)
+            if hip.hipGraphGetNodes(handle, None, ctypes.byref(n)) != 0:
+                continue
+            nodes = (ctypes.c_void_p * n.value)()
+            hip.hipGraphGetNodes(handle, nodes, ctypes.byref(n))
+            kernels = 0
+            for node in nodes:
+                kind = ctypes.c_int(-1)
+                if hip.hipGraphNodeGetType(ctypes.c_void_p(node), ctypes.byref(kind)) == 0 and kind.value == 0:
+                    kernels += 1                 # hipGraphNodeTypeKernel
+            out[key] = kernels
+        return out
 
     def decode_on_device(self, slots: Sequence[int], ids_dev: torch.Tensor) -> torch.Tensor | None:
         """A decode step (one token per sequence, logits of every one) whose tokens are int32 ids on the device,

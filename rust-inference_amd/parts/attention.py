@@ -15,12 +15,9 @@ from .registry import build_part, register_part
 from .spec import PartSpec
 
 
-# Up to this many sequences a decode step norms and rotates q and k inside the attention kernel (one
-# launch less per layer); beyond it the many workgroups each repeating that work cost more than the
-# launch (measured at 64 sequences of 2,048 tokens: 140 us against 111 + 6 us; at 24 and 32 sequences the
-# one kernel is still ahead, by 1% of the step).  Steps that the attention takes with its streaming kernel
-# (a workgroup per run of a sequence's pages: ops.decode_attention_streams) repeat little of it and are
-# fused at any size.
+# Up to this many sequences a decode step norms and rotates q and k inside the attention kernel (one launch
+# less per layer); beyond it the many workgroups each repeating that work cost more than the launch.  Steps
+# that the attention takes with its streaming kernel repeat little of it and are fused at any size.
 FUSED_DECODE_MAX_SEQS = 32
 
 

@@ -15,71 +15,28 @@ def _wide_plan(n: int, k: int, swiglu: bool) -> tuple[int, int]:
     """``ops.wide_product_plan``, asked once per matrix size."""
     return ops.wide_product_plan(n, k, swiglu)
 
-# Which product kernel runs, by the number of rows of x (measured on MI355X at Qwen3-8B sizes with the
-# weights streamed from HBM through non-temporal loads, every variant replayed as a graph):
-#   1 row      one wavefront per weight row (gemv_bf16): 5.6 to 5.7 TB/s on the large matrices, 7.0 on the
-#              output head.  (At two rows the packed kernel is ahead: 471 against 438 tok/s for the model;
-#              at one row it is behind, a decode step of 3.19 ms against 3.12.)
-#   2-16 rows  the matrix-core kernel on weights packed into MFMA tiles ahead of time, where a part asked for
-#              the packed copy; it hands its rows to the next packed product in the operand's order
-#              (ops.TiledRows) and does the norms around it.  Where there is no packed copy the vendor
-#              library's product is used (the rule is at PACKED_MAX_BYTES below).
-#   17-64      the same kernel with two or four tiles of x, on small matrices only (MID_MAX_BYTES below).
+# Which product kernel runs, by the number of rows of x (bfloat16; the measurements behind every constant
+# here are written up with the design notes, under "Which product kernel serves which step"):
+#   1 row      one wavefront per weight row (ops.gemv_bf16).
+#   2-16 rows  the matrix-core kernel on weights packed into MFMA tiles ahead of time, where a part asked for the
+#              packed copy (the rule is _packed_pays below); it hands its rows to the next packed product in the
+#              operand's order (ops.TiledRows) and does the norms around it.
+#   17-64      the wide kernel (tiles of x shared through LDS) where the reader adds stretches of K or the
+#              gate|up pairs fill the machine; the packed kernel with two or four tiles of x on small matrices
+#              and up to 32 rows of tiled x; else the library.
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
-#              Beating it on large matrices at 17 rows and more takes its own design: x staged through LDS,
-#              persistent workgroups.  Tried and dropped here: workgroups that own four row tiles and all
-#              tiles of x, with K cut into parts for the narrow matrices (at 64 rows: down 36 us against 39
-#              us, o 20 against 15, gate|up 80 against 52); x through a piece of LDS of each wavefront's
-#              own, fetched in whole cache lines (faster at 16 rows, slower at 4 and 8 and on short K).
 GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
-# 17 to 64 rows: the packed kernel with two or four tiles of x to every weight tile.  With x in plain rows,
-# which every workgroup fetches from the L2 cache sixteen half cache lines a load, it beats the library on
-# small matrices only (at 32 rows, 4096 x 1024: 5.5 us against 9.8; 6144 x 4096: 23.6 against 15.1).  With
-# x in tiles (whoever makes the rows makes them so when the product asks) it is level or ahead on the large
-# ones too up to 32 rows (Qwen3-8B sizes at 32 rows, us: q|k|v 16.6 : 16.1, o 10.9 : 13.0, gate|up 40.2 : 51.0
-# + 5 for the activation, down 28.3 : 28.5; 5120 x 25600: 97 : 146; the model's decode step at 24 and 32
-# sequences is 5% and 7% shorter).  From 33 rows on it is not: q|k|v 23.2 : 18.0, and gate|up, level alone
-# with the activation counted (51.8 : 51.8 + 5), made the step at 48 sequences 1% longer.  (These figures are
-# from before the kernel kept its loads in flight as a ring; with the ring the step at 17, 24 and 32 sequences
-# became 9, 4 and 3% shorter again, and q|k|v on it at 33, 48 and 64 rows still makes the step 2 to 3% longer
-# than the library does.)
 MID_MAX_ROWS = 64
-MID_MAX_BYTES = 20_000_000
-MID_TILED_ROWS = 32
-# 17 to 64 rows against a matrix whose result goes into the residual stream (`o`, `down`): the wide kernel
-# (ops.gemm_wide_packed_bf16: three or four row tiles a workgroup, the tiles of x shared through LDS) with K cut
-# into stretches that the next norm adds up.  Measured at Qwen3-8B sizes as graphs, in us, against the library
-# and the kernel above: 4096 x 12288 at 64 rows 26.0 : 38.8 : 38.6, at 32 rows 23.0 : 29.0 : 29.2.  4096 x 4096
-# takes 14 us against the library's 18 inside the model (alone, over a few copies of the matrix that the
-# memory-side cache holds, the library needs 12.5: such small matrices have to be timed in the model).  In the
-# model, with gate|up on it too (below) and the kernel above for q|k|v up to 32 rows, a decode step of 17, 24,
-# 32, 48 and 64 sequences takes 4.90, 5.31, 5.79, 7.23 and 8.10 ms, where the kernel above alone (to 32 rows)
-# and the library (beyond) took 5.10, 5.50, 5.98, 7.76 and 8.53.  A product whose reader cannot add stretches
-# (q|k|v: 6144 x 4096, with a kernel of its own to add them 22 us against 15 to 18) stays with the kernel above
-# or the library.
-WIDE_MIN_K = 4096
+MID_MAX_BYTES = 20_000_000       # up to this size the packed kernel beats the library at 17 to 64 plain rows
+MID_TILED_ROWS = 32              # and up to this many rows on any matrix when the rows come tiled
+WIDE_MIN_K = 4096                # rows shorter than this leave the wide kernel's stretches too little to do
 WIDE_MIN_ROWS = 17
-# The gate|up pair at 17 to 64 rows goes to the wide kernel where workgroups of three or four wavefronts with K
-# whole fill at least this share of the compute units' rounds (12288 pairs of rows: 256 workgroups of three,
-# at 64 rows 45 us against the library's 48 + 5 for the activation, at 48 rows 40 against 50; with groups of
-# four, 192 workgroups, it only drew level).  What bounds it then is what a compute unit can pull through its
-# vector memory path, about 30 GB/s whether the bytes come from memory or from the L2 cache: its share of the
-# weights plus all of x once.
-WIDE_GATED_FILL = 0.9
-SPLIT_K = 4096
-# Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation
-# rides in the kernel).  Measured at 8 rows, packed kernel against library, in us:
-#   4096 x 1024 (8 MB) 4.1 : 7.5     1024 x 3072 (6 MB) 7.0 : 11.9    2048 x 2048 (8 MB) 5.3 : 11.0
-#   4096 x 4096 (34 MB) 9.2 : 15.3   6144 x 4096 (50 MB) 15.4 : 15.5  2560 x 9728 (50 MB) 19.2 : 18.3
-#   4096 x 12288 (101 MB) 22.5 : 21.3   5120 x 8192 (84 MB) 27.3 : 19.5   10240 x 5120 (105 MB) 29.7 : 24.3
-#   5120 x 25600 (262 MB) 85 : 135, and 65 with K cut into four parts
-# A product of this library's own also does the norms next to it (about 6 us each at these sizes) when its
-# neighbours are its own too, so a draw goes to the packed kernel: with q|k|v and down on it a decode step
-# of 8 sequences at Qwen3-8B sizes has no norm kernel left and is 3% shorter.  The kernel is a workgroup per
-# 16 rows of the matrix, and what it loses by is a last round of workgroups that leaves most compute units
-# idle (5120 rows: 320 workgroups on 256 compute units); cutting K into parts fills the round, but the parts
-# cannot add themselves into the residual stream, so only rows of 16,384 elements and more are cut.
+WIDE_GATED_FILL = 0.9            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds
+SPLIT_K = 4096                   # pieces of a long K (PACKED_LONG_K and more) whose sums the next norm adds
+# Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation rides in
+# the kernel): up to 40 MB always; up to PACKED_MAX_BYTES unless the last round of workgroups (one per 16 rows)
+# would leave most compute units idle; rows of PACKED_LONG_K elements and more always, cut into parts.
 PACKED_MAX_BYTES = 101_000_000
 PACKED_LONG_K = 16384
 

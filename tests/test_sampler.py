@@ -62,3 +62,22 @@ def test_same_tokens_as_the_plain_sampler(params):
         a, b = ours.sample(logits, history), plain.sample(logits, history)
         assert a == b
         history.append(a)
+
+
+def test_logits_that_are_not_numbers_are_ordered_like_the_reference_orders_them():
+    """The candidates are sorted by a total order over every bit pattern (f32::total_cmp in the reference,
+    src/sampling.rs:96-101): a row with NaNs, infinities and both zeros is sorted without a fault (the
+    sanitized build runs the same code), the same way every time, and top-k 1 takes what that order puts first:
+    a positive NaN, which stands above +inf."""
+    rng = np.random.default_rng(8)
+    row = (2.0 * rng.normal(size=4096)).astype(np.float32)
+    row[::7] = np.nan
+    row[5::11] = -np.nan
+    row[3], row[100], row[200], row[201] = np.inf, -np.inf, 0.0, -0.0
+    s = HostSampler(SamplingParams(temperature=1.0, top_k=1, seed=2))
+    assert {s.sample(row) for _ in range(5)} == {0}                      # index 0: the first positive NaN
+    clean = np.where(np.isnan(row), np.float32(-1e30), row)
+    clean[3] = 50.0
+    t = HostSampler(SamplingParams(temperature=1.0, top_k=3, seed=2))
+    picks = [t.sample(clean) for _ in range(50)]
+    assert set(picks) == {3}                                             # e^(x - 50) of the others rounds to nothing
