@@ -48,7 +48,8 @@ def test_argmax_static_matches_argmax_on_two_calls_in_a_row():
         assert rc == 0, lib.ri_last_error().decode()
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated(dev) == before
-        assert free_bytes() == free_before, "the driver's free memory changed across the call"
+        # (the workspace this entry point spares is half a megabyte: an allocation of it could not hide in less)
+        assert free_before - free_bytes() < 256 * 1024, "the driver's free memory shrank across the call"
         assert torch.equal(got, want), (rows, vocab)
         assert got[1].item() == 7
         assert torch.equal(got.cpu().long(), logits.cpu().argmax(1))
