@@ -164,6 +164,131 @@ def sanitizer_runtime() -> str:
     raise KernelError("the address sanitizer's runtime library was not found beside the compiler")
 
 
+# ---- the kernels on the CPU
+EMU_LIB_NAME = "libri_emulated.so"
+EMU_SRC = os.path.join(CSRC, "emu")
+
+
+def _rewrite_launches(text: str) -> str:
+    """``kernel<...><<<grid, block, shared, stream>>>(args)`` as ``RI_EMU_LAUNCH(kernel<...>, grid, block,
+    shared, stream, args)`` and ``extern __shared__ T name[];`` as a pointer to the workgroup's dynamic shared
+    memory: what the CPU stand-in of the HIP runtime (csrc/emu) takes instead."""
+    import re
+
+    def matching(s: str, at: int, open_ch: str, close_ch: str, step: int) -> int:
+        depth, i = 0, at
+        while 0 <= i < len(s):
+            if s[i] == (open_ch if step > 0 else close_ch):
+                depth += 1
+            elif s[i] == (close_ch if step > 0 else open_ch):
+                depth -= 1
+                if depth == 0:
+                    return i
+            i += step
+        raise KernelError("unbalanced brackets around a kernel launch")
+
+    def split_top(s: str) -> list[str]:
+        parts, depth, start = [], 0, 0
+        for i, ch in enumerate(s):
+            if ch in "([{":
+                depth += 1
+            elif ch in ")]}":
+                depth -= 1
+            elif ch == "," and depth == 0:
+                parts.append(s[start:i])
+                start = i + 1
+        parts.append(s[start:])
+        return [p.strip() for p in parts]
+
+    out, pos = [], 0
+    while True:
+        at = text.find("<<<", pos)
+        if at < 0:
+            out.append(text[pos:])
+            break
+        # the kernel's name, with its template arguments if it has any, stands right before
+        begin = at
+        if text[begin - 1] == ">":
+            begin = matching(text, begin - 1, "<", ">", -1)
+        while begin > 0 and (text[begin - 1].isalnum() or text[begin - 1] in "_:"):
+            begin -= 1
+        close = text.index(">>>", at)
+        config = split_top(text[at + 3:close].replace("\\\n", " "))
+        while len(config) < 4:
+            config.append("0")
+        lpar = close + 3
+        while text[lpar] in " \\\n\t":
+            lpar += 1
+        if text[lpar] != "(":
+            raise KernelError("a kernel launch without arguments")
+        rpar = matching(text, lpar, "(", ")", 1)
+        kernel = text[begin:at].strip()
+        args = text[lpar + 1:rpar]
+        out.append(text[pos:begin])
+        out.append(f"RI_EMU_LAUNCH(({kernel}), {config[0]}, {config[1]}, {config[2]}, {config[3]}"
+                   + (", " + args if args.strip() else "") + ")")
+        pos = rpar + 1
+    text = "".join(out)
+    return re.sub(r"extern\s+__shared__\s+(\w+)\s+(\w+)\[\];", r"\1* \2 = (\1*)emu::dyn_shared();", text)
+
+
+def build_emulated(out_dir: str, patches: dict | None = None) -> str:
+    """Every kernel source built for the CPU over a stand-in for the HIP runtime (csrc/emu): a workgroup's threads
+    run as coroutines that meet at barriers and at every exchange between a wavefront's lanes, so the kernels
+    compute what they compute on the GPU, from buffers that the tests lay between guard pages: a load or store
+    outside its buffer ends the process with a report.  No GPU is needed.  ``patches``: ``{file: (old, new)}``
+    text replacements applied to the copies that are compiled (a test puts a mistake back in to see it caught)."""
+    clang = None
+    for cand in ("/opt/rocm/llvm/bin/clang++", "/opt/rocm/lib/llvm/bin/clang++", shutil.which("clang++")):
+        if cand and os.path.exists(cand):
+            clang = cand
+            break
+    if clang is None:
+        raise KernelError("no clang++ for the CPU build of the kernels")
+    os.makedirs(out_dir, exist_ok=True)
+    lib_path = os.path.join(out_dir, EMU_LIB_NAME)
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())
+    gen = os.path.join(out_dir, "emu_src")
+    os.makedirs(gen, exist_ok=True)
+    for name in os.listdir(CSRC):
+        if name.endswith(".h"):
+            shutil.copy(os.path.join(CSRC, name), os.path.join(gen, name))
+    objs = []
+    jobs = []
+    for src in sources():
+        name = os.path.basename(src)
+        with open(src) as f:
+            text = f.read()
+        if patches and name in patches:
+            old, new = patches[name]
+            if old not in text:
+                raise KernelError(f"{name} does not hold the text to be patched")
+            text = text.replace(old, new)
+        cpp = os.path.join(gen, name + ".cpp")
+        with open(cpp, "w") as f:
+            f.write(_rewrite_launches(text))
+        obj = cpp + ".o"
+        objs.append(obj)
+        flags = [f for f in FILE_FLAGS.get(name, [])]
+        jobs.append([clang, "-O1", "-g", "-std=c++17", "-fPIC", "-w", "-I", EMU_SRC, "-I", gen, *flags, "-c", cpp, "-o", obj])
+    emu_obj = os.path.join(gen, "emu.o")
+    jobs.append([clang, "-O1", "-g", "-std=c++17", "-fPIC", "-w", "-I", EMU_SRC, "-c", os.path.join(EMU_SRC, "emu.cpp"),
+                 "-o", emu_obj])
+
+    def one(cmd):
+        proc = subprocess.run(cmd, capture_output=True, text=True, env=env)
+        if proc.returncode != 0:
+            raise KernelError(f"the CPU build of {os.path.basename(cmd[-3])} failed:\n{proc.stderr[-6000:]}")
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        list(pool.map(one, jobs))
+    proc = subprocess.run([clang, "-shared", "-fPIC", *objs, emu_obj, "-o", lib_path], capture_output=True, text=True, env=env)
+    if proc.returncode != 0:
+        raise KernelError(f"linking {EMU_LIB_NAME} failed:\n{proc.stderr[-4000:]}")
+    return lib_path
+
+
 PLAIN_LIB_NAME = "libri_plain.so"
 PLAIN_SRC = os.path.join(CSRC, "plain")
 _plain = None

@@ -1,0 +1,75 @@
+"""The kernels without a GPU: every kernel source compiled for the CPU (kernels/build.py: build_emulated; a
+workgroup's threads are coroutines that meet at barriers and at every exchange between the lanes of a wavefront,
+the matrix-core product included) and run by the kernel tests themselves, tests/test_kernels_gpu.py, with every
+operand and every buffer the wrappers allocate between two guard pages.  The kernels keep their loads out of
+branches and issue them whatever the indices are, from addresses pulled back inside the data: here an address
+that was not pulled back far enough touches a guard page and ends the run with a report that names the kernel,
+the workgroup, the thread and the buffer.  The sizes are the GPU tests' own except the largest (the emulation
+runs a few thousand matrix instructions a second)."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HERE = os.path.join(ROOT, "tests")
+
+# What stays out: matrices of 4,096 and more rows or columns, and contexts of thousands of keys (minutes each
+# when emulated); every kernel and every form of it is still run, at the smaller sizes of the same tests.
+SELECT = ("not 4096 and not 12288 and not 5120 and not 5000 and not very_long and not more_pages_than "
+          "and not thousands and not many_sequences and not in_runs")
+
+
+def _run(args, env_extra=None, timeout=1500):
+    env = dict(os.environ, RI_TEST_KERNELS="emulated", **(env_extra or {}))
+    env.pop("RI_KERNEL_LIBRARY", None)
+    return subprocess.run([sys.executable, *args], capture_output=True, text=True, env=env, cwd=ROOT, timeout=timeout)
+
+
+def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages():
+    from rust_inference_amd.errors import KernelError
+    try:
+        sys.path.insert(0, HERE)
+        import emulated
+        emulated.library()
+    except KernelError as e:
+        pytest.skip(f"no CPU build of the kernels here: {e}")
+    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", os.path.join(HERE, "test_kernels_gpu.py"), "-k", SELECT])
+    assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-3000:]
+    assert " passed" in run.stdout and "[emu]" not in run.stderr
+
+
+# The product for 17 to 64 rows once read a tile of x that its buffer does not have (33 to 48 rows are three
+# tiles of 16 and run with code built for four; the loads that are issued whatever the indices are read the
+# fourth): a kilobyte per step past the end of the buffer, which on the GPU faulted once in many runs.  The
+# address is pulled back to the last tile now; with the old expression put back the emulated run must end at
+# the guard page and say where.
+OLD_MID = {"gemm_skinny_bf16.hip": ("min(rt, (M - 1) >> 4)", "rt")}
+PROBE = """
+import sys
+sys.path.insert(0, {here!r})
+import torch, emulated
+ops = emulated.ops(patches={patches!r})
+m, n, k = 40, 48, 1024
+w = (torch.randn(n, k) * 0.1).bfloat16()
+x = ops.TiledRows.empty(m, k, "cpu")
+x.data.zero_()
+ops.gemm_mid_packed_bf16(x, emulated.tensor(ops.pack_for_mfma(w), "packed weights"), n, torch.float32)
+print("no access outside a buffer")
+"""
+
+
+def test_a_load_that_leaves_its_buffer_is_caught_and_named():
+    from rust_inference_amd.errors import KernelError
+    try:
+        sys.path.insert(0, HERE)
+        import emulated
+        emulated.library(OLD_MID)
+    except KernelError as e:
+        pytest.skip(f"no CPU build of the kernels here: {e}")
+    bad = _run(["-c", PROBE.format(here=HERE, patches=OLD_MID)])
+    assert bad.returncode == 86, bad.stdout[-2000:] + bad.stderr[-2000:]
+    assert "gemm_mid_packed_kernel" in bad.stderr and "past the end of buffer" in bad.stderr
+    good = _run(["-c", PROBE.format(here=HERE, patches=None)])
+    assert good.returncode == 0 and "no access outside a buffer" in good.stdout, good.stdout[-2000:] + good.stderr[-2000:]

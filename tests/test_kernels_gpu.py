@@ -1,23 +1,41 @@
 """Each HIP kernel alone against its plain reference, at other sizes than the tiny models use.
-Where random inputs would hide a fault, the inputs are made so that it shows."""
+Where random inputs would hide a fault, the inputs are made so that it shows.
+
+The same tests run without a GPU when the environment says RI_TEST_KERNELS=emulated: then the kernels are the
+CPU build of the same sources (tests/emulated.py), every operand lies between guard pages, and a kernel that
+touches memory outside a buffer ends the run with a report.  tests/test_kernels_emulated.py starts that run."""
+import os
+
 import numpy as np
 import pytest
 import torch
 
 from plain import qwen3_plain as P
 
-pytestmark = pytest.mark.gpu
-DEV = "cuda:0"
+EMULATED = os.environ.get("RI_TEST_KERNELS") == "emulated"
+pytestmark = [] if EMULATED else pytest.mark.gpu
+DEV = "cpu" if EMULATED else "cuda:0"
 
 
 @pytest.fixture(scope="module")
 def ops():
+    if EMULATED:
+        import emulated
+        return emulated.ops()
     from rust_inference_amd.kernels import ops
     return ops
 
 
+def guarded(x):
+    """On the GPU the tensor itself; emulated, a copy between guard pages."""
+    if EMULATED:
+        import emulated
+        return emulated.tensor(x.contiguous(), "a test's operand")
+    return x
+
+
 def t(a, dtype=torch.float32):
-    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+    return guarded(torch.tensor(np.asarray(a), dtype=dtype, device=DEV))
 
 
 def f64(x):
@@ -27,6 +45,10 @@ def f64(x):
 def close(got, want, rel, what=""):
     want = np.asarray(want, dtype=np.float64)
     err = np.abs(f64(got) - want).max() / max(np.abs(want).max(), 1e-30)
+    report = os.environ.get("RI_TEST_ERROR_REPORT")          # a file that collects what every comparison measured
+    if report:
+        with open(report, "a") as f:
+            f.write(f"{os.environ.get('PYTEST_CURRENT_TEST', '?')}\t{what}\t{err:.3e}\t{rel:.0e}\n")
     assert err <= rel, f"{what}: error {err:.3e} of the largest value exceeds {rel:.0e}"
 
 
@@ -54,17 +76,17 @@ def test_add_rmsnorm(ops, dim, pending_dtype):
     gain = t(1 + 0.1 * rng.normal(size=dim))
     total = f64(res) + (0 if pend is None else f64(pend))
     want = P.rms_norm(total, f64(gain), 1e-5)
-    before = res.clone()
+    before = guarded(res.clone())
     out = ops.add_rmsnorm(res, pend, gain, 1e-5, torch.float32)
     close(out, want, 2e-6, "norm")
     close(res, total, 1e-7, "residual written back")
     # rows: the same sums for a few rows, nothing written back
-    res2 = before.clone()
+    res2 = guarded(before.clone())
     rows = t([5, 0, 5], torch.int32)
     out2 = ops.add_rmsnorm(res2, pend, gain, 1e-5, torch.bfloat16, rows)
     assert torch.equal(res2, before) and out2.dtype == torch.bfloat16
     close(out2, P.bf16_round(want[[5, 0, 5]].astype(np.float32)), 5e-3, "gathered rows")
-    close(ops.add_rows(before.clone(), pend, rows), total[[5, 0, 5]], 1e-7, "add_rows")
+    close(ops.add_rows(guarded(before.clone()), pend, rows), total[[5, 0, 5]], 1e-7, "add_rows")
 
 
 def test_add_rmsnorm_adds_the_parts_of_a_split_product(ops):
@@ -92,10 +114,10 @@ def test_the_norm_adds_any_number_of_parts_in_their_order(ops, n_parts, dim):
     res = t(rng.normal(size=(5, dim)))
     parts = t(rng.normal(size=(n_parts, 5, dim)))
     gain = t(1 + 0.1 * rng.normal(size=dim))
-    want_sum = res.clone()
+    want_sum = guarded(res.clone())
     for q in range(n_parts):
         want_sum += parts[q]
-    got = res.clone()
+    got = guarded(res.clone())
     out = ops.add_rmsnorm(got, parts, gain, 1e-6, torch.float32)
     assert torch.equal(got, want_sum)
     close(out, P.rms_norm(f64(want_sum), f64(gain), 1e-6), 2e-6, "norm over parts")
@@ -142,11 +164,11 @@ def test_add_rmsnorm_fused_equals_unfused_bit_for_bit(ops):
     # src/ops/norm.rs:84-98
     a, r = t([[0.5, -1.0, 2.0, 0.25]]), t([[1.0, 1.0, -1.0, 0.0]])
     w = t([1.0, 0.5, 2.0, 1.0])
-    res = r.clone()
+    res = guarded(r.clone())
     fused = ops.add_rmsnorm(res, a, w, 1e-6, torch.float32)
     plain_sum = (a + r).contiguous()
     assert torch.equal(res, plain_sum)
-    assert torch.equal(fused, ops.add_rmsnorm(plain_sum.clone(), None, w, 1e-6, torch.float32))
+    assert torch.equal(fused, ops.add_rmsnorm(guarded(plain_sum.clone()), None, w, 1e-6, torch.float32))
 
 
 def paged(rng, lens, hkv, dh, page_size=32, dtype=torch.float32, spare=3):
@@ -638,14 +660,14 @@ def test_products_linked_to_norms(ops, packed, m, hidden, k, inter):
     prep = (lambda w, **kw: ops.pack_for_mfma(w, **kw)) if packed else (lambda w, **kw: w)
 
     r1 = f64(r0) + f64(x) @ f64(w_out).T
-    residual = r0.clone()
+    residual = guarded(r0.clone())
     later = ops.linked_product(x, prep(w_out), hidden, packed, residual=residual, next_gain=gain, next_eps=eps)
     close(residual, r1, 3e-6, "residual after the linked product")
     close(later.xg, f64(residual) * f64(gain), 4e-3, "rows times gain")       # one rounding to bfloat16
     close(later.ssq.sum(1), (f64(residual) ** 2).sum(1), 1e-5, "sums of squares")
     assert later.dim == hidden and later.eps == eps
     # a second call leaves the same partial sums: they do not depend on scheduling
-    again = ops.linked_product(x, prep(w_out), hidden, packed, residual=r0.clone(), next_gain=gain, next_eps=eps)
+    again = ops.linked_product(x, prep(w_out), hidden, packed, residual=guarded(r0.clone()), next_gain=gain, next_eps=eps)
     assert torch.equal(again.ssq, later.ssq) and torch.equal(again.xg, later.xg)
 
     normed = P.rms_norm(f64(residual), f64(gain), eps)
@@ -691,8 +713,8 @@ def test_every_maker_of_rows_can_tile_them(ops, m, dim, n):
     residual = t(rng.normal(size=(m, dim)) * 2)
     pending = t(rng.normal(size=(m, dim)), torch.bfloat16)
     gain = t(1 + 0.2 * rng.normal(size=dim))
-    plain = ops.add_rmsnorm(residual.clone(), pending, gain, 1e-5, torch.bfloat16)
-    r2 = residual.clone()
+    plain = ops.add_rmsnorm(guarded(residual.clone()), pending, gain, 1e-5, torch.bfloat16)
+    r2 = guarded(residual.clone())
     tiled = ops.add_rmsnorm(r2, pending, gain, 1e-5, torch.bfloat16, tiled=True)
     assert isinstance(tiled, ops.TiledRows) and tiled.shape == (m, dim) and torch.equal(tiled.rows(), plain)
     close(r2, f64(residual) + f64(pending), 1e-6, "the sum is written back either way")
@@ -717,22 +739,22 @@ def test_streaming_attention_walks_a_run_of_more_pages_than_it_holds_table_entri
     that length, eight kv heads (512 runs: one a sequence and kv head), against the generic kernel on the same
     pages; the sequences are of unequal length and one key far back in one of them gets a score that stands out."""
     heads, kv_heads, dh, B = 8, 8, 32, 64
-    gen = torch.Generator(device="cuda").manual_seed(3)
+    gen = torch.Generator(device=DEV).manual_seed(3)
     lens = [33_000 + 37 * b for b in range(B)]
     lens[5] = 40_000
     pages_per = [-(-n // 32) for n in lens]
     width = max(pages_per)
     num_pages = sum(pages_per)
     assert ops.decode_attention_runs(B, kv_heads, max(lens)) == 1
-    kp = torch.randn((num_pages, kv_heads, 32, dh), device="cuda", generator=gen).to(torch.bfloat16)
-    vp = torch.randn((num_pages, kv_heads, dh, 32), device="cuda", generator=gen).to(torch.bfloat16)
-    order = torch.randperm(num_pages, device="cuda", generator=gen).to(torch.int32)
-    table = torch.zeros((B, width), dtype=torch.int32, device="cuda")
+    kp = torch.randn((num_pages, kv_heads, 32, dh), device=DEV, generator=gen).to(torch.bfloat16)
+    vp = torch.randn((num_pages, kv_heads, dh, 32), device=DEV, generator=gen).to(torch.bfloat16)
+    order = torch.randperm(num_pages, device=DEV, generator=gen).to(torch.int32)
+    table = torch.zeros((B, width), dtype=torch.int32, device=DEV)
     at = 0
     for b, n in enumerate(pages_per):
         table[b, :n] = order[at:at + n]
         at += n
-    qkv = torch.randn((B, (heads + 2 * kv_heads) * dh), device="cuda", generator=gen).to(torch.bfloat16)
+    qkv = torch.randn((B, (heads + 2 * kv_heads) * dh), device=DEV, generator=gen).to(torch.bfloat16)
     # Queries that are a multiple of one far key, so that the output is that key's value: a key among a
     # wavefront's first 256 pages (position 9,000 of sequence 5) and keys among its later ones (pages from 1,024
     # on: position 39,990 of sequence 5, a key of sequence 9's last pages and one of sequence 20's page 1,024)
@@ -805,7 +827,7 @@ def test_rows_in_the_matrix_cores_order(ops, m, hidden, k, inter):
     # a layer's chain of links: norm left to the products, rows handed on in either layout
     outs = []
     for tiles in (False, True):
-        residual = r0.clone()
+        residual = guarded(r0.clone())
         later = ops.linked_product(x, pw_a, hidden, True, residual=residual, next_gain=gain, next_eps=eps,
                                    tiled_out=tiles)
         assert isinstance(later.xg, ops.TiledRows) == tiles
@@ -847,8 +869,9 @@ def test_argmax(ops):
 
 def test_kernels_refuse_what_they_cannot_do(ops):
     from rust_inference_amd.errors import KernelError, ShapeError
-    with pytest.raises(KernelError, match="GPU only"):
-        ops.swiglu(torch.zeros(2, 4))
+    if not EMULATED:
+        with pytest.raises(KernelError, match="GPU only"):
+            ops.swiglu(torch.zeros(2, 4))
     with pytest.raises(KernelError, match="1 to 8"):
         ops.gemv_bf16(torch.zeros(9, 16, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 16, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(KernelError, match="between 1 and 512"):
