@@ -929,7 +929,9 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 // the step 2% shorter, 4 of them 2%, one sequence of 131,000 keys in 64 runs 10%.  Fewer or shorter streams
 // do not keep the memory busy (one sequence of 131,000 keys in 16 runs: 12% longer; runs of four chunks: no
 // gain), and runs that need a join lose at a few thousand keys (2 runs at 48 sequences of 2,080 keys: -2.5%;
-// 4 runs at 16 sequences of 4,100: -1.5%; 32 sequences of 4,100 gain 2.5% and are left to the chunks with them).
+// 4 runs at 16 sequences of 4,100: -1.5%; 32 sequences of 4,100 gain 2.5% and are left to the chunks with them;
+// one run a sequence at 16 sequences of 16 to 1,300 keys, 128 workgroups and no join: 7% of a small model's step
+// longer than the chunks with their join).
 // (The counts of workgroups above were measured on 256 compute units and are kept per compute unit: two of
 // them for each to stream at all, four for each where runs are joined.)
 #define STREAM_WORKGROUPS_PER_CU 4

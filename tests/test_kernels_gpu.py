@@ -26,6 +26,17 @@ def ops():
     return ops
 
 
+@pytest.fixture(autouse=True)
+def _guarded_buffers_go_back():
+    """Emulated: what a test laid between guard pages is unmapped when it ends (a later touch of it would fault)."""
+    yield
+    if EMULATED:
+        import gc
+        import emulated
+        gc.collect()
+        emulated.free_all()
+
+
 def guarded(x):
     """On the GPU the tensor itself; emulated, a copy between guard pages."""
     if EMULATED:
