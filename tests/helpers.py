@@ -52,4 +52,8 @@ BF16_BOUND = 3e-2
 def assert_logits_close(got, want, dtype_name, what=""):
     bound = F32_BOUND if dtype_name == "float32" else BF16_BOUND
     err = rel_to_max(got, want)
+    report = os.environ.get("RI_TEST_ERROR_REPORT")          # a file that collects what every comparison measured
+    if report:
+        with open(report, "a") as f:
+            f.write(f"{os.environ.get('PYTEST_CURRENT_TEST', '?')}\t{what}\t{err:.3e}\t{bound:.0e}\n")
     assert err <= bound, f"{what}: error {err:.3e} of the largest logit exceeds {bound:.0e} ({dtype_name})"

@@ -53,6 +53,18 @@ def f64(x):
     return x.detach().to("cpu", torch.float64).numpy()
 
 
+# What a kernel that hands out bfloat16 is held to, from what the comparisons below measured on an MI355X (every
+# comparison can write what it measures into the file RI_TEST_ERROR_REPORT names): a bfloat16 result is rounded once
+# at the end, half a unit of its last place, which is up to 3.9e-3 of its own size; the attention kernels, the norms
+# with rotation and the products with bfloat16 out measure 2.2e-3 to 3.8e-3 of the largest value, and are held to
+# twice that.  Where the result went through two such roundings (the fused decode attention reads the key it has just
+# rounded; a linked gate|up product rounds its normed input and its result) 4.2e-3 to 4.7e-3 was measured.  Where the
+# wanted result is one value row picked out by a score that stands out, rounding hardly shows: 2.8e-4 measured.
+BF16_OUT = 7.5e-3
+BF16_TWICE = 9.5e-3
+BF16_ONE_KEY = 6e-4
+
+
 def close(got, want, rel, what=""):
     want = np.asarray(want, dtype=np.float64)
     err = np.abs(f64(got) - want).max() / max(np.abs(want).max(), 1e-30)
@@ -203,7 +215,7 @@ def paged(rng, lens, hkv, dh, page_size=32, dtype=torch.float32, spare=3):
 
 
 @pytest.mark.parametrize("paged_values", [False, True])
-@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, BF16_OUT)])
 @pytest.mark.parametrize("heads, kv_heads, dh", [(6, 2, 48), (4, 4, 128), (9, 1, 16), (2, 1, 256), (5, 5, 64), (8, 2, 32),
                                                  (4, 2, 8), (6, 3, 24), (3, 1, 40), (2, 2, 2), (2, 1, 328), (4, 2, 512)])
 def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh, paged_values):
@@ -247,7 +259,7 @@ def test_qk_norm_rope_kv_write(ops, dtype, rel, heads, kv_heads, dh, paged_value
     assert np.array_equal(f64(qkv2), qkv)
 
 
-@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, BF16_OUT)])
 @pytest.mark.parametrize("dh, rot", [(64, 16), (48, 24), (40, 8), (7, 4), (9, 0), (130, 128), (512, 64)])
 def test_rotation_over_part_of_the_head(ops, dtype, rel, dh, rot):
     """The first `rot` elements of a head are rotated in pairs (i, i + rot/2) by frequencies of their own, the rest
@@ -319,7 +331,7 @@ def attention_case(ops, rng, lens, new, heads, kv_heads, dh, dtype, window=None,
     return out.reshape(tokens, heads, dh), want
 
 
-@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("dtype, rel", [(torch.float32, 3e-6), (torch.bfloat16, BF16_OUT)])
 @pytest.mark.parametrize("heads, kv_heads, dh", [(4, 2, 16), (6, 2, 48), (8, 1, 128), (3, 3, 64), (9, 1, 32),
                                                  # any head size: the reference's own attention test runs 8
                                                  # (src/attention.rs:189-219); odd ones; beyond 256
@@ -342,7 +354,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
             kf = f64(kp[table[0, far // 32].item(), 0, far % 32])
             qkv[0, dh:2 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
         out, want = attention_case(ops, rng, [700], [1], heads, kv_heads, dh, dtype, boost=boost)
-        close(out, want, 3e-6 if dtype == torch.float32 else 1e-2, f"far key {far}")
+        close(out, want, 3e-6 if dtype == torch.float32 else BF16_ONE_KEY, f"far key {far}")
         # and the plain result really is that one value (the test is not vacuous)
         assert np.abs(want[0, 1]).max() > 0
 
@@ -352,7 +364,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
 def test_attention_window_edges(ops, dtype, window):
     rng = np.random.default_rng(window)
     out, want = attention_case(ops, rng, [290, 40], [34, 40], 4, 2, 32, dtype, window=window)
-    close(out, want, 3e-6 if dtype == torch.float32 else 1e-2, f"window {window}")
+    close(out, want, 3e-6 if dtype == torch.float32 else BF16_OUT, f"window {window}")
 
 
 MFMA_SHAPES = [(4, 1, 32), (8, 2, 32), (6, 2, 64), (3, 3, 64), (32, 8, 128), (16, 1, 128), (5, 5, 128)]
@@ -365,7 +377,7 @@ def test_mfma_prefill_attention(ops, heads, kv_heads, dh):
     # continue sequences already in the cache, all in one call
     out, want = attention_case(ops, rng, [70, 300, 257, 1, 45, 131], [70, 5, 1, 1, 45, 99], heads, kv_heads, dh,
                                torch.bfloat16, kernel="prefill")
-    close(out, want, 1e-2, "prefill attention on the matrix cores")
+    close(out, want, BF16_OUT, "prefill attention on the matrix cores")
 
 
 @pytest.mark.parametrize("heads, kv_heads, dh", MFMA_SHAPES)
@@ -374,7 +386,7 @@ def test_mfma_decode_attention(ops, heads, kv_heads, dh):
     # lengths at and around page and chunk edges: 1, 32, 33, 256, 257, 512, 700
     lens = [1, 32, 33, 256, 257, 512, 700, 5]
     out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, kernel="decode")
-    close(out, want, 1e-2, "decode attention on the matrix cores")
+    close(out, want, BF16_OUT, "decode attention on the matrix cores")
 
 
 @pytest.mark.parametrize("window", [None, 4500])
@@ -391,7 +403,7 @@ def test_mfma_decode_attention_over_thousands_of_keys(ops, window):
             qkv[2, dh:2 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
         out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16,
                                    window=window, boost=boost, kernel="decode")
-        close(out, want, 1e-2, f"far key {far}, window {window}")
+        close(out, want, BF16_OUT, f"far key {far}, window {window}")
 
 
 @pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 100), (16, 8, 32, 300),
@@ -410,7 +422,7 @@ def test_mfma_decode_attention_streams_over_many_sequences(ops, heads, kv_heads,
         qkv[9, head * dh:(head + 1) * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
     out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, window=window,
                                boost=boost, kernel="decode")
-    close(out, want, 1e-2, f"streaming decode attention, window {window}")
+    close(out, want, BF16_OUT, f"streaming decode attention, window {window}")
 
 
 @pytest.mark.parametrize("window", [None, 4500])
@@ -429,7 +441,7 @@ def test_mfma_decode_attention_streams_long_sequences_in_runs(ops, window):
             qkv[0, 5 * dh:6 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
         out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16,
                                    window=window, boost=boost, kernel="decode")
-        close(out, want, 1e-2, f"far key {far}, window {window}")
+        close(out, want, BF16_OUT, f"far key {far}, window {window}")
 
 
 def test_mfma_decode_attention_streams_one_very_long_sequence(ops):
@@ -447,7 +459,7 @@ def test_mfma_decode_attention_streams_one_very_long_sequence(ops):
             qkv[0, 2 * dh:3 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
         out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, boost=boost,
                                    kernel="decode")
-        close(out, want, 1e-2, f"far key {far}")
+        close(out, want, BF16_OUT, f"far key {far}")
         assert np.abs(want[0, 2]).max() > 0
 
 
@@ -461,7 +473,7 @@ def test_mfma_attention_finds_one_far_key(ops, kernel):
             qkv[0, 6 * dh:7 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
         out, want = attention_case(ops, rng, [700], [1], heads, kv_heads, dh, torch.bfloat16, boost=boost,
                                    kernel=kernel)
-        close(out, want, 1e-2, f"far key {far}")
+        close(out, want, BF16_ONE_KEY, f"far key {far}")
         vfar = f64(out[0, 6])
         assert np.abs(vfar - want[0, 6]).max() < 0.05
 
@@ -472,7 +484,7 @@ def test_mfma_attention_window_edges(ops, kernel, window):
     rng = np.random.default_rng(window + 5)
     new = [1, 1] if kernel == "decode" else [34, 40]
     out, want = attention_case(ops, rng, [290, 40], new, 4, 2, 64, torch.bfloat16, window=window, kernel=kernel)
-    close(out, want, 1e-2, f"window {window}")
+    close(out, want, BF16_OUT, f"window {window}")
 
 
 @pytest.mark.parametrize("heads, kv_heads, dh", MFMA_SHAPES)
@@ -529,12 +541,12 @@ def fused_decode_case(ops, heads, kv_heads, dh, window, lens, steps=2, repeats=2
             tab = table.cpu().numpy()
             for b in range(B):
                 page, off = tab[b, pos[b] // 32], pos[b] % 32
-                close(kp[page, :, off], kn[b], 1e-2, "the new key in its page")
+                close(kp[page, :, off], kn[b], BF16_OUT, "the new key in its page")
                 assert np.array_equal(f64(vp[page, :, :, off]), vn[b]), "the new value in its page"
                 kb = np.stack([f64(kp[tab[b, p // 32], :, p % 32]) for p in range(cur[b])])
                 vb = np.stack([f64(vp[tab[b, p // 32], :, :, p % 32]) for p in range(cur[b])])
                 want = P.attention(q[b:b + 1], kb, vb, window=window)
-                close(out[b].reshape(1, heads, dh), want, 1e-2, f"sequence {b}, step {step}, repeat {repeat}")
+                close(out[b].reshape(1, heads, dh), want, BF16_TWICE, f"sequence {b}, step {step}, repeat {repeat}")
 
 
 def test_mfma_and_generic_attention_agree(ops):
@@ -686,7 +698,7 @@ def test_products_linked_to_norms(ops, packed, m, hidden, k, inter):
           "product that finishes the norm")
     y = normed @ f64(w_gu).T
     close(ops.linked_product(later, prep(w_gu, swiglu=True) if packed else w_gu, inter, packed, torch.bfloat16,
-                             swiglu=True), P.silu(y[:, :inter]) * y[:, inter:], 1e-2, "the same with swiglu")
+                             swiglu=True), P.silu(y[:, :inter]) * y[:, inter:], BF16_TWICE, "the same with swiglu")
     # both sides at once: the next branch's product reads prepared rows and prepares the following norm
     w_back = t(rng.normal(size=(hidden, hidden)) / np.sqrt(hidden), torch.bfloat16)
     r2 = f64(residual) + normed @ f64(w_back).T
@@ -706,7 +718,7 @@ def test_packed_product_of_17_to_64_rows(ops, m, n, k):
     out = ops.gemm_mid_packed_bf16(x, pw, n, torch.float32)
     close(out, f64(x) @ f64(w).T, 2e-5, "packed product, 17 to 64 rows")
     y = f64(x) @ f64(gu).T
-    close(ops.gemm_mid_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True), P.silu(y[:, :n]) * y[:, n:], 1e-2,
+    close(ops.gemm_mid_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True), P.silu(y[:, :n]) * y[:, n:], BF16_OUT,
           "the same with swiglu")
     # a row's result is the same whatever the number of rows, and the same as the kernel for up to 16 rows gives
     first = min(m, 16)
@@ -777,11 +789,11 @@ def test_streaming_attention_walks_a_run_of_more_pages_than_it_holds_table_entri
     seq = t(np.arange(B), torch.int32)
     got = ops.attention_decode_bf16(qkv, kp, vp, cu, pos, table, B, max(lens), heads, kv_heads, dh, None, dh ** -0.5)
     want = ops.attention(qkv, kp, vp, pos, seq, table, heads, kv_heads, dh, None, dh ** -0.5)
-    close(got, f64(want), 1e-2, "a run of more than 1,024 pages")
+    close(got, f64(want), BF16_OUT, "a run of more than 1,024 pages")
     for b, head in ((5, 2), (5, 3), (9, 1), (20, 4)):       # and these rows are not drowned by the others' size
         row = slice(head * dh, (head + 1) * dh)
         assert want[b, row].float().abs().max() > 0.5
-        close(got[b, row], f64(want[b, row]), 1e-2, f"sequence {b}, head {head}")
+        close(got[b, row], f64(want[b, row]), BF16_OUT, f"sequence {b}, head {head}")
 
 
 @pytest.mark.parametrize("fused", [False, True])
