@@ -12,7 +12,8 @@ import torch
 
 from .cache import PAGE_SIZE
 from .engine import Engine, GenerationResult, StepEntry, generate as _generate
-from .parts import load_model, random_model
+from .engine.plain_engine import PlainEngine
+from .parts import load_model, load_model_plain, random_model
 from .sampling import DEFAULT_SEED, SamplingParams
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -32,15 +33,25 @@ class Model:
     """A loaded model with a cache sized for ``max_batch`` sequences of ``max_seq_len`` tokens."""
 
     def __init__(self, decoder, max_batch: int = 8, max_seq_len: int = 4096, max_tokens: int | None = None,
-                 use_graphs: bool = True):
+                 use_graphs: bool = True, plain: bool = False):
         self.decoder = decoder
         self.config = getattr(decoder, "config", None)
         per_seq = -(-max_seq_len // PAGE_SIZE) * PAGE_SIZE
-        self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
-        self.engine = Engine(decoder, self.cache, use_graphs=use_graphs)
+        if plain:
+            self.engine = PlainEngine(decoder, max_batch, max_tokens or per_seq * max_batch, max_seq_len)
+            self.cache = self.engine.cache
+        else:
+            self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
+            self.engine = Engine(decoder, self.cache, use_graphs=use_graphs)
 
     @classmethod
     def load(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **cache_options) -> "Model":
+        """``device="cpu"`` chooses the plain backend (the reference's ``--device cpu``, src/bin/runner.rs:98-100):
+        the whole model in float32 on the scalar C++ twins of the kernels, for the parts that have a plain form."""
+        if str(device).startswith("cpu"):
+            if as_dtype(dtype) != torch.float32:
+                raise ValueError("the CPU backend computes in float32 (weights stay as stored and are widened exactly)")
+            return cls(load_model_plain(model_dir), plain=True, **cache_options)
         return cls(load_model(model_dir, as_dtype(dtype), device), **cache_options)
 
     @classmethod

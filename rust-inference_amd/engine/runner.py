@@ -3,7 +3,7 @@ option names and meanings where it has them.
 
     runner <MODEL_DIR> [-p PROMPT] [-n N] [--chat [--think]] [--temperature T] [--top-k K] [--top-p P]
            [--repetition-penalty R] [--seed S] [--ignore-eos] [--max-pages N] [--pages-per-seq N]
-           [-t THREADS] [--dtype bfloat16|float32] [--profile] [--random [--random-seed S]]
+           [-t THREADS] [--device cuda|cpu] [--dtype bfloat16|float32] [--profile] [--random [--random-seed S]]
 
 The prompt is text when the model folder has a tokenizer.json (read with the `tokenizers` package),
 else a list of token ids (`-p "5 17 3"` or `--prompt-ids 5,17,3`); it is read from standard input when
@@ -40,7 +40,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--top-p", type=float, default=1.0, help="nucleus sampling threshold (1.0 = off)")
     ap.add_argument("--repetition-penalty", type=float, default=1.0, help="penalty for tokens already in the context")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=DEFAULT_SEED, help="sampling seed")
-    ap.add_argument("--device", default="cuda", choices=["cuda"], help="this build runs on the GPU only")
+    ap.add_argument("--device", default="cuda", choices=["cuda", "cpu"],
+                    help="cuda: the HIP kernels; cpu: the plain backend (float32, slow: for reading a checkpoint's "
+                    "output without a GPU)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="compute precision")
     ap.add_argument("--stop-token-ids", default=None, help="comma-separated ids that end a sequence "
                     "(default: eos_token_id of generation_config.json or config.json, if present)")
@@ -153,13 +155,18 @@ def main(argv=None) -> int:
         per_seq = args.pages_per_seq * PAGE_SIZE
         options = dict(max_batch=min(len(prompts), 64), max_seq_len=per_seq, max_tokens=args.max_pages * PAGE_SIZE,
                        use_graphs=not args.no_graphs)
-        if args.random:
+        if args.device == "cpu":
+            if args.random or args.profile:
+                print("error: --device cpu reads a model folder and has no section timers", file=sys.stderr)
+                return 1
+            model = Model.load(args.model_dir, dtype="float32", device="cpu", **options)
+        elif args.random:
             path = args.model_dir if os.path.isfile(args.model_dir) else os.path.join(args.model_dir, "config.json")
             with open(path) as f:
                 model = Model.random(json.load(f), seed=args.random_seed, dtype=args.dtype, **options)
         else:
             model = Model.load(args.model_dir, dtype=args.dtype, **options)
-    except (InferenceError, OSError, json.JSONDecodeError) as e:
+    except (InferenceError, OSError, ValueError, json.JSONDecodeError) as e:
         print(f"error: {e}", file=sys.stderr)
         return 1
     print(f"loaded {args.model_dir} in {time.perf_counter() - t0:.2f} s", file=sys.stderr)

@@ -91,6 +91,38 @@ class GroupedQueryAttention(Mixer):
             self.b_o = rt.place_gain(weights[p + "o_proj.bias"])
         self.position.bind(weights, rt)
 
+    def bind_plain(self, weights):
+        f32 = lambda name: weights[self.prefix + name].to(torch.float32).numpy()
+        self.plain_w = {n: f32(n + "_proj.weight") for n in "qkvo"}
+        self.plain_gain = {n: f32(n + "_norm.weight") for n in "qk"} if self.qk_norm else {}
+        self.plain_bias = {n: f32(n + "_proj.bias") for n in ("qkv" if self.qkv_bias else "") + ("o" if self.o_bias else "")}
+        if getattr(self.position, "acts_after_norm", False) or not hasattr(self.position, "plain"):
+            raise ConfigError(f"the position encoding {type(self.position).__name__} has no plain form")
+        self.position.bind_plain(weights)
+
+    def plain(self, x, ctx, store, page_table):
+        """The same over numpy arrays and the plain C++ twins: three products, per-head norm, rotation, the new keys
+        and values into their pages (``store = (k_pages, v_pages)``, values transposed inside a page), attention
+        over the pages, output product."""
+        from ..kernels import plain
+        t, dh, page = x.shape[0], self.head_dim, store[0].shape[2]
+        heads = {}
+        for n, count in (("q", self.heads), ("k", self.kv_heads), ("v", self.kv_heads)):
+            y = plain.linear(x, self.plain_w[n])
+            if n in self.plain_bias:
+                y = y + self.plain_bias[n]
+            heads[n] = y.reshape(t, count, dh)
+        for n in "qk":
+            if self.qk_norm:
+                heads[n] = plain.rms_norm(heads[n], self.plain_gain[n], self.eps)
+            heads[n] = self.position.plain(heads[n], ctx.tok_pos)
+        phys = page_table[ctx.tok_seq, ctx.tok_pos // page]
+        store[0][phys, :, ctx.tok_pos % page, :] = heads["k"]
+        store[1][phys, :, :, ctx.tok_pos % page] = heads["v"]
+        o = plain.attention(heads["q"], store[0], store[1], ctx.tok_pos, ctx.tok_seq, page_table, self.window, self.scale)
+        y = plain.linear(o.reshape(t, self.heads * dh), self.plain_w["o"])
+        return y + self.plain_bias["o"] if "o" in self.plain_bias else y
+
     def takes_tiled_at(self, m: int) -> bool:
         """Whether this part's first product reads ``m`` rows in the matrix cores' order."""
         return self.rt.takes_tiled(self.w_qkv, m)

@@ -11,6 +11,12 @@ from ..weights.loader import TensorSpec
 
 
 class Part:
+    """A part may also run on the CPU, for the plain backend (engine/plain_engine.py: the whole model over the
+    scalar C++ twins of the kernels, in float32, as the reference's CPU path computes: src/ops/mod.rs:36-41,
+    src/cpu/linear.rs:119-130): ``bind_plain(weights)`` keeps what it needs as float32 numpy arrays and
+    ``plain(...)`` is its forward over numpy arrays, with the arguments of ``forward`` (a mixer's store is the
+    pair of page arrays ``(k_pages, v_pages)`` or its state arena).  A part without them cannot run there."""
+
     def tensors(self) -> dict[str, TensorSpec]:
         """Checkpoint names and shapes of this part's weights."""
         return {}

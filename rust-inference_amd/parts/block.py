@@ -115,6 +115,11 @@ class PreNormBlock:
         """Whether the part behind that norm reads ``rows`` rows in the matrix cores' order."""
         return _takes_tiled(self.mixer, rows)
 
+    def plain(self, h, ctx, store, page_table):
+        """``h`` after this layer, float32 numpy (the plain backend)."""
+        r = h + self.mixer.plain(self.mixer_norm.plain(h), ctx, store, page_table)
+        return r + self.feed_forward.plain(self.feed_forward_norm.plain(r), ctx)
+
     def forward(self, stream: ResidualStream, ctx, store, page_table, act_dtype) -> None:
         # a part with ``links_norms`` takes a NormedLater as input and a NormLink for its output
         rows = stream.sum.shape[0]

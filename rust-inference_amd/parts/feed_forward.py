@@ -35,6 +35,16 @@ class SwiGLU(FeedForward):
         self.w_gate_up = rt.pack(gate_up, swiglu=True)
         self.w_down = rt.pack(rt.place_matrix(weights[p + "down_proj.weight"]))
 
+    def bind_plain(self, weights):
+        p = self.prefix
+        self.plain_w = {n: weights[p + n + "_proj.weight"].to(torch.float32).numpy() for n in ("gate", "up", "down")}
+
+    def plain(self, x, ctx):
+        from ..kernels import plain
+        import numpy as np
+        y = np.concatenate([plain.linear(x, self.plain_w["gate"]), plain.linear(x, self.plain_w["up"])], axis=1)
+        return plain.linear(plain.swiglu(y), self.plain_w["down"])
+
     def takes_tiled_at(self, m: int) -> bool:
         """Whether this part's first product reads ``m`` rows in the matrix cores' order."""
         return self.rt.takes_tiled(self.w_gate_up, m)

@@ -37,6 +37,13 @@ class TokenEmbedding(Embedding):
     def forward(self, ctx):
         return ops.embed_gather(self.table, ctx.tokens)
 
+    def bind_plain(self, weights):
+        self.table_plain = weights[self.name].to(torch.float32).numpy()
+
+    def plain(self, ctx):
+        from ..kernels import plain
+        return plain.embedding(self.table_plain, ctx.tokens)
+
 
 @register_part("head", "linear")
 class OutputHead(Head):
@@ -66,6 +73,21 @@ class OutputHead(Head):
                 raise ConfigError(f"{self.name} is absent and there is no embedding table of {self.vocab} x {self.dim} "
                                   "to tie it to")
             self.weight = table                     # the same device tensor: tying costs no memory
+
+    def bind_plain(self, weights):
+        self.weight_plain = None
+        if not self.tied and self.name in weights:
+            self.weight_plain = weights[self.name].to(torch.float32).numpy()
+
+    def connect_plain(self, parts):
+        if self.weight_plain is None:
+            self.weight_plain = getattr(parts.get("embedding"), "table_plain", None)
+            if self.weight_plain is None or self.weight_plain.shape != (self.vocab, self.dim):
+                raise ConfigError(f"{self.name} is absent and there is no embedding table to tie it to")
+
+    def plain(self, x):
+        from ..kernels import plain
+        return plain.linear(x, self.weight_plain)
 
     def _packed_copy(self):
         """A second copy of the matrix in the matrix cores' tile order, for steps that want 2 to 16 rows of
@@ -131,6 +153,35 @@ class DecoderModel:
             if connect is not None:
                 connect(named)
         return self
+
+    def bind_plain(self, weights: dict) -> "DecoderModel":
+        """Take the weights for the plain backend: every part keeps float32 numpy arrays.  A part that has no
+        plain form is named in the error."""
+        for part in self.parts():
+            if not hasattr(part, "bind_plain") or not hasattr(part, "plain"):
+                raise ConfigError(f"the part {type(part).__name__} has no plain form: the CPU backend cannot run this model")
+        for layer in self.layers:
+            if not hasattr(layer, "plain"):
+                raise ConfigError(f"the arrangement {type(layer).__name__} has no plain form")
+        for part in self.parts():
+            part.bind_plain(weights)
+        named = {"embedding": self.embedding, "layers": self.layers, "final_norm": self.final_norm, "head": self.head}
+        for part in self.parts():
+            if hasattr(part, "connect_plain"):
+                part.connect_plain(named)
+        return self
+
+    def plain_forward(self, ctx, stores, page_tables):
+        """float32 logits ``[n_want, vocab]`` (numpy) of a step on the CPU: ``stores[entry]`` is the cache entry's
+        storage (a pair of page arrays), ``page_tables[group]`` the step's table of its group."""
+        h = self.embedding.plain(ctx)
+        for run in self.schedule:
+            entries = run.entries()
+            if len(entries) != 1:
+                raise ConfigError("the plain backend runs layers with one cache entry")
+            store, group = stores[entries[0]]
+            h = self.layers[run.layer].plain(h, ctx, store, page_tables[group])
+        return self.head.plain(self.final_norm.plain(h[ctx.want_rows]))
 
     # ---- cache
     def cache_needs(self) -> list:
@@ -209,6 +260,15 @@ def load_model(model_dir: str, dtype=torch.bfloat16, device="cuda:0") -> Decoder
     model.config = cfg
     weights = load_checked(model_dir, model.tensors())
     return model.bind(weights, Runtime(device, dtype))
+
+
+def load_model_plain(model_dir: str) -> DecoderModel:
+    """The model of a folder for the CPU backend: the same class and the same checks, the weights kept as
+    float32 numpy arrays by the parts' plain forms."""
+    arch, cfg = load_config(model_dir)
+    model = DecoderModel(arch.build_spec(cfg))
+    model.config = cfg
+    return model.bind_plain(load_checked(model_dir, model.tensors()))
 
 
 def random_model(config, seed: int, dtype=torch.bfloat16, device="cuda:0", store_dtype=torch.bfloat16) -> DecoderModel:

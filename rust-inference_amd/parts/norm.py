@@ -1,7 +1,9 @@
 """RMSNorm, fused with the residual add that precedes it."""
 from __future__ import annotations
 
-from ..kernels import ops
+import torch
+
+from ..kernels import ops, plain
 from ..weights.loader import GAIN, TensorSpec
 from .base import Norm
 from .registry import register_part
@@ -25,6 +27,12 @@ class RMSNorm(Norm):
     def bind(self, weights, rt):
         self.rt = rt
         self.gain = rt.place_gain(weights[self.name])
+
+    def bind_plain(self, weights):
+        self.gain_plain = weights[self.name].to(torch.float32).numpy()
+
+    def plain(self, x):
+        return plain.rms_norm(x, self.gain_plain, self.eps)
 
     def apply(self, residual, pending, out_dtype, rows=None, tiled=False):
         tiled = tiled and self.dim % 4 == 0 and self.dim <= 8192        # what the vectorised kernel takes

@@ -27,6 +27,15 @@ class RotateHalf(PositionEncoding):
         theta = torch.tensor(self.theta, dtype=torch.float32)
         self.inv_freq = (1.0 / torch.pow(theta, expo)).to(torch.float32).to(rt.device).contiguous()
 
+    def bind_plain(self, weights):
+        from ..kernels import plain
+        self.inv_freq_plain = plain.rope_inv_freq(self.head_dim, self.theta)
+
+    def plain(self, heads, positions):
+        """Rotates ``heads: [tokens, n, head_dim]`` (already normed) by their tokens' positions."""
+        from ..kernels import plain
+        return plain.rope(heads, positions, self.inv_freq_plain)
+
     def rotation_table(self):
         return self.inv_freq
 
@@ -37,3 +46,9 @@ class NoPosition(PositionEncoding):
 
     def __init__(self, **_):
         pass
+
+    def bind_plain(self, weights):
+        pass
+
+    def plain(self, heads, positions):
+        return heads
