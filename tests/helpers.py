@@ -45,6 +45,9 @@ def rel_to_max(got, want):
 # (tests/model_parity.rs:23-28); this build's target is 1e-4.  bfloat16: activations are rounded to
 # 8 bits of mantissa after every product, the reference allows 1e-2 to 3e-2 of the largest value per
 # op (tests/cuda_parity.rs:43-127); whole-model logits get 3e-2.
+# Measured over all whole-model comparisons of the GPU tests (RI_TEST_ERROR_REPORT collects them): float32 5e-7 to
+# 1.8e-5 of the largest logit; bfloat16 7e-3 to 2.0e-2 (the tiny models' weights are six times the benchmark's, so
+# that logits are of order one and every layer's rounding shows).
 F32_BOUND = 1e-4
 BF16_BOUND = 3e-2
 
