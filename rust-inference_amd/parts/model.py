@@ -90,7 +90,7 @@ class OutputHead(Head):
         return plain.linear(x, self.weight_plain)
 
     def _packed_copy(self):
-        """A second copy of the matrix in the matrix cores' tile order, for steps that want 2 to 16 rows of
+        """A second copy of the matrix in the matrix cores' tile order, for steps that want 2 to 32 rows of
         logits (a decode step of as many sequences): at 151,936 x 4,096 the packed kernel takes 0.21 ms where
         the library's product takes 0.26 (1% of such a step), for 1.2 GB more memory.  It is made at the first
         such step, so that a model which never runs one (a single slot, or only larger batches) does not pay
@@ -99,11 +99,20 @@ class OutputHead(Head):
             self.packed = self.rt.pack(self.weight, always=True)
         return self.packed
 
+    # Rows of logits up to which the packed copy serves: 2 to 16 the packed kernel; 17 to 32 the wide kernel with
+    # four row tiles a workgroup (151,936 x 4,096 at 17 and 32 rows: 222 and 247 us against the library's 279 and
+    # 274; from 48 rows on the library is ahead, 266 against 279 us, with 39 MB of float32 logits to write).
+    PACKED_MAX_ROWS = 32
+
     def forward(self, x):
-        if 2 <= x.shape[0] <= 16:
+        rows = x.shape[0]
+        if 2 <= rows <= self.PACKED_MAX_ROWS and self.dim % 8 == 0:
             packed = self._packed_copy()
             if packed is not None and packed.packed is not None:
-                return self.rt.linear_packed(x, packed, out_dtype=torch.float32)
+                if rows <= 16:
+                    return self.rt.linear_packed(x, packed, out_dtype=torch.float32)
+                return ops.gemm_wide_packed_bf16(self.rt.normed_now(x), packed.packed, self.vocab, torch.float32,
+                                                 depth=1, waves=4)
         return self.rt.linear(x, self.weight, out_dtype=torch.float32)
 
 
