@@ -45,19 +45,23 @@ class Model:
             self.engine = Engine(decoder, self.cache, use_graphs=use_graphs)
 
     @classmethod
-    def load(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **cache_options) -> "Model":
-        """``device="cpu"`` chooses the plain backend (the reference's ``--device cpu``, src/bin/runner.rs:98-100):
+    def load(cls, model_dir: str, dtype="bfloat16", device="cuda:0", batch_invariant: bool = False,
+             **cache_options) -> "Model":
+        """``batch_invariant`` (bfloat16 on the GPU): every step runs the same form of every kernel, so that a
+        request's logits and tokens are the same bits in any batch and any cut (``parts.runtime.Runtime``).
+        ``device="cpu"`` chooses the plain backend (the reference's ``--device cpu``, src/bin/runner.rs:98-100):
         the whole model in float32 on the scalar C++ twins of the kernels, for the parts that have a plain form."""
         if str(device).startswith("cpu"):
             if as_dtype(dtype) != torch.float32:
                 raise ValueError("the CPU backend computes in float32 (weights stay as stored and are widened exactly)")
             return cls(load_model_plain(model_dir), plain=True, **cache_options)
-        return cls(load_model(model_dir, as_dtype(dtype), device), **cache_options)
+        return cls(load_model(model_dir, as_dtype(dtype), device, batch_invariant), **cache_options)
 
     @classmethod
-    def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", **cache_options) -> "Model":
+    def random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", batch_invariant: bool = False,
+               **cache_options) -> "Model":
         """Random weights made in memory from a config.json dict or a typed configuration."""
-        return cls(random_model(config, seed, as_dtype(dtype), device), **cache_options)
+        return cls(random_model(config, seed, as_dtype(dtype), device, invariant=batch_invariant), **cache_options)
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 600, temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 1.0, repetition_penalty: float = 1.0, seed: int = DEFAULT_SEED,

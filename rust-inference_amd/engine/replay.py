@@ -60,11 +60,11 @@ def engine_for_trace(model, max_tokens: int) -> Engine:
 
 
 def run(model_dir: str, dtype: torch.dtype, out_dir: str, max_tokens: int, lines=None, device="cuda:0",
-        reply=None) -> int:
+        reply=None, invariant: bool = False) -> int:
     lines = sys.stdin if lines is None else lines
     reply = reply or (lambda s: print(s, flush=True))
     os.makedirs(out_dir, exist_ok=True)
-    player = Replayer(engine_for_trace(load_model(model_dir, dtype, device), max_tokens))
+    player = Replayer(engine_for_trace(load_model(model_dir, dtype, device, invariant), max_tokens))
     for line in lines:
         line = line.strip()
         if not line:

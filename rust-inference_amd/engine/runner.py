@@ -47,6 +47,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--stop-token-ids", default=None, help="comma-separated ids that end a sequence "
                     "(default: eos_token_id of generation_config.json or config.json, if present)")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    ap.add_argument("--batch-invariant", action="store_true", help="bfloat16 on the GPU: every step runs the same form "
+                    "of every kernel, so that a request's tokens do not depend on its batch (slower, above all on prompts)")
     ap.add_argument("--random", action="store_true", help="MODEL_DIR needs only a config.json (or is one): the weights "
                     "are made in memory, N(0, 0.02) with gains 1 + N(0, 0.1), from --random-seed")
     ap.add_argument("--random-seed", type=int, default=0, help="seed of the weights made by --random")
@@ -163,9 +165,10 @@ def main(argv=None) -> int:
         elif args.random:
             path = args.model_dir if os.path.isfile(args.model_dir) else os.path.join(args.model_dir, "config.json")
             with open(path) as f:
-                model = Model.random(json.load(f), seed=args.random_seed, dtype=args.dtype, **options)
+                model = Model.random(json.load(f), seed=args.random_seed, dtype=args.dtype,
+                                     batch_invariant=args.batch_invariant, **options)
         else:
-            model = Model.load(args.model_dir, dtype=args.dtype, **options)
+            model = Model.load(args.model_dir, dtype=args.dtype, batch_invariant=args.batch_invariant, **options)
     except (InferenceError, OSError, ValueError, json.JSONDecodeError) as e:
         print(f"error: {e}", file=sys.stderr)
         return 1

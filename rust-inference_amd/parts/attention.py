@@ -141,7 +141,7 @@ class GroupedQueryAttention(Mixer):
         table = self.position.rotation_table()
         whole = table is None or 2 * table.shape[0] == self.head_dim      # the fused kernel rotates whole heads
         after_norm = getattr(self.position, "acts_after_norm", False)
-        if (ctx.is_decode and whole and not after_norm
+        if (ctx.is_decode and whole and not after_norm and not rt.invariant
                 and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, True)
                 and (ctx.B <= FUSED_DECODE_MAX_SEQS
                      or ops.decode_attention_streams(ctx.B, self.kv_heads, ctx.max_len))):
@@ -162,6 +162,10 @@ class GroupedQueryAttention(Mixer):
                 self.position.apply_normed(qkv, ctx, *shape)
                 ops.qk_norm_rope_kv_write(qkv, None, None, self.eps, None, ctx.tok_pos, ctx.tok_seq, page_table,
                                           store.k_pages, store.v_pages, *shape, ctx.cu_seqlens, ctx.max_new)
+            elif rt.invariant:
+                # the kernel of one wavefront per token and head, whatever the step looks like
+                ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, table, ctx.tok_pos, ctx.tok_seq,
+                                          page_table, store.k_pages, store.v_pages, *shape)
             else:
                 ops.qk_norm_rope_kv_write(qkv, self.q_gain, self.k_gain, self.eps, table, ctx.tok_pos, ctx.tok_seq,
                                           page_table, store.k_pages, store.v_pages, *shape, ctx.cu_seqlens, ctx.max_new)
@@ -180,7 +184,7 @@ class GroupedQueryAttention(Mixer):
         sequence, or any number), the generic kernel for everything else."""
         args = (self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
         group = self.heads // self.kv_heads
-        if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
+        if not self.rt.invariant and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
             if ctx.is_decode:
                 return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                                  page_table, ctx.B, ctx.max_len, *args,

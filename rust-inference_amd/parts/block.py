@@ -39,11 +39,12 @@ class ResidualStream:
         self.later = None            # (NormedLater, the norm it was prepared for)
         self.next_entry_norm = None  # the norm that reads the stream after the current layer, if known
         self.next_entry_tiled = False  # and whether the part behind it reads tiled rows
+        self.links_ok = True         # whether norms may be left to products at all (not where every step must run alike)
 
     def link(self, norm, act_dtype, tiled: bool = False):
         """A ``NormLink`` for the branch that is about to run, if ``norm`` is the next reader of the
         stream and can be left to a product.  ``tiled``: the part behind that norm reads tiled rows."""
-        if (norm is None or not getattr(norm, "linkable", False) or self.pending is not None or self.later is not None
+        if (not self.links_ok or norm is None or not getattr(norm, "linkable", False) or self.pending is not None or self.later is not None
                 or act_dtype != torch.bfloat16 or self.sum.shape[0] > LINK_MAX_TOKENS
                 or norm.dim != self.sum.shape[1]):
             return None

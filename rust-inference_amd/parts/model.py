@@ -106,6 +106,8 @@ class OutputHead(Head):
 
     def forward(self, x):
         rows = x.shape[0]
+        if self.rt.invariant:
+            return self.rt.linear_packed(x, self._packed_copy(), out_dtype=torch.float32)
         if 2 <= rows <= self.PACKED_MAX_ROWS and self.dim % 8 == 0:
             packed = self._packed_copy()
             if packed is not None and packed.packed is not None:
@@ -227,6 +229,7 @@ class DecoderModel:
         rt = self.rt
         with profiler.section(profiler.EMBEDDING):
             stream = ResidualStream(self.embedding.forward(ctx))
+        stream.links_ok = not rt.invariant
         for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]
             follower = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
@@ -262,13 +265,13 @@ def expected_tensors(spec: ModelSpec, for_writing: bool = False) -> dict[str, Te
     return DecoderModel(spec).tensors(for_writing)
 
 
-def load_model(model_dir: str, dtype=torch.bfloat16, device="cuda:0") -> DecoderModel:
-    """The model of a folder: the class by config.json, the weights by name."""
+def load_model(model_dir: str, dtype=torch.bfloat16, device="cuda:0", invariant: bool = False) -> DecoderModel:
+    """The model of a folder: the class by config.json, the weights by name.  ``invariant``: see ``Runtime``."""
     arch, cfg = load_config(model_dir)
     model = DecoderModel(arch.build_spec(cfg))
     model.config = cfg
     weights = load_checked(model_dir, model.tensors())
-    return model.bind(weights, Runtime(device, dtype))
+    return model.bind(weights, Runtime(device, dtype, invariant))
 
 
 def load_model_plain(model_dir: str) -> DecoderModel:
@@ -280,12 +283,13 @@ def load_model_plain(model_dir: str) -> DecoderModel:
     return model.bind_plain(load_checked(model_dir, model.tensors()))
 
 
-def random_model(config, seed: int, dtype=torch.bfloat16, device="cuda:0", store_dtype=torch.bfloat16) -> DecoderModel:
+def random_model(config, seed: int, dtype=torch.bfloat16, device="cuda:0", store_dtype=torch.bfloat16,
+                 invariant: bool = False) -> DecoderModel:
     """A model with random weights made in memory, for sizes one would not write to disk."""
     from ..config import config_from_dict
     arch, cfg = config_from_dict(config if isinstance(config, dict) else config.to_dict())
     model = DecoderModel(arch.build_spec(cfg))
     model.config = cfg
-    rt = Runtime(device, dtype)
+    rt = Runtime(device, dtype, invariant)
     weights = random_tensors(model.tensors(for_writing=True), seed, store_dtype, device=rt.device)
     return model.bind(weights, rt)

@@ -71,15 +71,26 @@ class PackedWeight:
 class Runtime:
     """``dtype`` is the compute dtype: bfloat16 (16-bit activations and cache,
     float32 statistics and residual stream) or float32 (everything in true 32-bit;
-    weights stay as stored and are widened exactly inside the kernels)."""
+    weights stay as stored and are widened exactly inside the kernels).
 
-    def __init__(self, device="cuda:0", dtype=torch.bfloat16):
+    ``invariant`` (bfloat16 only; float32 is so by itself): every step runs the same form of every kernel whatever
+    its size, so that a request's logits are the same bits alone and in any batch, whole and token by token, as a
+    graph and launched from the host.  The bfloat16 path otherwise chooses the product kernel by the number of rows,
+    the attention kernel by the number of sequences and leaves small steps' norms to the products, and each form
+    rounds at other places.  Here every product is the packed kernel for 17 to 64 rows in slices of 64 rows
+    (a row's sums in it do not depend on the other rows), every norm the plain kernel, the q/k norm, rotation
+    and cache write the kernel of one wavefront per token and head, and the attention the generic kernel, whose
+    key tiles start at fixed positions.  It is several times slower on prompts; it is for runs that must
+    reproduce bit for bit."""
+
+    def __init__(self, device="cuda:0", dtype=torch.bfloat16, invariant: bool = False):
         if dtype not in (torch.bfloat16, torch.float32):
             raise ShapeError(f"compute dtype {dtype} is neither bfloat16 nor float32")
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise KernelError(f"this library computes on the GPU only, not on {self.device}")
         self.dtype = dtype
+        self.invariant = bool(invariant) and dtype == torch.bfloat16
         self._mm_out_dtype = None
 
     # ---- weights
@@ -123,7 +134,9 @@ class Runtime:
         """A placed weight, with a packed copy where the packed kernel is the faster one for 2 to 16
         rows (bfloat16 compute only), or wherever it can be used when the caller says ``always``."""
         n, k = w.shape
-        pays = always or swiglu or _packed_pays(n, k)
+        if self.invariant and k % 8:
+            raise ShapeError(f"the invariant mode's product takes rows of a multiple of 8 elements, not {k}")
+        pays = always or swiglu or self.invariant or _packed_pays(n, k)
         if self.dtype != torch.bfloat16 or k % 8 or not pays:
             return PackedWeight(w, None, swiglu)
         return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
@@ -151,7 +164,7 @@ class Runtime:
     def takes_tiled(self, pw: PackedWeight, m: int, parts_ok: bool = False) -> bool:
         """Whether the product of ``m`` rows with this weight (called with this ``parts_ok``) runs on a packed
         kernel: whoever makes its rows then makes them as ``ops.TiledRows``."""
-        if self.dtype != torch.bfloat16 or pw.packed is None or pw.k % 8:
+        if self.dtype != torch.bfloat16 or pw.packed is None or pw.k % 8 or self.invariant:
             return False
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
@@ -173,6 +186,12 @@ class Runtime:
         return value is then ``(NormedLater, norm)`` for the stream instead of a tensor."""
         out_dtype = out_dtype or self.dtype
         m = x.shape[0]
+        if self.invariant:
+            # one kernel for every step: a row's sums in it depend on the row and the matrix alone
+            x = self.normed_now(x)
+            outs = [ops.gemm_mid_packed_bf16(x[i:i + MID_MAX_ROWS], pw.packed, pw.n, out_dtype, swiglu=pw.swiglu)
+                    for i in range(0, m, MID_MAX_ROWS)]
+            return outs[0] if len(outs) == 1 else torch.cat(outs, 0)
         if self.dtype == torch.bfloat16 and pw.k % 8 == 0:
             later = isinstance(x, ops.NormedLater)
             mine = None

@@ -367,6 +367,46 @@ def test_any_cut_of_the_work_gives_the_same_logits(model_dirs, loaded, name, dty
                         "any cut")
 
 
+@pytest.mark.parametrize("name", ["B", "C", "D"])
+def test_the_invariant_mode_gives_the_same_bits_however_the_work_is_cut(model_dirs, name):
+    """bfloat16 with ``invariant``: whole prompts alone, the last 32 tokens one by one (as graphs), unequal
+    batches in two orders and pieces of 70 tokens (two slices of the product kernel) give the same logits bit
+    for bit, and they are the plain implementation's within the bfloat16 bound."""
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.parts import load_model
+    cfg, _ = read_model_f64(model_dirs[name])
+    reqs = requests_for(name, cfg, [150, 37, 70, 1, 97], 77)
+    model = load_model(model_dirs[name], torch.bfloat16, invariant=True)
+    assert model.rt.invariant
+    whole = replay_in_process(model, plans.whole(reqs))
+    check_against_plain(model_dirs[name], whole, reqs, "bfloat16", "invariant mode, whole")
+    ids = list(reqs)
+    cuts = {
+        "one by one": replay_in_process(model, plans.tail_one_by_one(reqs, 32)),
+        "a batch": replay_in_process(model, plans.unequal_batches([{r: (reqs[r], max(1, len(reqs[r]) - 9)) for r in ids}])),
+        "the batch the other way round": replay_in_process(
+            model, plans.unequal_batches([{r: (reqs[r], max(1, len(reqs[r]) - 20)) for r in reversed(ids)}])),
+    }
+    engine = Engine(model, model.new_cache(max_tokens=5 * 192, num_slots=5, max_seq_len=192))
+    slots = {r: engine.cache.acquire() for r in ids}
+    pieces = {r: [] for r in ids}
+    for at in range(0, 150, 70):
+        live = [r for r in ids if len(reqs[r]) > at]
+        logits = engine.step([StepEntry(slots[r], reqs[r][at:at + 70], "all") for r in live]).cpu().numpy()
+        row = 0
+        for r in live:
+            n = len(reqs[r][at:at + 70])
+            pieces[r].append(logits[row:row + n])
+            row += n
+    cuts["pieces of 70"] = {r: np.concatenate(p) for r, p in pieces.items()}
+    for what, got in cuts.items():
+        for r in ids:
+            assert got[r].shape == whole[r].shape
+            differ = np.flatnonzero((got[r].view(np.uint32) != whole[r].view(np.uint32)).any(axis=1))
+            assert differ.size == 0, (f"{what}, request {r}: position {differ[0]} is the first of {differ.size} whose "
+                                      f"logits differ from the whole prompt's, by {rel_to_max(got[r], whole[r]):.1e}")
+
+
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_one_layer_of_the_large_model(tmp_path_factory, dtype_name):
     """The layer sizes of Qwen3-8B (one layer, a small vocabulary): the sizes at which the decode kernels

@@ -82,6 +82,28 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name, lengths, st
     assert model.cache.slots.free_count == 4
 
 
+def test_batch_invariant_generation_gives_a_request_the_same_tokens_in_any_batch(model_dirs):
+    """``batch_invariant=True``: sampled tokens (temperature, so that a last bit of a logit can show) of each
+    request alone, in a batch of all and in batches of four and three are the same, with graphs and without."""
+    from rust_inference_amd import Model, SamplingParams
+    cfg, _ = read_model_f64(model_dirs["D"])
+    prompts = prompts_for(cfg, [70, 2, 40, 1, 33, 17, 64], 5)
+    # (sequence i of a call draws from the generator seeded seed + i)
+    sampling = [SamplingParams(temperature=1.5, top_k=0, top_p=1.0, seed=100)] * len(prompts)
+    outs = {}
+    for graphs in (False, True):
+        model = Model.load(model_dirs["D"], dtype="bfloat16", batch_invariant=True, max_batch=7, max_seq_len=128,
+                           use_graphs=graphs)
+        outs[graphs, "together"] = model.generate(prompts, max_new_tokens=24, sampling=sampling).tokens
+        outs[graphs, "in fours"] = model.generate(prompts, max_new_tokens=24, sampling=sampling, max_batch=4).tokens
+        outs[graphs, "alone"] = [model.generate([p], max_new_tokens=24, temperature=1.5, seed=100 + i).tokens[0]
+                                 for i, p in enumerate(prompts)]
+    first = outs[False, "alone"]
+    assert len({tuple(t) for t in first}) > 1
+    for key, tokens in outs.items():
+        assert tokens == first, f"{key}: a request's tokens depend on its batch"
+
+
 @pytest.mark.parametrize("requests", [20, 40])
 def test_batches_of_tens_of_sequences(model_dirs, requests):
     """Twenty and forty sequences a batch (the decode steps of 17 to 32 rows and of 33 to 64 take other kernels
