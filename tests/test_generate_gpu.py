@@ -108,7 +108,7 @@ def test_batch_invariant_generation_gives_a_request_the_same_tokens_in_any_batch
 def test_batches_of_tens_of_sequences(model_dirs, requests):
     """Twenty and forty sequences a batch (the decode steps of 17 to 32 rows and of 33 to 64 take other kernels
     than the smaller ones), some stopping early so that the batch shrinks through those sizes: graphs and
-    eager steps give the same tokens, and those are the plain implementation's."""
+    eager steps both give the plain implementation's tokens."""
     from rust_inference_amd import Model
     cfg, _ = read_model_f64(model_dirs["D"])
     rng = np.random.default_rng(requests)
@@ -122,10 +122,14 @@ def test_batches_of_tens_of_sequences(model_dirs, requests):
         model.cache.check_consistent()
         assert model.cache.slots.free_count == requests
         outs.append(res)
-    assert outs[0].tokens == outs[1].tokens and outs[0].finish_reasons == outs[1].finish_reasons
-    assert "stop" in outs[0].finish_reasons
-    assert_same_tokens(outs[0].tokens, plain_greedy_with_margins(model_dirs["D"], prompts, 12, stop), "bfloat16",
-                       model_dirs["D"], prompts, stop)
+    # (The loop over graphs runs one step ahead of the ids it has read, so a sequence that stops is carried one
+    # step further than in the other loop: a step of 17 rows here is one of 16 there, on another kernel, and in
+    # bfloat16 two logits closer than its rounding may then change places.  Both are held to the plain
+    # implementation, which lets a sequence part from it at such a place only.)
+    want = plain_greedy_with_margins(model_dirs["D"], prompts, 12, stop)
+    for res in outs:
+        assert "stop" in res.finish_reasons
+        assert_same_tokens(res.tokens, want, "bfloat16", model_dirs["D"], prompts, stop)
 
 
 def test_stop_tokens_and_batches_one_after_another(model_dirs):
