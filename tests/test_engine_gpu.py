@@ -19,12 +19,16 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 _plain_cache = {}
+_last_read = {}
 
 
 def plain_logits(model_dir, tokens):
     key = (model_dir, tuple(tokens))
     if key not in _plain_cache:
-        cfg, w = read_model_f64(model_dir)
+        if _last_read.get("dir") != model_dir:               # one folder's float64 weights are kept at a time
+            _last_read.clear()
+            _last_read.update(dir=model_dir, model=read_model_f64(model_dir))
+        cfg, w = _last_read["model"]
         _plain_cache[key] = P.forward(cfg, w, list(tokens))
     return _plain_cache[key]
 
@@ -433,6 +437,49 @@ def test_one_layer_of_the_large_model(tmp_path_factory, dtype_name):
                     outs[s["step"]] = logits.cpu().numpy().copy()
             got = plans.collect(steps, lambda i: outs[i], 1000)
             check_against_plain(folder, got, reqs, dtype_name, f"large layer, {what}, graphs {graphs}")
+
+
+# The layer sizes of the published Qwen3 dense checkpoints other than 8B (name: hidden, intermediate, heads, kv
+# heads): what the kernels' rules choose at each (rows of 1,024 to 25,600 elements, 2 to 8 query heads a kv head,
+# K of 2,560 and 9,728 that the ring of eight steps does not divide).
+PUBLISHED = {"0.6B": (1024, 3072, 16, 8), "1.7B": (2048, 6144, 16, 8), "4B": (2560, 9728, 32, 8),
+             "14B": (5120, 17408, 40, 8), "32B": (5120, 25600, 64, 8)}
+
+
+@pytest.mark.parametrize("size", list(PUBLISHED))
+def test_one_layer_of_every_published_size(tmp_path, size):
+    """One layer and a small vocabulary at each size, bfloat16, through graphs: a request alone with its last
+    tokens one by one (the one-row products), batches of five, twenty and forty-four of unequal lengths (the
+    packed products of 2 to 16 rows, the wide ones of 17 to 32, those of 33 to 64, the library's for the prompts)."""
+    from rust_inference_amd.engine import Engine
+    from rust_inference_amd.engine.replay import Replayer
+    from rust_inference_amd.parts import load_model
+    from rust_inference_amd.weights import write_random_model
+    hidden, inter, heads, kv_heads = PUBLISHED[size]
+    cfg = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": 1000, "hidden_size": hidden,
+           "intermediate_size": inter, "num_hidden_layers": 1, "num_attention_heads": heads,
+           "num_key_value_heads": kv_heads, "head_dim": 128, "rope_theta": 1e6, "rms_norm_eps": 1e-6,
+           "tie_word_embeddings": size in ("0.6B", "1.7B", "4B")}
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=11, dtype=torch.bfloat16, matrix_std=0.02, gain_std=0.1)
+    rng = np.random.default_rng(len(size) + hidden)
+    model = load_model(folder, torch.bfloat16)
+    try:
+        for count, tail in ((1, 12), (5, 6), (20, 5), (44, 4)):
+            reqs = {f"{size}_{count}_{i}": [int(t) for t in rng.integers(0, 1000, n)]
+                    for i, n in enumerate(rng.integers(tail + 1, 48 if count > 1 else 140, count))}
+            steps = (plans.tail_one_by_one(reqs, tail) if count == 1 else
+                     plans.unequal_batches([{k: (v, len(v) - int(rng.integers(1, tail + 1))) for k, v in reqs.items()}]))
+            cache = model.new_cache(max_tokens=plans.max_live_tokens(steps), num_slots=count, max_seq_len=192)
+            player, outs = Replayer(Engine(model, cache, use_graphs=True)), {}
+            for st in steps:
+                logits = player.feed(st)
+                if logits is not None:
+                    outs[st["step"]] = logits.cpu().numpy().copy()
+            got = plans.collect(steps, lambda i: outs[i], 1000)
+            check_against_plain(folder, got, reqs, "bfloat16", f"one layer of {size}, {count} at a time")
+    finally:
+        _plain_cache.clear()
+        _last_read.clear()                                    # (the float64 weights of the largest are 4 GB)
 
 
 _large = {}
