@@ -36,7 +36,14 @@ def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages():
         emulated.library()
     except KernelError as e:
         pytest.skip(f"no CPU build of the kernels here: {e}")
-    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", os.path.join(HERE, "test_kernels_gpu.py"), "-k", SELECT])
+    workers = []
+    try:                                   # a few processes side by side where the plugin for that is installed
+        import xdist  # noqa: F401
+        workers = ["-n", str(max(1, min(4, (os.cpu_count() or 2) // 2)))]
+    except ImportError:
+        pass
+    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", *workers, os.path.join(HERE, "test_kernels_gpu.py"),
+                "-k", SELECT])
     assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-3000:]
     assert " passed" in run.stdout and "[emu]" not in run.stderr
 
