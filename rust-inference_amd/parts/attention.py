@@ -184,7 +184,15 @@ class GroupedQueryAttention(Mixer):
         sequence, or any number), the generic kernel for everything else."""
         args = (self.heads, self.kv_heads, self.head_dim, self.window, self.scale)
         group = self.heads // self.kv_heads
-        if not self.rt.invariant and ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
+        if self.rt.invariant:
+            # one kernel for prompts and single tokens alike: in the prompt kernel a token's sums run over its
+            # sequence's pages in order whatever the other rows of its tile are (a page that a row does not
+            # see changes none of its bits); the generic kernel where that one does not take the sizes
+            if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, False):
+                return ops.attention_prefill_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
+                                                  page_table, ctx.B, ctx.max_new, *args)
+            return ops.attention(qkv, store.k_pages, store.v_pages, ctx.tok_pos, ctx.tok_seq, page_table, *args)
+        if ops.mfma_attention_fits(qkv.dtype, self.head_dim, group, store.page_size, ctx.is_decode):
             if ctx.is_decode:
                 return ops.attention_decode_bf16(qkv, store.k_pages, store.v_pages, ctx.cu_seqlens, ctx.tok_pos,
                                                  page_table, ctx.B, ctx.max_len, *args,

@@ -79,9 +79,10 @@ class Runtime:
     the attention kernel by the number of sequences and leaves small steps' norms to the products, and each form
     rounds at other places.  Here every product is the packed kernel for 17 to 64 rows in slices of 64 rows
     (a row's sums in it do not depend on the other rows), every norm the plain kernel, the q/k norm, rotation
-    and cache write the kernel of one wavefront per token and head, and the attention the generic kernel, whose
-    key tiles start at fixed positions.  It is several times slower on prompts; it is for runs that must
-    reproduce bit for bit."""
+    and cache write the kernel of one wavefront per token and head, and the attention the prompt kernel for
+    single tokens too (a token's sums run over its sequence's pages in order whatever shares its tile), or the
+    generic kernel, whose key tiles start at fixed positions, where that one does not take the sizes.  It is
+    several times slower on prompts; it is for runs that must reproduce bit for bit."""
 
     def __init__(self, device="cuda:0", dtype=torch.bfloat16, invariant: bool = False):
         if dtype not in (torch.bfloat16, torch.float32):
