@@ -9,6 +9,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <type_traits>
@@ -38,8 +39,23 @@ enum hipError_t { hipSuccess = 0, hipErrorNoDevice = 100 };
 enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 63 };
 static inline hipError_t hipGetLastError() { return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "no error (emulated)"; }
-static inline hipError_t hipGetDevice(int*) { return hipErrorNoDevice; }
-static inline hipError_t hipDeviceGetAttribute(int*, hipDeviceAttribute_t, int) { return hipErrorNoDevice; }
+// There is no device, unless the environment names a number of compute units (RI_EMU_COMPUTE_UNITS): then
+// there is one, of that size, so that the rules which size launches by the machine choose on a few thousand keys
+// what they choose on an MI355X from tens of thousands on.
+static inline int emu_compute_units() {
+    const char* s = getenv("RI_EMU_COMPUTE_UNITS");
+    return s ? atoi(s) : 0;
+}
+static inline hipError_t hipGetDevice(int* dev) {
+    if (emu_compute_units() <= 0) return hipErrorNoDevice;
+    *dev = 0;
+    return hipSuccess;
+}
+static inline hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t, int) {
+    if (emu_compute_units() <= 0) return hipErrorNoDevice;
+    *value = emu_compute_units();
+    return hipSuccess;
+}
 template <class T>
 static inline hipError_t hipGetSymbolAddress(void** p, T& symbol) { *p = (void*)&symbol; return hipSuccess; }
 static inline hipError_t hipMalloc(void**, size_t) { return hipErrorNoDevice; }

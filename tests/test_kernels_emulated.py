@@ -28,6 +28,15 @@ def _run(args, env_extra=None, timeout=1500):
     return subprocess.run([sys.executable, *args], capture_output=True, text=True, env=env, cwd=ROOT, timeout=timeout)
 
 
+def _workers():
+    """A few processes side by side where the plugin for that is installed."""
+    try:
+        import xdist  # noqa: F401
+        return ["-n", str(max(1, min(4, (os.cpu_count() or 2) // 2)))]
+    except ImportError:
+        return []
+
+
 def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages():
     from rust_inference_amd.errors import KernelError
     try:
@@ -36,16 +45,36 @@ def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages():
         emulated.library()
     except KernelError as e:
         pytest.skip(f"no CPU build of the kernels here: {e}")
-    workers = []
-    try:                                   # a few processes side by side where the plugin for that is installed
-        import xdist  # noqa: F401
-        workers = ["-n", str(max(1, min(4, (os.cpu_count() or 2) // 2)))]
-    except ImportError:
-        pass
-    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", *workers, os.path.join(HERE, "test_kernels_gpu.py"),
+    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", *_workers(), os.path.join(HERE, "test_kernels_gpu.py"),
                 "-k", SELECT])
     assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-3000:]
     assert " passed" in run.stdout and "[emu]" not in run.stderr
+
+
+# With one compute unit every launch "fills the machine": the prompt attention keeps its tiles of 32 and 64 rows a
+# wavefront (on 256 units the small cases above all run with the smallest), and the wide product plans for one unit.
+ONE_UNIT = ("one_run or mfma_prefill_attention or (mfma_attention_window_edges and prefill) or "
+            "(mfma_attention_finds_one_far_key and prefill) or (wide_packed and not 4096 and not 12288 and not 5120 "
+            "and not (1000 and not (1000-1024-33 or 1000-1024-64)))")
+
+
+@pytest.mark.parametrize("units, tests", [(16, 4), (1, 31)])
+def test_the_forms_that_a_large_step_chooses_on_a_machine_made_small(units, tests):
+    """tests/small_machine_kernels.py: the emulated runtime reports a few compute units, so that the walk in runs, the
+    joins of many pieces and the run of more than 1,024 pages are chosen for one or two heads; with one unit also
+    the kernel tests whose launches are sized by the machine."""
+    from rust_inference_amd.errors import KernelError
+    try:
+        sys.path.insert(0, HERE)
+        import emulated
+        emulated.library()
+    except KernelError as e:
+        pytest.skip(f"no CPU build of the kernels here: {e}")
+    more = [os.path.join(HERE, "test_kernels_gpu.py"), "-k", ONE_UNIT, *_workers()] if units == 1 else []
+    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", os.path.join(HERE, "small_machine_kernels.py"), *more],
+               {"RI_EMU_COMPUTE_UNITS": str(units)})
+    assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-3000:]
+    assert f"{tests} passed" in run.stdout and "[emu]" not in run.stderr, run.stdout[-2000:]
 
 
 # The product for 17 to 64 rows once read a tile of x that its buffer does not have (33 to 48 rows are three
