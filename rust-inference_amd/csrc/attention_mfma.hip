@@ -762,21 +762,23 @@ __device__ __forceinline__ void finish_head(bf16_t* dst_lds, const HeadLoads<DH>
 // kernel writes the output itself and no join follows, with more the runs' results go to the workspace
 // [seqs, heads, splits, DH + 2] and the join adds them in run order (more than 16 of them in eight groups
 // side by side, as it does with chunks).
-#define STREAM_WAVES 4
+// W wavefronts a workgroup: four, two workgroups a compute unit, where the step has workgroups enough; eight in
+// one workgroup a compute unit for steps of short sequences that have one run for every compute unit but not
+// two (a wavefront's walk is then half as long, and there is no join).
 
 // FUSED: qkv is the raw projection; the kernel norms and rotates the group's queries for itself, and the
 // workgroup whose run ends at the new token's position makes the new key and value and stores them into their
 // page before any page is read.
-template <int DH, bool FUSED>
-__global__ void __launch_bounds__(STREAM_WAVES * 64, 2)
+template <int DH, bool FUSED, int W>
+__global__ void __launch_bounds__(W * 64, W == 4 ? 2 : 1)
 attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride,
                           const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
                           const float* __restrict__ inv_freq, bf16_t* k_pages, bf16_t* v_pages,
                           const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
                           int heads, int kv_heads, int window, float scale_log2, int splits, int tiled) {
     static_assert(!FUSED || DH <= 128, "one (d, d + DH/2) pair per lane");
-    __shared__ float o_lds[STREAM_WAVES][DH * 17];
-    __shared__ float ml_lds[STREAM_WAVES][2][16];
+    __shared__ float o_lds[W][DH * 17];
+    __shared__ float ml_lds[W][2][16];
     __shared__ __attribute__((aligned(16))) bf16_t q_lds[FUSED ? 16 : 1][DH];
     __shared__ __attribute__((aligned(16))) bf16_t knew[DH];
     const int lane = threadIdx.x & 63;
@@ -792,7 +794,7 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     const int p_last = min(c1 * (DECODE_CHUNK / PAGE) + DECODE_CHUNK / PAGE - 1, qpos / PAGE);   // below p_first: an empty run
     const int32_t* table = page_table + (long)b * table_width;
 
-    // This wavefront's pages are p_first + wave + STREAM_WAVES * j, j = 0 .. n_mine - 1, taken in blocks of
+    // This wavefront's pages are p_first + wave + W * j, j = 0 .. n_mine - 1, taken in blocks of
     // 64 * HELD: lane l of held[i] holds the table's entry for page j = block + 64 * i + l of the block, fetched
     // before the block begins, so that a page's address never waits for a trip to memory of its own.  No load
     // of the walk sits in a branch (the compiler counts loads in flight only along code without branches, and
@@ -800,13 +802,13 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     // is pulled back to the last page, an entry that is not mapped reads page 0, and neither is used.
     constexpr int HELD = 4;
     const int mine = p_first + wave;
-    const int n_mine = mine <= p_last ? (p_last - mine) / STREAM_WAVES + 1 : 0;
+    const int n_mine = mine <= p_last ? (p_last - mine) / W + 1 : 0;
     int held[HELD];
     auto fetch_table = [&](int j0) {
 #pragma unroll
         for (int i = 0; i < HELD; ++i) {
             const int j = min(j0 + 64 * i + lane, max(n_mine - 1, 0));
-            held[i] = max(table[min(mine + STREAM_WAVES * j, table_width - 1)], 0);
+            held[i] = max(table[min(mine + W * j, table_width - 1)], 0);
         }
     };
     auto phys_of = [&](int r) -> long {                      // r: the page's number inside the block
@@ -829,25 +831,25 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
     if (FUSED) {
         const bf16_t* row = qkv + (long)b * q_stride;
         const int page_new = qpos / PAGE;
-        HeadLoads<DH> hq[4];                                 // up to 16 query heads a kv head: four a wavefront
+        HeadLoads<DH> hq[16 / W];                            // up to 16 query heads a kv head: 16 / W a wavefront
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            hq[i] = fetch_head<DH>(row + (kvh * group + min(wave + STREAM_WAVES * i, group - 1)) * DH, q_gain, inv_freq, lane);
+        for (int i = 0; i < 16 / W; ++i)
+            hq[i] = fetch_head<DH>(row + (kvh * group + min(wave + W * i, group - 1)) * DH, q_gain, inv_freq, lane);
         const HeadLoads<DH> hk = fetch_head<DH>(row + (heads + kvh) * DH, k_gain, inv_freq, lane);
         const bf16_t* v_row = row + (heads + kv_heads + kvh) * DH;
         const bf16_t v0 = v_row[lane & (DH - 1)], v1 = v_row[(lane + 64) & (DH - 1)];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (wave + STREAM_WAVES * i < group)
-                finish_head<DH>(q_lds[wave + STREAM_WAVES * i], hq[i], q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
+        for (int i = 0; i < 16 / W; ++i)
+            if (wave + W * i < group)
+                finish_head<DH>(q_lds[wave + W * i], hq[i], q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
         if (p_first <= p_last && p_last == page_new) {       // this run holds the new token's position
             const int slot = qpos % PAGE;
             const long head_base = ((long)table[page_new] * kv_heads + kvh) * (long)(PAGE * DH);
-            if (wave == STREAM_WAVES - 1) {                  // the key: norm, rotation, into its page
+            if (wave == W - 1) {                  // the key: norm, rotation, into its page
                 finish_head<DH>(knew, hk, k_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
                 __builtin_amdgcn_wave_barrier();
                 for (int d = lane; d < DH; d += 64) k_pages[head_base + (long)slot * DH + d] = knew[d];
-            } else if (wave == STREAM_WAVES - 2) {           // the value: a copy, transposed inside the page
+            } else if (wave == W - 2) {           // the value: a copy, transposed inside the page
                 if (lane < DH) v_pages[head_base + (long)lane * PAGE + slot] = v0;
                 if (lane + 64 < DH) v_pages[head_base + (long)(lane + 64) * PAGE + slot] = v1;
             }
@@ -874,7 +876,7 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
         const int n_blk = min(n_mine - j0, 64 * HELD);
         load_page<DH>(fa, k_pages, v_pages, phys_of(0), kv_heads, kvh, lane);
         for (int r = 0; r < n_blk; r += 2) {
-            const int pa = mine + STREAM_WAVES * (j0 + r), pb = pa + STREAM_WAVES;
+            const int pa = mine + W * (j0 + r), pb = pa + W;
             load_page<DH>(fb, k_pages, v_pages, phys_of(min(r + 1, n_blk - 1)), kv_heads, kvh, lane, r + 1 < n_blk);
             process_page<DH, 1>(c, fa, pa, lane, scale_log2, open_page(pa));
             load_page<DH>(fa, k_pages, v_pages, phys_of(min(r + 2, n_blk - 1)), kv_heads, kvh, lane, r + 2 < n_blk);
@@ -892,14 +894,14 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
         ml_lds[wave][1][col] = c.l[0];
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < group * DH; idx += STREAM_WAVES * 64) {
+    for (int idx = threadIdx.x; idx < group * DH; idx += W * 64) {
         const int g = idx / DH, d = idx - g * DH;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < STREAM_WAVES; ++w) m = fmaxf(m, ml_lds[w][0][g]);
+        for (int w = 0; w < W; ++w) m = fmaxf(m, ml_lds[w][0][g]);
         float acc = 0.f, l = 0.f;
 #pragma unroll
-        for (int w = 0; w < STREAM_WAVES; ++w) {              // always in wavefront order
+        for (int w = 0; w < W; ++w) {              // always in wavefront order
             const float mw = ml_lds[w][0][g];
             const float f2 = mw == -INFINITY ? 0.f : exp2f(mw - m);
             acc += o_lds[w][d * 17 + g] * f2;
@@ -938,10 +940,24 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 #define STREAM_MIN_PER_CU 2
 #define STREAM_MIN_CHUNKS 8
 #define STREAM_JOINED_FROM 64
+// Eight wavefronts a workgroup and one run a sequence: from one workgroup per compute unit on, for sequences of
+// up to STREAM_WIDE_MAX_CHUNKS chunks.  Measured against the chunks and their join: with 256 (sequence, kv head)
+// pairs a small model's step is 4% shorter (32 sequences of 16 to 1,300 keys) and one at Qwen3-8B sizes 2.6% (32
+// of 1,900), with 384 pairs of 900 keys level; with 128 pairs, half the compute units, 6 to 9% longer (the units
+// that walk pull no faster for the others being idle), so those stay with the chunks.
+#ifndef STREAM_WIDE_MAX_CHUNKS
+#define STREAM_WIDE_MAX_CHUNKS 8
+#endif
+static bool stream_wide(int seqs, int kv_heads, int max_chunks) {
+    const long rows = (long)seqs * kv_heads;
+    const long cus = ri_compute_units();
+    return rows >= cus && rows < STREAM_MIN_PER_CU * cus && max_chunks <= STREAM_WIDE_MAX_CHUNKS;
+}
+
 static int stream_splits(int seqs, int kv_heads, int max_chunks) {
     const long rows = (long)seqs * kv_heads;
     const long cus = ri_compute_units();
-    if (rows >= STREAM_MIN_PER_CU * cus) return 1;
+    if (rows >= STREAM_MIN_PER_CU * cus || stream_wide(seqs, kv_heads, max_chunks)) return 1;
     if (max_chunks < STREAM_JOINED_FROM) return 0;
     const long splits = min((STREAM_WORKGROUPS_PER_CU * cus + rows - 1) / rows, (long)max_chunks / STREAM_MIN_CHUNKS);
     if (splits < 2 || rows * splits < STREAM_MIN_PER_CU * cus) return 0;
@@ -1184,14 +1200,21 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
     const int splits = stream_splits(seqs, kv_heads, max_chunks);
+    const bool wide = stream_wide(seqs, kv_heads, max_chunks);
     if (splits > 0) {
         dim3 sgrid(seqs, kv_heads, splits);
 #define RI_STREAM_CASE(DH)                                                                                        \
     case DH:                                                                                                      \
-        attn_decode_stream_kernel<DH, false><<<sgrid, STREAM_WAVES * 64, 0, s>>>(                                 \
-            (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,                \
-            (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,        \
-            scale_log2, splits, tiled_out);                                                                       \
+        if (wide)                                                                                                 \
+            attn_decode_stream_kernel<DH, false, 8><<<sgrid, 8 * 64, 0, s>>>(                                     \
+                (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,            \
+                (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
+                scale_log2, splits, tiled_out);                                                                   \
+        else                                                                                                      \
+            attn_decode_stream_kernel<DH, false, 4><<<sgrid, 4 * 64, 0, s>>>(                                     \
+                (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, nullptr, nullptr, 0.f, nullptr,            \
+                (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
+                scale_log2, splits, tiled_out);                                                                   \
         if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {
@@ -1241,14 +1264,21 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
     const int splits = stream_splits(seqs, kv_heads, max_chunks);
+    const bool wide = stream_wide(seqs, kv_heads, max_chunks);
     if (splits > 0) {
         dim3 sgrid(seqs, kv_heads, splits);
 #define RI_STREAM_CASE(DH)                                                                                        \
     case DH:                                                                                                      \
-        attn_decode_stream_kernel<DH, true><<<sgrid, STREAM_WAVES * 64, 0, s>>>(                                  \
-            (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,                 \
-            (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,        \
-            scale_log2, splits, tiled_out);                                                                       \
+        if (wide)                                                                                                 \
+            attn_decode_stream_kernel<DH, true, 8><<<sgrid, 8 * 64, 0, s>>>(                                      \
+                (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,             \
+                (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
+                scale_log2, splits, tiled_out);                                                                   \
+        else                                                                                                      \
+            attn_decode_stream_kernel<DH, true, 4><<<sgrid, 4 * 64, 0, s>>>(                                      \
+                (bf16_t*)out, workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq,             \
+                (bf16_t*)k_pages, (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window,    \
+                scale_log2, splits, tiled_out);                                                                   \
         if (splits > 1) launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, -1, splits, tiled_out, s); \
         break;
         switch (head_dim) {

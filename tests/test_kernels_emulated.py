@@ -19,7 +19,7 @@ HERE = os.path.join(ROOT, "tests")
 # when emulated); every kernel and every form of it is still run, at the smaller sizes of the same tests.
 SELECT = ("not 4096 and not 12288 and not 5120 and not 5000 and not very_long and not more_pages_than and not thousands "
           "and not (many_sequences and not (16-8-32-100 or 16-8-32-40)) and not (in_runs and not 8-8-32) "
-          "and not (wide_packed and 1000 and not (1000-1024-33 or 1000-1024-64))")
+          "and not (wide_packed and 1000 and not (1000-1024-33 or 1000-1024-64)) and not (eight_wavefronts and 128)")
 
 
 def _run(args, env_extra=None, timeout=1500):

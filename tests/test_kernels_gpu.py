@@ -425,6 +425,42 @@ def test_mfma_decode_attention_streams_over_many_sequences(ops, heads, kv_heads,
     close(out, want, BF16_OUT, f"streaming decode attention, window {window}")
 
 
+WIDE_LENS = [1, 32, 33, 256, 257, 512, 700, 5, 1025, 1200, 1199, 31, 64, 1024, 300, 97,
+             2, 63, 65, 100, 129, 255, 258, 400, 511, 513, 640, 767, 769, 900, 1000, 1100]
+
+
+@pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 100), (32, 8, 128, None),
+                                                         (16, 8, 128, 300), (8, 8, 64, None)])
+def test_mfma_decode_attention_streams_short_sequences_with_eight_wavefronts(ops, heads, kv_heads, dh, window):
+    """Thirty-two sequences of eight kv heads and up to 1,200 keys: a run for every compute unit but not two, and
+    no sequence longer than eight chunks, is walked in one run by workgroups of eight wavefronts; some of the
+    sequences have fewer pages than wavefronts."""
+    if ops.compute_units() != 256:
+        pytest.skip("the rule is written for the machine's size")
+    rng = np.random.default_rng(78)
+    assert ops.decode_attention_runs(len(WIDE_LENS), kv_heads, max(WIDE_LENS) + 300) == 1
+    assert ops.decode_attention_runs(len(WIDE_LENS) - 1, kv_heads, max(WIDE_LENS) + 300) == 0
+    assert ops.decode_attention_runs(len(WIDE_LENS), kv_heads, 2049) == 0
+
+    def boost(qkv, k, kp, table):
+        head = 3 * (heads // kv_heads)                                 # sequence 9, kv head 3: its first query head
+        kf = f64(kp[table[9, 40 // 32].item(), 3, 40 % 32])
+        qkv[9, head * dh:(head + 1) * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+    out, want = attention_case(ops, rng, WIDE_LENS, [1] * len(WIDE_LENS), heads, kv_heads, dh, torch.bfloat16,
+                               window=window, boost=boost, kernel="decode")
+    close(out, want, BF16_OUT, f"eight wavefronts a run, window {window}")
+
+
+@pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 40), (32, 8, 128, None),
+                                                         (16, 8, 128, 40), (128, 8, 64, None)])
+def test_fused_decode_attention_streams_short_sequences_with_eight_wavefronts(ops, heads, kv_heads, dh, window):
+    """The same from the raw projection (two query heads a wavefront to norm where a kv head has sixteen)."""
+    if ops.compute_units() != 256:
+        pytest.skip("the rule is written for the machine's size")
+    assert ops.decode_attention_runs(len(WIDE_LENS), kv_heads, max(WIDE_LENS) + 301) == 1
+    fused_decode_case(ops, heads, kv_heads, dh, window, WIDE_LENS, steps=2 if dh == 32 else 1, repeats=2 if dh == 32 else 1)
+
+
 @pytest.mark.parametrize("window", [None, 4500])
 def test_mfma_decode_attention_streams_long_sequences_in_runs(ops, window):
     """Long sequences with 64 (sequence, kv head) pairs and more are cut into 16 runs of whole chunks each, by
