@@ -763,8 +763,8 @@ __device__ __forceinline__ void finish_head(bf16_t* dst_lds, const HeadLoads<DH>
 // [seqs, heads, splits, DH + 2] and the join adds them in run order (more than 16 of them in eight groups
 // side by side, as it does with chunks).
 // W wavefronts a workgroup: four, two workgroups a compute unit, where the step has workgroups enough; eight in
-// one workgroup a compute unit for steps of short sequences that have one run for every compute unit but not
-// two (a wavefront's walk is then half as long, and there is no join).
+// one workgroup a compute unit for steps that have one run for every compute unit and few more (a wavefront's
+// walk is then half as long, and there is no join).
 
 // FUSED: qkv is the raw projection; the kernel norms and rotates the group's queries for itself, and the
 // workgroup whose run ends at the new token's position makes the new key and value and stores them into their
@@ -940,18 +940,20 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 #define STREAM_MIN_PER_CU 2
 #define STREAM_MIN_CHUNKS 8
 #define STREAM_JOINED_FROM 64
-// Eight wavefronts a workgroup and one run a sequence: from one workgroup per compute unit on, for sequences of
-// up to STREAM_WIDE_MAX_CHUNKS chunks.  Measured against the chunks and their join: with 256 (sequence, kv head)
-// pairs a small model's step is 4% shorter (32 sequences of 16 to 1,300 keys) and one at Qwen3-8B sizes 2.6% (32
-// of 1,900), with 384 pairs of 900 keys level; with 128 pairs, half the compute units, 6 to 9% longer (the units
-// that walk pull no faster for the others being idle), so those stay with the chunks.
+// Eight wavefronts a workgroup and one run a sequence: where the step has one workgroup for every compute unit and
+// few more (up to an eighth), for sequences of up to STREAM_WIDE_MAX_CHUNKS chunks.  Measured against the chunks
+// and their join, at 8 kv heads: with 256 (sequence, kv head) pairs a small model's step is 4% shorter (32
+// sequences of 16 to 1,300 keys) and one at Qwen3-8B sizes 2.4 to 4.4% (32 of 1,900, 2,100 and 3,600); with 384
+// pairs, a second round on half the compute units, level at 900 keys and 2.4% longer at 2,100; with 320 pairs of
+// 6,000 keys 3.5% longer; with 128 pairs, half the compute units, 6 to 9% longer (the units that walk pull no
+// faster for the others being idle).
 #ifndef STREAM_WIDE_MAX_CHUNKS
-#define STREAM_WIDE_MAX_CHUNKS 8
+#define STREAM_WIDE_MAX_CHUNKS 16
 #endif
 static bool stream_wide(int seqs, int kv_heads, int max_chunks) {
     const long rows = (long)seqs * kv_heads;
     const long cus = ri_compute_units();
-    return rows >= cus && rows < STREAM_MIN_PER_CU * cus && max_chunks <= STREAM_WIDE_MAX_CHUNKS;
+    return rows >= cus && rows <= cus + cus / 8 && rows < STREAM_MIN_PER_CU * cus && max_chunks <= STREAM_WIDE_MAX_CHUNKS;
 }
 
 static int stream_splits(int seqs, int kv_heads, int max_chunks) {

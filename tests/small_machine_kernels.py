@@ -70,6 +70,21 @@ def test_more_than_sixteen_chunks_are_joined_in_runs(ops):
         close(out, want, BF16_OUT, f"chunks, far key {far}, window {window}")
 
 
+@pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (8, 8, 64, 100), (128, 8, 64, None)])
+def test_one_run_for_every_compute_unit_walks_with_eight_wavefronts(ops, heads, kv_heads, dh, window):
+    """Two sequences of eight kv heads on sixteen compute units: a run for each, walked by eight wavefronts, from
+    the normed queries and from the raw projection (sixteen query heads a kv head: two for a wavefront to norm)."""
+    machine(ops, 16)
+    lens = [1200, 33]
+    assert ops.decode_attention_runs(2, kv_heads, max(lens) + 301) == 1      # (too few pairs for the walk by four)
+    assert ops.decode_attention_runs(3, kv_heads, max(lens) + 301) == 0
+    if heads <= 16:
+        out, want = attention_case(ops, np.random.default_rng(dh), lens, [1, 1], heads, kv_heads, dh, torch.bfloat16,
+                                   window=window, boost=far_key(0, 3, 3 * (heads // kv_heads), dh, 40), kernel="decode")
+        close(out, want, BF16_OUT, f"eight wavefronts a run, window {window}")
+    fused_decode_case(ops, heads, kv_heads, dh, window, lens, steps=2, repeats=1)
+
+
 def test_one_run_of_more_pages_than_a_wavefront_holds_table_entries_for(ops):
     """A wavefront fetches the table's entries for 256 of its pages at a time; in one run of more than 1,024
     pages it goes round that loop again.  Two sequences on a machine of one compute unit: one run each."""
