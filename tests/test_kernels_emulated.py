@@ -9,6 +9,7 @@ runs a few thousand matrix instructions a second)."""
 import os
 import subprocess
 import sys
+import tempfile
 
 import pytest
 
@@ -23,47 +24,44 @@ SELECT = ("not 4096 and not 12288 and not 5120 and not 5000 and not very_long an
           "and not (wide_packed and 1000 and not (1000-1024-33 or 1000-1024-64)) and not eight_wavefronts")
 
 
-def _run(args, env_extra=None, timeout=1500):
-    env = dict(os.environ, RI_TEST_KERNELS="emulated", **(env_extra or {}))
+def _env(extra=None):
+    env = dict(os.environ, RI_TEST_KERNELS="emulated", **(extra or {}))
     env.pop("RI_KERNEL_LIBRARY", None)
-    return subprocess.run([sys.executable, *args], capture_output=True, text=True, env=env, cwd=ROOT, timeout=timeout)
+    return env
 
 
-def _workers():
+def _run(args, env_extra=None, timeout=1500):
+    return subprocess.run([sys.executable, *args], capture_output=True, text=True, env=_env(env_extra), cwd=ROOT,
+                          timeout=timeout)
+
+
+def _start(args, env_extra=None):
+    """The same in the background, its output in files (a pipe that fills up would stop it)."""
+    out, err = tempfile.TemporaryFile("w+"), tempfile.TemporaryFile("w+")
+    return subprocess.Popen([sys.executable, *args], stdout=out, stderr=err, text=True, env=_env(env_extra), cwd=ROOT), out, err
+
+
+def _workers(most):
     """A few processes side by side where the plugin for that is installed."""
     try:
         import xdist  # noqa: F401
-        return ["-n", str(max(1, min(4, (os.cpu_count() or 2) // 2)))]
+        return ["-n", str(max(1, min(most, (os.cpu_count() or 2) // 2)))]
     except ImportError:
         return []
 
 
-def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages():
-    from rust_inference_amd.errors import KernelError
-    try:
-        sys.path.insert(0, HERE)
-        import emulated
-        emulated.library()
-    except KernelError as e:
-        pytest.skip(f"no CPU build of the kernels here: {e}")
-    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", *_workers(), os.path.join(HERE, "test_kernels_gpu.py"),
-                "-k", SELECT])
-    assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-3000:]
-    assert " passed" in run.stdout and "[emu]" not in run.stderr
-
-
 # With one compute unit every launch "fills the machine": the prompt attention keeps its tiles of 32 and 64 rows a
-# wavefront (on 256 units the small cases above all run with the smallest), and the wide product plans for one unit.
+# wavefront (on 256 units the small cases all run with the smallest), and the wide product plans for one unit.
 ONE_UNIT = ("one_run or mfma_prefill_attention or (mfma_attention_window_edges and prefill) or "
             "(mfma_attention_finds_one_far_key and prefill) or (wide_packed and not 4096 and not 12288 and not 5120 "
             "and not (1000 and not (1000-1024-33 or 1000-1024-64)))")
+PYTEST = ["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider"]
+KERNEL_TESTS, SMALL_MACHINE = os.path.join(HERE, "test_kernels_gpu.py"), os.path.join(HERE, "small_machine_kernels.py")
 
 
-@pytest.mark.parametrize("units, tests", [(16, 7), (1, 31)])
-def test_the_forms_that_a_large_step_chooses_on_a_machine_made_small(units, tests):
-    """tests/small_machine_kernels.py: the emulated runtime reports a few compute units, so that the walk in runs, the
-    joins of many pieces and the run of more than 1,024 pages are chosen for one or two heads; with one unit also
-    the kernel tests whose launches are sized by the machine."""
+@pytest.fixture(scope="module")
+def runs():
+    """The three emulated runs, side by side (each is a pytest of its own; together they take what the longest takes)."""
     from rust_inference_amd.errors import KernelError
     try:
         sys.path.insert(0, HERE)
@@ -71,11 +69,41 @@ def test_the_forms_that_a_large_step_chooses_on_a_machine_made_small(units, test
         emulated.library()
     except KernelError as e:
         pytest.skip(f"no CPU build of the kernels here: {e}")
-    more = [os.path.join(HERE, "test_kernels_gpu.py"), "-k", ONE_UNIT, *_workers()] if units == 1 else []
-    run = _run(["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider", os.path.join(HERE, "small_machine_kernels.py"), *more],
-               {"RI_EMU_COMPUTE_UNITS": str(units)})
-    assert run.returncode == 0, run.stdout[-3000:] + run.stderr[-3000:]
-    assert f"{tests} passed" in run.stdout and "[emu]" not in run.stderr, run.stdout[-2000:]
+    started = {
+        "kernel tests": _start([*PYTEST, *_workers(4), KERNEL_TESTS, "-k", SELECT]),
+        "sixteen units": _start([*PYTEST, SMALL_MACHINE], {"RI_EMU_COMPUTE_UNITS": "16"}),
+        "one unit": _start([*PYTEST, *_workers(2), SMALL_MACHINE, KERNEL_TESTS, "-k", ONE_UNIT], {"RI_EMU_COMPUTE_UNITS": "1"}),
+    }
+    done = {}
+    try:
+        for name, (proc, out, err) in started.items():
+            proc.wait(timeout=1500)
+            out.seek(0), err.seek(0)
+            done[name] = (proc.returncode, out.read(), err.read())
+    finally:
+        for proc, out, err in started.values():
+            if proc.poll() is None:
+                proc.kill()
+            out.close(), err.close()
+    return done
+
+
+def _passed(run, tests=None):
+    code, out, err = run
+    assert code == 0, out[-3000:] + err[-3000:]
+    assert (f"{tests} passed" if tests else " passed") in out and "[emu]" not in err, out[-2000:]
+
+
+def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages(runs):
+    _passed(runs["kernel tests"])
+
+
+@pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 31)])
+def test_the_forms_that_a_large_step_chooses_on_a_machine_made_small(runs, units, tests):
+    """tests/small_machine_kernels.py: the emulated runtime reports a few compute units, so that the walk in runs, the
+    joins of many pieces and the run of more than 1,024 pages are chosen for one or two heads; with one unit also
+    the kernel tests whose launches are sized by the machine."""
+    _passed(runs[units], tests)
 
 
 # The product for 17 to 64 rows once read a tile of x that its buffer does not have (33 to 48 rows are three
