@@ -946,7 +946,8 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 // sequences of 16 to 1,300 keys) and one at Qwen3-8B sizes 2.4 to 4.4% (32 of 1,900, 2,100 and 3,600); with 384
 // pairs, a second round on half the compute units, level at 900 keys and 2.4% longer at 2,100; with 320 pairs of
 // 6,000 keys 3.5% longer; with 128 pairs, half the compute units, 6 to 9% longer (the units that walk pull no
-// faster for the others being idle).
+// faster for the others being idle), and in two runs a sequence with a join, a workgroup for every unit again,
+// still 1 to 5% longer than the chunks.
 #ifndef STREAM_WIDE_MAX_CHUNKS
 #define STREAM_WIDE_MAX_CHUNKS 16
 #endif
