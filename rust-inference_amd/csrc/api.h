@@ -63,10 +63,13 @@ int ri_attention_prefill_bf16(void* out, const void* qkv, int q_stride, const vo
                               int table_width, int seqs, int max_new, int heads, int kv_heads, int head_dim,
                               int page_size, int window, float scale, void* stream);
 
-// Decode form: exactly one new token per sequence; keys in chunks of 256, joined by a second kernel.
-// workspace: float32 [seqs, heads, max_chunks, head_dim + 2]; max_chunks >= ri_attention_decode_chunks(longest
-// sequence after this step); at most 16 query heads per kv head.
+// Decode form: exactly one new token per sequence; keys in chunks of 256 (in a step of few workgroups each cut into
+// 2 or 4 pieces), joined by a second kernel.
+// workspace: float32 [seqs, heads, max_chunks * pieces, head_dim + 2]; max_chunks >= ri_attention_decode_chunks(longest
+// sequence after this step), pieces = ri_attention_decode_pieces(seqs, kv_heads, heads, max_chunks); at most 16
+// query heads per kv head.
 int ri_attention_decode_chunks(int max_len);
+int ri_attention_decode_pieces(int seqs, int kv_heads, int heads, int max_chunks);
 // Whether ri_attention_decode_bf16 takes a step of this size with its streaming kernel (a workgroup walks a
 // whole run of a sequence's pages; no join when a sequence is one run): the number of runs per sequence, or
 // 0 for one workgroup per chunk.

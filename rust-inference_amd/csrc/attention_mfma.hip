@@ -44,8 +44,9 @@ union Frag {
 };
 
 #define PAGE 32
-#define DECODE_CHUNK 256          // keys per workgroup of the decode kernel: 8 pages
+#define DECODE_CHUNK 256          // keys per workgroup of the decode kernel: 8 pages; the unit of every count of chunks
 #define DECODE_WAVES 8            // wavefronts of a decode workgroup: one page each
+// (a step with few workgroups cuts every chunk into 2 or 4 pieces, workgroups of 4 or 2 wavefronts: CW below)
 
 // The maximum over the four lanes of a column (lanes l, l ^ 16, l ^ 32, l ^ 48), in every one of them, by the
 // two lane-swap instructions of gfx950: v_permlane32_swap exchanges the upper half of its first operand with
@@ -501,14 +502,15 @@ attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qk
 
 // ------------------------------------------------------------------ decode: chunks of 256 keys, then a join
 // Workspace: [seqs, heads, max_chunks, DH + 2] float32: the unnormalised output, then m and l.
-template <int DH>
-__global__ void __launch_bounds__(DECODE_WAVES * 64)
+// CW: wavefronts, and pages, of a workgroup; `chunk` counts pieces of CW pages, `max_chunks` such pieces.
+template <int DH, int CW>
+__global__ void __launch_bounds__(CW * 64)
 attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride,
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
                         int heads, int kv_heads, int window, float scale_log2, int max_chunks) {
-    __shared__ float o_lds[DECODE_WAVES][DH * 17];           // [d * 17 + col]: no bank conflicts either way
-    __shared__ float ml_lds[DECODE_WAVES][2][16];
+    __shared__ float o_lds[CW][DH * 17];           // [d * 17 + col]: no bank conflicts either way
+    __shared__ float ml_lds[CW][2][16];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int b = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;      // chunks last: the empty ones start last
@@ -516,11 +518,11 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
     const int tok = b;                                       // one new token per sequence: token b is sequence b's
     // The position and this wavefront's entry of the page table are asked for together: neither address
     // depends on the other's value, and each is a trip to memory that the page's loads would wait for in turn.
-    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;   // this wavefront's page
+    const int page = chunk * CW + wave;   // this wavefront's page
     const int qpos = tok_pos[tok];
     const int phys = max(page_table[(long)b * table_width + min(page, table_width - 1)], 0);   // not mapped: page 0, unused
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
+    if (chunk * (CW * PAGE) > qpos || chunk * (CW * PAGE) + CW * PAGE - 1 < lo) return;   // whole workgroup
 
     // No load sits in a branch (the compiler counts loads in flight only along code without branches): a
     // wavefront without a page of its own fetches page `phys` all the same, a lane without a column the
@@ -555,14 +557,14 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
         ml_lds[wave][1][col] = c.l[0];
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < group * DH; idx += DECODE_WAVES * 64) {
+    for (int idx = threadIdx.x; idx < group * DH; idx += CW * 64) {
         const int g = idx / DH, d = idx - g * DH;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, ml_lds[w][0][g]);
+        for (int w = 0; w < CW; ++w) m = fmaxf(m, ml_lds[w][0][g]);
         float acc = 0.f, l = 0.f;
 #pragma unroll
-        for (int w = 0; w < DECODE_WAVES; ++w) {
+        for (int w = 0; w < CW; ++w) {
             const float mw = ml_lds[w][0][g];
             const float f2 = mw == -INFINITY ? 0.f : exp2f(mw - m);
             acc += o_lds[w][d * 17 + g] * f2;
@@ -594,7 +596,7 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 template <int DH, int PB>
 __global__ void __launch_bounds__(DH * PB)
 attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
-                        int heads, int window, int max_chunks, int tiled) {
+                        int heads, int window, int max_chunks, int chunk_keys, int tiled) {
     __shared__ float part_o[JOIN_PARTS][DH];
     __shared__ float part_ml[JOIN_PARTS][2];
     const int b = blockIdx.x, h = blockIdx.y;                       // token b is sequence b's one new token
@@ -602,7 +604,7 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
     const int qpos = tok_pos[b];
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     // window < 0: the entries are the runs of the streaming kernel, all of them written
-    const int c_lo = window < 0 ? 0 : lo / DECODE_CHUNK, c_hi = window < 0 ? max_chunks - 1 : qpos / DECODE_CHUNK;
+    const int c_lo = window < 0 ? 0 : lo / chunk_keys, c_hi = window < 0 ? max_chunks - 1 : qpos / chunk_keys;
     const int n = c_hi - c_lo + 1;
     const int parts = n <= JOIN_SERIAL ? 1 : JOIN_PARTS;
     const int per = (n + parts - 1) / parts;
@@ -644,20 +646,20 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
     out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
 }
 
-// The join of up to JOIN_SERIAL chunks with every load asked for at once, before the position is known:
+// The join of up to CAP chunks (JOIN_SERIAL) with every load asked for at once, before the position is known:
 // the chunks' results and markers lie at places that depend on the grid alone, so one trip to memory
 // fetches them all (those of chunks the sequence has not reached are fetched and not used), where the
 // loop above makes three trips in turn (the position, the maxima, the results).  The same operations in
 // the same order as that loop: the results are equal bit for bit.
-template <int DH>
+template <int DH, int CAP>
 __global__ void __launch_bounds__(DH)
 attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
-                              int heads, int window, int max_chunks, int tiled) {
+                              int heads, int window, int max_chunks, int chunk_keys, int tiled) {
     const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
     const float* base = ws + ((long)b * heads + h) * max_chunks * (DH + 2);
-    float o[JOIN_SERIAL], mc[JOIN_SERIAL], lc[JOIN_SERIAL];
+    float o[CAP], mc[CAP], lc[CAP];
 #pragma unroll
-    for (int c = 0; c < JOIN_SERIAL; ++c) {
+    for (int c = 0; c < CAP; ++c) {
         o[c] = 0.f;
         mc[c] = -INFINITY;
         lc[c] = 0.f;
@@ -671,14 +673,14 @@ attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict_
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
     // window < 0: the entries are not chunks at fixed places but the runs of the streaming kernel, all of
     // them written (an empty run as a maximum of -inf)
-    const int c_lo = window < 0 ? 0 : lo / DECODE_CHUNK, c_hi = window < 0 ? max_chunks - 1 : qpos / DECODE_CHUNK;
+    const int c_lo = window < 0 ? 0 : lo / chunk_keys, c_hi = window < 0 ? max_chunks - 1 : qpos / chunk_keys;
     float m = -INFINITY;
 #pragma unroll
-    for (int c = 0; c < JOIN_SERIAL; ++c)
+    for (int c = 0; c < CAP; ++c)
         if (c >= c_lo && c <= c_hi) m = fmaxf(m, mc[c]);
     float acc = 0.f, l = 0.f;
 #pragma unroll
-    for (int c = 0; c < JOIN_SERIAL; ++c) {                          // always in chunk order
+    for (int c = 0; c < CAP; ++c) {                          // always in chunk order
         if (c >= c_lo && c <= c_hi) {
             const float f = mc[c] == -INFINITY ? 0.f : exp2f(mc[c] - m);
             acc += o[c] * f;
@@ -690,12 +692,13 @@ attn_decode_join_small_kernel(bf16_t* __restrict__ out, const float* __restrict_
 
 template <int DH>
 static void launch_join(bf16_t* out, const float* ws, const int32_t* tok_pos, int seqs, int heads, int window,
-                        int max_chunks, int tiled, hipStream_t s) {
+                        int max_chunks, int tiled, hipStream_t s, int chunk_keys = DECODE_CHUNK) {
     if (max_chunks <= JOIN_SERIAL)
-        attn_decode_join_small_kernel<DH><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window, max_chunks, tiled);
+        attn_decode_join_small_kernel<DH, JOIN_SERIAL><<<dim3(seqs, heads), DH, 0, s>>>(out, ws, tok_pos, heads, window,
+                                                                                     max_chunks, chunk_keys, tiled);
     else
         attn_decode_join_kernel<DH, JOIN_PARTS><<<dim3(seqs, heads), DH * JOIN_PARTS, 0, s>>>(out, ws, tok_pos, heads,
-                                                                                           window, max_chunks, tiled);
+                                                                                           window, max_chunks, chunk_keys, tiled);
 }
 
 // ------------------------------------------------------------------ decode: the new token's own q, k and v
@@ -980,16 +983,16 @@ extern "C" int ri_attention_decode_streams(int seqs, int kv_heads, int max_chunk
 // has just read from the page (the page in memory does not have them yet).  (Joining inside the same
 // kernel, by the workgroup that finishes last, was tried: the device-wide fences it needs write the
 // whole L2 back and cost many times what the second launch costs.)
-template <int DH>
-__global__ void __launch_bounds__(DECODE_WAVES * 64)
+template <int DH, int CW>
+__global__ void __launch_bounds__(CW * 64)
 attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, int q_stride, const float* __restrict__ q_gain,
                          const float* __restrict__ k_gain, float eps, const float* __restrict__ inv_freq,
                          bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages,
                          const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table, int table_width,
                          int heads, int kv_heads, int window, float scale_log2, int max_chunks) {
     static_assert(DH <= 128, "one (d, d + DH/2) pair per lane");
-    __shared__ float o_lds[DECODE_WAVES][DH * 17];
-    __shared__ float ml_lds[DECODE_WAVES][2][16];
+    __shared__ float o_lds[CW][DH * 17];
+    __shared__ float ml_lds[CW][2][16];
     __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][DH];
     __shared__ __attribute__((aligned(16))) bf16_t knew[DH];
     __shared__ __attribute__((aligned(16))) bf16_t vnew[DH];
@@ -1001,18 +1004,18 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
     // (two of the group's queries at most, and the new key), the new value, the position and this wavefront's
     // entry of the page table.  An entry that is not mapped reads page 0, which is never used then.
     const bf16_t* row = qkv + (long)b * q_stride;
-    const int g0 = min(wave, group - 1), g1 = min(wave + DECODE_WAVES, group - 1);
+    const int g0 = min(wave, group - 1), g1 = min(wave + CW, group - 1);
     const HeadLoads<DH> hq0 = fetch_head<DH>(row + (kvh * group + g0) * DH, q_gain, inv_freq, lane);
     const HeadLoads<DH> hq1 = fetch_head<DH>(row + (kvh * group + g1) * DH, q_gain, inv_freq, lane);
     const HeadLoads<DH> hk = fetch_head<DH>(row + (heads + kvh) * DH, k_gain, inv_freq, lane);
     const bf16_t* v_row = row + (heads + kv_heads + kvh) * DH;
     const bf16_t v0 = v_row[lane & (DH - 1)], v1 = v_row[(lane + 64) & (DH - 1)];
-    const int page = chunk * (DECODE_CHUNK / PAGE) + wave;
+    const int page = chunk * CW + wave;
     const int qpos = tok_pos[b];                             // token b is sequence b's one new token
     const int phys = max(page_table[(long)b * table_width + min(page, table_width - 1)], 0);
     const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
-    if (chunk * DECODE_CHUNK > qpos || chunk * DECODE_CHUNK + DECODE_CHUNK - 1 < lo) return;   // whole workgroup
-    const bool owner = chunk == qpos / DECODE_CHUNK;         // this chunk holds the new token's position
+    if (chunk * (CW * PAGE) > qpos || chunk * (CW * PAGE) + CW * PAGE - 1 < lo) return;   // whole workgroup
+    const bool owner = chunk == qpos / (CW * PAGE);         // this chunk holds the new token's position
 
     // 2. this wavefront's page is on its way while the queries are made (a wavefront without a page of its own
     // fetches page `phys` all the same and leaves it unused)
@@ -1023,16 +1026,16 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
 
     // 3. queries of the group; in the owner also the new key and value
     if (wave < group) finish_head<DH>(q_lds[wave], hq0, q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
-    if (wave + DECODE_WAVES < group)
-        finish_head<DH>(q_lds[wave + DECODE_WAVES], hq1, q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
+    if (wave + CW < group)
+        finish_head<DH>(q_lds[wave + CW], hq1, q_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
     if (owner) {
         const int slot = qpos % PAGE;
         const long head_base = (phys_new * kv_heads + kvh) * (long)(PAGE * DH);
-        if (wave == DECODE_WAVES - 1) {                      // the key: norm, rotation, into LDS and into its page
+        if (wave == CW - 1) {                      // the key: norm, rotation, into LDS and into its page
             finish_head<DH>(knew, hk, k_gain != nullptr, inv_freq != nullptr, eps, qpos, lane);
             __builtin_amdgcn_wave_barrier();
             for (int d = lane; d < DH; d += 64) k_pages[head_base + (long)slot * DH + d] = knew[d];
-        } else if (wave == DECODE_WAVES - 2) {               // the value: a copy, transposed inside the page
+        } else if (wave == CW - 2) {               // the value: a copy, transposed inside the page
             if (lane < DH) {
                 vnew[lane] = v0;
                 v_pages[head_base + (long)lane * PAGE + slot] = v0;
@@ -1091,14 +1094,14 @@ attn_decode_fused_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv,
         ml_lds[wave][1][col] = c.l[0];
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < group * DH; idx += DECODE_WAVES * 64) {
+    for (int idx = threadIdx.x; idx < group * DH; idx += CW * 64) {
         const int g = idx / DH, d = idx - g * DH;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, ml_lds[w][0][g]);
+        for (int w = 0; w < CW; ++w) m = fmaxf(m, ml_lds[w][0][g]);
         float acc = 0.f, l = 0.f;
 #pragma unroll
-        for (int w = 0; w < DECODE_WAVES; ++w) {
+        for (int w = 0; w < CW; ++w) {
             const float mw = ml_lds[w][0][g];
             const float f2 = mw == -INFINITY ? 0.f : exp2f(mw - m);
             acc += o_lds[w][d * 17 + g] * f2;
@@ -1188,6 +1191,32 @@ extern "C" int ri_attention_prefill_bf16(void* out, const void* qkv, int q_strid
 
 extern "C" int ri_attention_decode_chunks(int max_len) { return (max_len + DECODE_CHUNK - 1) / DECODE_CHUNK; }
 
+// Pieces that the chunk kernels cut every chunk into: 1, or 2 or 4 (workgroups of four or two wavefronts, one page
+// each) while the step's workgroups, counted by the bound on the lengths, stay within one for every compute unit and
+// the pieces of a sequence within what the join fetches at once.  A compute unit pulls its pages at a rate of its
+// own, so a step of few short sequences has a fraction of the machine fetch what all of it could: a small model's
+// step at batch 1, 2 and 4 is 1.6, 3.8 and 4.2% shorter for the cut (Qwen3-0.6B sizes; 600, 1,600 and 800 keys), one
+// sequence of 900 and of 1,500 keys at Qwen3-8B sizes 1.7 and 2.4%.  Past what the join fetches at once the cut loses
+// what it gains (one sequence of 2,100 keys at Qwen3-8B sizes in 18 pieces: 0.7% longer; in 36: 1.8%).  A workgroup norms two query
+// heads a wavefront at most, so a kv head's query heads bound the cut too.
+#ifndef DECODE_SPLIT_FILL
+#define DECODE_SPLIT_FILL 1
+#endif
+static int decode_pieces(int seqs, int kv_heads, int group, int max_chunks) {
+    if (stream_splits(seqs, kv_heads, max_chunks) > 0) return 1;
+    const long wgs = (long)seqs * kv_heads * max_chunks, cus = ri_compute_units();
+    int pieces = 1;
+    while (pieces < 4 && wgs * pieces * 2 <= DECODE_SPLIT_FILL * cus && max_chunks * pieces * 2 <= JOIN_SERIAL &&
+           group <= 2 * (DECODE_WAVES / (pieces * 2)))
+        pieces *= 2;
+    return pieces;
+}
+
+// The workspace of a decode attention call has room for max_chunks times this many results a sequence and head.
+extern "C" int ri_attention_decode_pieces(int seqs, int kv_heads, int heads, int max_chunks) {
+    return decode_pieces(seqs, kv_heads, heads / (kv_heads > 0 ? kv_heads : 1), max_chunks);
+}
+
 extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void* qkv, int q_stride,
                                         const void* k_pages, const void* v_pages, const int32_t* cu_seqlens,
                                         const int32_t* tok_pos, const int32_t* page_table, int table_width, int seqs,
@@ -1229,17 +1258,25 @@ extern "C" int ri_attention_decode_bf16(void* out, float* workspace, const void*
         RI_LAUNCH_CHECK("attention_decode_bf16 (streaming)");
         return 0;
     }
-#define RI_DECODE_CASE(DH)                                                                                        \
-    case DH:                                                                                                      \
-        attn_decode_mfma_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                           \
+    const int pieces = decode_pieces(seqs, kv_heads, group, max_chunks), all = max_chunks * pieces;
+    const dim3 pgrid(seqs, kv_heads, all);
+#define RI_DECODE_CASE(DH, CW)                                                                                    \
+    case DH * 16 + CW:                                                                                            \
+        attn_decode_mfma_kernel<DH, CW><<<pgrid, CW * 64, 0, s>>>(                                                \
             workspace, (const bf16_t*)qkv, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,             \
-            tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks);                   \
-        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, max_chunks, tiled_out, s);                    \
+            tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all);                          \
+        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, all, tiled_out, s, CW * PAGE);     \
         break;
-    switch (head_dim) {
-        RI_DECODE_CASE(32)
-        RI_DECODE_CASE(64)
-        RI_DECODE_CASE(128)
+    switch (head_dim * 16 + DECODE_WAVES / pieces) {
+        RI_DECODE_CASE(32, 8)
+        RI_DECODE_CASE(32, 4)
+        RI_DECODE_CASE(32, 2)
+        RI_DECODE_CASE(64, 8)
+        RI_DECODE_CASE(64, 4)
+        RI_DECODE_CASE(64, 2)
+        RI_DECODE_CASE(128, 8)
+        RI_DECODE_CASE(128, 4)
+        RI_DECODE_CASE(128, 2)
     }
 #undef RI_DECODE_CASE
     RI_LAUNCH_CHECK("attention_decode_bf16");
@@ -1293,17 +1330,25 @@ extern "C" int ri_attention_decode_fused_bf16(void* out, float* workspace, const
         RI_LAUNCH_CHECK("attention_decode_fused_bf16 (streaming)");
         return 0;
     }
-#define RI_FUSED_CASE(DH)                                                                                         \
-    case DH:                                                                                                      \
-        attn_decode_fused_kernel<DH><<<grid, DECODE_WAVES * 64, 0, s>>>(                                          \
+    const int pieces = decode_pieces(seqs, kv_heads, group, max_chunks), all = max_chunks * pieces;
+    const dim3 pgrid(seqs, kv_heads, all);
+#define RI_FUSED_CASE(DH, CW)                                                                                     \
+    case DH * 16 + CW:                                                                                            \
+        attn_decode_fused_kernel<DH, CW><<<pgrid, CW * 64, 0, s>>>(                                               \
             workspace, (const bf16_t*)qkv, q_stride, q_gain, k_gain, eps, inv_freq, (bf16_t*)k_pages,             \
-            (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, max_chunks); \
-        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, max_chunks, tiled_out, s);                    \
+            (bf16_t*)v_pages, tok_pos, page_table, table_width, heads, kv_heads, window, scale_log2, all);        \
+        launch_join<DH>((bf16_t*)out, workspace, tok_pos, seqs, heads, window, all, tiled_out, s, CW * PAGE);     \
         break;
-    switch (head_dim) {
-        RI_FUSED_CASE(32)
-        RI_FUSED_CASE(64)
-        RI_FUSED_CASE(128)
+    switch (head_dim * 16 + DECODE_WAVES / pieces) {
+        RI_FUSED_CASE(32, 8)
+        RI_FUSED_CASE(32, 4)
+        RI_FUSED_CASE(32, 2)
+        RI_FUSED_CASE(64, 8)
+        RI_FUSED_CASE(64, 4)
+        RI_FUSED_CASE(64, 2)
+        RI_FUSED_CASE(128, 8)
+        RI_FUSED_CASE(128, 4)
+        RI_FUSED_CASE(128, 2)
     }
 #undef RI_FUSED_CASE
     RI_LAUNCH_CHECK("attention_decode_fused_bf16");

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "ri_sum_parts": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
     "ri_attention_decode_streams": [c_int, c_int, c_int],
+    "ri_attention_decode_pieces": [c_int, c_int, c_int, c_int],
     "ri_gemv_bf16_partials": [c_int, c_int],
     "ri_gemm_skinny_packed_bf16_partials": [c_int],
     "ri_gemv_bf16_linked": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_float,
@@ -330,7 +331,8 @@ def attention_decode_bf16(qkv, k_pages, v_pages, cu_seqlens, tok_pos, page_table
     chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
     out = (TiledRows.empty(tokens, heads * head_dim, qkv.device) if tiled_out else
            torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device))
-    ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
+    pieces = _get("ri_attention_decode_pieces")(int(seqs), int(kv_heads), int(heads), chunks)
+    ws = torch.empty((seqs, heads, chunks * pieces, head_dim + 2), dtype=torch.float32, device=qkv.device)
     _call("ri_attention_decode_bf16", _dev(out.data if tiled_out else out, "out"), _dev(ws, "workspace"), _dev(qkv, "qkv", torch.bfloat16), stride,
           _dev(k_pages, "k_pages", torch.bfloat16), _dev(v_pages, "v_pages", torch.bfloat16),
           _dev(cu_seqlens, "cu_seqlens", torch.int32, (seqs + 1,)), _dev(tok_pos, "tok_pos", torch.int32, (tokens,)),
@@ -355,7 +357,8 @@ def attention_decode_fused_bf16(qkv, q_gain, k_gain, eps, inv_freq, k_pages, v_p
     chunks = _get("ri_attention_decode_chunks")(int(max_len))      # the kernels' own chunk size
     out = (TiledRows.empty(tokens, heads * head_dim, qkv.device) if tiled_out else
            torch.empty((tokens, heads * head_dim), dtype=torch.bfloat16, device=qkv.device))
-    ws = torch.empty((seqs, heads, chunks, head_dim + 2), dtype=torch.float32, device=qkv.device)
+    pieces = _get("ri_attention_decode_pieces")(int(seqs), int(kv_heads), int(heads), chunks)
+    ws = torch.empty((seqs, heads, chunks * pieces, head_dim + 2), dtype=torch.float32, device=qkv.device)
     half = head_dim // 2
     _call("ri_attention_decode_fused_bf16", _dev(out.data if tiled_out else out, "out"), _dev(ws, "workspace"),
           _dev(qkv, "qkv", torch.bfloat16), stride, _opt(q_gain, "q_gain", torch.float32, (head_dim,)),
