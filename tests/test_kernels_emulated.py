@@ -57,11 +57,13 @@ ONE_UNIT = ("one_run or mfma_prefill_attention or (mfma_attention_window_edges a
             "and not (1000 and not (1000-1024-33 or 1000-1024-64)))")
 PYTEST = ["-m", "pytest", "-q", "-x", "-p", "no:cacheprovider"]
 KERNEL_TESTS, SMALL_MACHINE = os.path.join(HERE, "test_kernels_gpu.py"), os.path.join(HERE, "small_machine_kernels.py")
+SAMPLER_TESTS = os.path.join(HERE, "test_sampling_gpu.py")
+SAMPLER_SELECT = "(same_token_as_the_plain_sampler or top_p_drops) and not large"     # not the 151,936 entries, not the engine
 
 
 @pytest.fixture(scope="module")
 def runs():
-    """The three emulated runs, side by side (each is a pytest of its own; together they take what the longest takes)."""
+    """The four emulated runs, side by side (each is a pytest of its own; together they take what the longest takes)."""
     from rust_inference_amd.errors import KernelError
     try:
         sys.path.insert(0, HERE)
@@ -73,6 +75,7 @@ def runs():
         "kernel tests": _start([*PYTEST, *_workers(4), KERNEL_TESTS, "-k", SELECT]),
         "sixteen units": _start([*PYTEST, SMALL_MACHINE], {"RI_EMU_COMPUTE_UNITS": "16"}),
         "one unit": _start([*PYTEST, *_workers(2), SMALL_MACHINE, KERNEL_TESTS, "-k", ONE_UNIT], {"RI_EMU_COMPUTE_UNITS": "1"}),
+        "sampler": _start([*PYTEST, *_workers(2), SAMPLER_TESTS, "-k", SAMPLER_SELECT]),
     }
     done = {}
     try:
@@ -96,6 +99,10 @@ def _passed(run, tests=None):
 
 def test_the_kernel_tests_pass_on_the_cpu_build_between_guard_pages(runs):
     _passed(runs["kernel tests"])
+
+
+def test_the_sampler_tests_pass_on_the_cpu_build_between_guard_pages(runs):
+    _passed(runs["sampler"], 33)
 
 
 @pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 31)])

@@ -1,18 +1,45 @@
-"""The device sampler against the plain sampler: the same logits and the same uniform draw give the same token."""
+"""The device sampler against the plain sampler: the same logits and the same uniform draw give the same token.
+
+The kernel tests of this file also run without a GPU, on the CPU build of the kernels between guard pages, when
+the environment says RI_TEST_KERNELS=emulated (tests/test_kernels_emulated.py starts that run)."""
+import os
+
 import numpy as np
 import pytest
 import torch
 
 from plain.sampler_plain import PlainRng, argmax, candidates, draw, penalise
 
-pytestmark = pytest.mark.gpu
-DEV = "cuda:0"
+EMULATED = os.environ.get("RI_TEST_KERNELS") == "emulated"
+pytestmark = [] if EMULATED else pytest.mark.gpu
+DEV = "cpu" if EMULATED else "cuda:0"
 
 
 @pytest.fixture(scope="module")
 def ops():
+    if EMULATED:
+        import emulated
+        return emulated.ops()
     from rust_inference_amd.kernels import ops
     return ops
+
+
+@pytest.fixture(autouse=True)
+def _guarded_buffers_go_back():
+    yield
+    if EMULATED:
+        import gc
+        import emulated
+        gc.collect()
+        emulated.free_all()
+
+
+def g(x):
+    """On the GPU the tensor itself; emulated, a copy between guard pages."""
+    if EMULATED:
+        import emulated
+        return emulated.tensor(x.contiguous(), "a test's operand")
+    return x
 
 
 def plain_pick(logits, r, temperature, top_k, top_p, penalty, history):
@@ -40,11 +67,11 @@ def test_same_token_as_the_plain_sampler(ops, temperature, top_k, top_p, penalty
     gen = PlainRng(5)
     rs = [gen.next_f32() for _ in range(rows)]
     rs[0], rs[1] = 0.0, float(np.float32(1.0) - np.float32(2.0 ** -24))   # the ends of [0, 1)
-    seen = torch.zeros((rows, vocab), dtype=torch.uint8, device=DEV)
+    seen = g(torch.zeros((rows, vocab), dtype=torch.uint8, device=DEV))
     hr = [r for r in range(rows) for _ in history[r]]
     ht = [t for r in range(rows) for t in history[r]]
-    ops.mark_seen(seen, torch.tensor(hr, dtype=torch.int32, device=DEV), torch.tensor(ht, dtype=torch.int32, device=DEV))
-    got = ops.sample(torch.tensor(logits, device=DEV), torch.tensor(rs, dtype=torch.float32, device=DEV), temperature,
+    ops.mark_seen(seen, g(torch.tensor(hr, dtype=torch.int32, device=DEV)), g(torch.tensor(ht, dtype=torch.int32, device=DEV)))
+    got = ops.sample(g(torch.tensor(logits, device=DEV)), g(torch.tensor(rs, dtype=torch.float32, device=DEV)), temperature,
                      top_k, top_p, penalty, seen if penalty != 1.0 else None, split=split).tolist()
     want = [plain_pick(logits[r], rs[r], temperature, top_k, top_p, penalty, history[r]) for r in range(rows)]
     # the device sums masses exactly, the plain sampler in float32 in drawing order: a draw that falls within
@@ -63,7 +90,7 @@ def test_large_vocabulary_and_distribution(ops):
     logits = torch.full((1, vocab), -30.0, device=DEV)
     logits[0, 1000], logits[0, 150000] = 0.0, float(np.log(3.0))
     gen = PlainRng(7)
-    rs = torch.tensor([gen.next_f32() for _ in range(4000)], dtype=torch.float32, device=DEV)
+    rs = g(torch.tensor([gen.next_f32() for _ in range(4000)], dtype=torch.float32, device=DEV))
     picks = ops.sample(logits.expand(4000, vocab).contiguous(), rs, 1.0).tolist()
     assert set(picks) <= {1000, 150000}
     assert abs(np.mean([p == 150000 for p in picks]) - 0.75) < 0.03
@@ -83,12 +110,12 @@ def test_both_forms_pick_the_same_tokens_of_a_large_vocabulary(ops):
     logits[2, :] = 1.5                                           # more ties than are listed
     logits[3, 70000] = 30.0                                      # one token owns the row
     history = [[int(t) for t in rng.integers(0, vocab, 50)] for _ in range(rows)]
-    seen = torch.zeros((rows, vocab), dtype=torch.uint8, device=DEV)
-    ops.mark_seen(seen, torch.tensor([r for r in range(rows) for _ in history[r]], dtype=torch.int32, device=DEV),
-                  torch.tensor([t for r in range(rows) for t in history[r]], dtype=torch.int32, device=DEV))
+    seen = g(torch.zeros((rows, vocab), dtype=torch.uint8, device=DEV))
+    ops.mark_seen(seen, g(torch.tensor([r for r in range(rows) for _ in history[r]], dtype=torch.int32, device=DEV)),
+                  g(torch.tensor([t for r in range(rows) for t in history[r]], dtype=torch.int32, device=DEV)))
     gen = PlainRng(3)
     rs = [gen.next_f32() for _ in range(rows)]
-    dl, dr = torch.tensor(logits, device=DEV), torch.tensor(rs, dtype=torch.float32, device=DEV)
+    dl, dr = g(torch.tensor(logits, device=DEV)), g(torch.tensor(rs, dtype=torch.float32, device=DEV))
     # (47 kept of a row of equal logits: 0.9 of them is no whole number, so float32 sums cannot sit on the edge)
     for temperature, top_k, top_p, penalty in ((0.8, 0, 1.0, 1.0), (1.0, 47, 0.9, 1.2), (1.5, 0, 0.95, 1.0),
                                                (0.7, 3000, 1.0, 1.1)):
@@ -104,15 +131,15 @@ def test_both_forms_pick_the_same_tokens_of_a_large_vocabulary(ops):
 
 
 def test_top_p_drops_the_tail_and_top_k_one_is_greedy(ops):
-    row = torch.tensor([[3.0, 1.0, 0.5, 0.0]], device=DEV).expand(50, 4).contiguous()
-    rs = torch.linspace(0, 0.999, 50, device=DEV)
+    row = g(torch.tensor([[3.0, 1.0, 0.5, 0.0]], device=DEV).expand(50, 4).contiguous())
+    rs = g(torch.linspace(0, 0.999, 50, device=DEV))
     assert set(ops.sample(row, rs, 1.0, top_p=0.5).tolist()) == {0}              # src/sampling.rs:179-187
-    row = torch.tensor([[0.5, 0.4, 0.6, 0.1]], device=DEV).expand(50, 4).contiguous()
+    row = g(torch.tensor([[0.5, 0.4, 0.6, 0.1]], device=DEV).expand(50, 4).contiguous())
     assert set(ops.sample(row, rs, 1.0, top_k=1).tolist()) == {2}                # src/sampling.rs:157-164
-    assert ops.sample(torch.tensor([[0.1, 3.0, 2.0]], device=DEV), None, 0.0).tolist() == [1]
-    seen = torch.zeros((1, 3), dtype=torch.uint8, device=DEV)
+    assert ops.sample(g(torch.tensor([[0.1, 3.0, 2.0]], device=DEV)), None, 0.0).tolist() == [1]
+    seen = g(torch.zeros((1, 3), dtype=torch.uint8, device=DEV))
     seen[0, 1] = 1
-    assert ops.sample(torch.tensor([[0.1, 3.0, 2.0]], device=DEV), None, 0.0, penalty=2.0, seen=seen).tolist() == [2]
+    assert ops.sample(g(torch.tensor([[0.1, 3.0, 2.0]], device=DEV)), None, 0.0, penalty=2.0, seen=seen).tolist() == [2]
 
 
 def test_generation_with_penalty_and_temperature_is_seeded(model_dirs):
