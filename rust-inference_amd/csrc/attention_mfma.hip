@@ -944,13 +944,8 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 #define STREAM_MIN_CHUNKS 8
 #define STREAM_JOINED_FROM 64
 // Eight wavefronts a workgroup and one run a sequence: where the step has one workgroup for every compute unit and
-// few more (up to an eighth), for sequences of up to STREAM_WIDE_MAX_CHUNKS chunks.  Measured against the chunks
-// and their join, at 8 kv heads: with 256 (sequence, kv head) pairs a small model's step is 4% shorter (32
-// sequences of 16 to 1,300 keys) and one at Qwen3-8B sizes 2.4 to 4.4% (32 of 1,900, 2,100 and 3,600); with 384
-// pairs, a second round on half the compute units, level at 900 keys and 2.4% longer at 2,100; with 320 pairs of
-// 6,000 keys 3.5% longer; with 128 pairs, half the compute units, 6 to 9% longer (the units that walk pull no
-// faster for the others being idle), and in two runs a sequence with a join, a workgroup for every unit again,
-// still 1 to 5% longer than the chunks.
+// few more (up to an eighth: a second round on some units, or half the units idle, loses more than the join costs),
+// for sequences of up to STREAM_WIDE_MAX_CHUNKS chunks.
 #ifndef STREAM_WIDE_MAX_CHUNKS
 #define STREAM_WIDE_MAX_CHUNKS 16
 #endif
@@ -1193,12 +1188,8 @@ extern "C" int ri_attention_decode_chunks(int max_len) { return (max_len + DECOD
 
 // Pieces that the chunk kernels cut every chunk into: 1, or 2 or 4 (workgroups of four or two wavefronts, one page
 // each) while the step's workgroups, counted by the bound on the lengths, stay within one for every compute unit and
-// the pieces of a sequence within what the join fetches at once.  A compute unit pulls its pages at a rate of its
-// own, so a step of few short sequences has a fraction of the machine fetch what all of it could: a small model's
-// step at batch 1, 2 and 4 is 1.6, 3.8 and 4.2% shorter for the cut (Qwen3-0.6B sizes; 600, 1,600 and 800 keys), one
-// sequence of 900 and of 1,500 keys at Qwen3-8B sizes 1.7 and 2.4%.  Past what the join fetches at once the cut loses
-// what it gains (one sequence of 2,100 keys at Qwen3-8B sizes in 18 pieces: 0.7% longer; in 36: 1.8%).  A workgroup norms two query
-// heads a wavefront at most, so a kv head's query heads bound the cut too.
+// the pieces of a sequence within what the join fetches at once (past that the cut loses what it gains).  A
+// workgroup norms two query heads a wavefront at most, so a kv head's query heads bound the cut too.
 #ifndef DECODE_SPLIT_FILL
 #define DECODE_SPLIT_FILL 1
 #endif
