@@ -12,6 +12,14 @@ for p in (ROOT, os.path.dirname(os.path.abspath(__file__))):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # A test that hangs (a kernel whose waves never finish) should end the run and name itself rather than hold
+    # the machine: where the timeout plugin is installed and the command line sets no limit, twenty minutes a test
+    # (the longest, the kernels built for the CPU at a first call, takes five), ended from a watching thread (a
+    # signal cannot interrupt a test that is stuck inside a GPU call).
+    if config.pluginmanager.hasplugin("timeout") and not getattr(config.option, "timeout", None):
+        config.option.timeout = 1200
+        if not getattr(config.option, "timeout_method", None):
+            config.option.timeout_method = "thread"
 
 
 # Two tiny configurations of the architecture that differ in every size and option.
