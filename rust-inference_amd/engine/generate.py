@@ -11,8 +11,8 @@ token comes from the prompt's logits and counts toward ``max_new_tokens``; a sto
 token is tested before it is put out, is not part of the output and is never fed
 back; the last token allowed is put out but not fed.
 
-Where the engine can take a step's tokens from the device (``decode_on_device``: captured graphs) and no
-repetition penalty needs them on the host first, the loop runs one step ahead of what it has read: it
+Where the engine can take a step's tokens from the device (``decode_on_device``: captured graphs; a repetition
+penalty's history is then marked on the device from those ids too), the loop runs one step ahead of what it has read: it
 launches step n + 1 with the ids step n picked, still on the device, and reads step n's ids while step n + 1
 runs, so that the host's share of a step (the rules below, the step's layout, the launch) hides behind the
 GPU's.  A sequence whose token then turns out to be a stop token has been carried through one step too many:
@@ -168,7 +168,9 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
             held.discard(s.slot)
             return False
 
-        ahead = not penalised and hasattr(engine, "decode_on_device")
+        # (with a repetition penalty the loop runs ahead only where the history is kept on the device, which is then
+        # marked from the ids in flight; the host sampler reads a history that the host must have written first)
+        ahead = (not penalised or history is not None) and hasattr(engine, "decode_on_device")
         pinned = [None, None]
         flight = None                                           # the step whose picks the host has not read yet
         while True:
@@ -210,7 +212,9 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
                 continue
             carried = [members[i] for i in going]
             with profiler.section(profiler.SAMPLING):
-                picks = pick_batch(logits, [s.sampler for s in carried], None)
+                if history is not None:                         # the tokens this step was fed count as seen from now on
+                    history.mark_on_device([s.sampler.seen_row for s in carried], ids)
+                picks = pick_batch(logits, [s.sampler for s in carried], history)
             for s in members:
                 if s.reason is None:
                     settle(s)

@@ -33,6 +33,11 @@ class DeviceHistory:
             toks.extend(s.history)
         self.mark(rows, toks)
 
+    def mark_on_device(self, rows, tokens: torch.Tensor) -> None:
+        """The same with the tokens still on the device (int32), so that nobody has to have read them."""
+        if rows:
+            ops.mark_seen(self.seen, torch.tensor(rows, dtype=torch.int32, device=self.seen.device), tokens)
+
     def mark(self, rows, tokens) -> None:
         if rows:
             dev = self.seen.device

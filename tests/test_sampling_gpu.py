@@ -153,6 +153,31 @@ def test_generation_with_penalty_and_temperature_is_seeded(model_dirs):
     assert a == b and alone[0] == a[0] and a != model.generate(prompts, seed=4, **kw).tokens
 
 
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_a_repetition_penalty_gives_the_same_tokens_with_the_loop_running_ahead(model_dirs, dtype_name):
+    """With graphs the loop launches a step before it has read the ids of the one before, and marks the penalty's
+    history on the device from the ids in flight; without, the host marks it from the ids it has read.  The same
+    tokens either way (the steps are the same kernels on the same rows as long as nobody stops), with stop tokens
+    too in float32 (a sequence that stops is carried one step further by the one loop; nobody else's logits
+    change for that in 32-bit)."""
+    from rust_inference_amd import Model
+    prompts = [[1, 2, 3, 4, 2, 2], [9, 8], [5], [7, 7, 7, 7]]
+    kw = dict(max_new_tokens=24, temperature=0.9, top_k=30, repetition_penalty=1.4, seed=11)
+    outs = {}
+    for graphs in (True, False):
+        model = Model.load(model_dirs["A"], dtype=dtype_name, max_batch=4, max_seq_len=64, use_graphs=graphs)
+        outs[graphs] = [model.generate(prompts, ignore_eos=True, **kw)]
+        if dtype_name == "float32":
+            outs[graphs].append(model.generate(prompts, stop_token_ids=[int(t) for t in outs[graphs][0].tokens[1][3:9]], **kw))
+        model.cache.check_consistent()
+    for a, b in zip(outs[True], outs[False]):
+        assert a.tokens == b.tokens and a.finish_reasons == b.finish_reasons
+    if dtype_name == "float32":
+        assert "stop" in outs[True][1].finish_reasons
+    plain = Model.load(model_dirs["A"], dtype=dtype_name, max_batch=4, max_seq_len=64, use_graphs=True)
+    assert plain.generate(prompts, ignore_eos=True, **dict(kw, repetition_penalty=1.0)).tokens != outs[True][0].tokens
+
+
 def test_sequences_of_one_batch_sample_each_in_their_own_way(model_dirs):
     """Per-request sampling parameters through the entry point: greedy, temperature, top-k with a penalty side
     by side in one batch give each request the tokens it gets when the whole batch samples its way (float32:
