@@ -29,6 +29,7 @@ from ..errors import CacheError, ShapeError
 import torch
 
 from ..sampling import DeviceHistory, SamplingParams, SequenceSampler, pick_batch, sample_batch
+from ..sampling.batch import upload
 from .step import StepEntry
 
 
@@ -202,7 +203,7 @@ def run_batch(engine, requests: Sequence[int], prompts, max_new_tokens: int, sam
             going = [i for i, s in enumerate(members) if s.reason is None and s.generated < max_new_tokens]
             logits = None
             if going:
-                ids = flight.ids if len(going) == len(members) else flight.ids[torch.tensor(going, device=flight.ids.device)]
+                ids = flight.ids if len(going) == len(members) else flight.ids[upload(going, torch.int64, flight.ids.device)]
                 logits = engine.decode_on_device([members[i].slot for i in going], ids)
             for s, tok in zip(members, flight.read()):
                 if s.reason is None:

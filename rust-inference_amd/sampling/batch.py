@@ -10,6 +10,17 @@ from .host import HostSampler
 from .params import SamplingParams
 
 
+def upload(values, dtype, device) -> torch.Tensor:
+    """A short list of numbers as a tensor on ``device`` without the host waiting for the GPU: through pinned
+    memory, the copy in stream order (a copy from ordinary memory makes the host wait until everything launched
+    before it is done, which is the step that the loop has just launched ahead)."""
+    t = torch.tensor(values, dtype=dtype)
+    device = torch.device(device)
+    if device.type != "cuda":
+        return t.to(device)
+    return t.pin_memory().to(device, non_blocking=True)
+
+
 class SequenceSampler:
     """The sampling state of one sequence.  Sequence ``index`` of a call draws from the generator
     seeded ``seed + index``; sequence 0 has the reference's stream."""
@@ -36,13 +47,12 @@ class DeviceHistory:
     def mark_on_device(self, rows, tokens: torch.Tensor) -> None:
         """The same with the tokens still on the device (int32), so that nobody has to have read them."""
         if rows:
-            ops.mark_seen(self.seen, torch.tensor(rows, dtype=torch.int32, device=self.seen.device), tokens)
+            ops.mark_seen(self.seen, upload(rows, torch.int32, self.seen.device), tokens)
 
     def mark(self, rows, tokens) -> None:
         if rows:
             dev = self.seen.device
-            ops.mark_seen(self.seen, torch.tensor(rows, dtype=torch.int32, device=dev),
-                          torch.tensor(tokens, dtype=torch.int32, device=dev))
+            ops.mark_seen(self.seen, upload(rows, torch.int32, dev), upload(tokens, torch.int32, dev))
 
 
 def _pick_alike(logits: torch.Tensor, samplers: list[SequenceSampler], history: DeviceHistory | None) -> torch.Tensor:
@@ -53,13 +63,13 @@ def _pick_alike(logits: torch.Tensor, samplers: list[SequenceSampler], history: 
     dev = logits.device
     uniform = None
     if not p.greedy:
-        uniform = torch.tensor([s.host.rng.next_f32() for s in samplers], dtype=torch.float32, device=dev)
+        uniform = upload([s.host.rng.next_f32() for s in samplers], torch.float32, dev)
     seen = seen_rows = None
     if p.repetition_penalty != 1.0:
         if history is None:
             raise ValueError("a repetition penalty needs the device history of the batch")
         seen = history.seen
-        seen_rows = torch.tensor([s.seen_row for s in samplers], dtype=torch.int32, device=dev)
+        seen_rows = upload([s.seen_row for s in samplers], torch.int32, dev)
     return ops.sample(logits, uniform, p.temperature, p.top_k, p.top_p, p.repetition_penalty, seen, seen_rows)
 
 
@@ -85,7 +95,7 @@ def pick_batch(logits: torch.Tensor, samplers: list[SequenceSampler], history: D
         return _pick_alike(logits, samplers, history)
     out = torch.empty(len(samplers), dtype=torch.int32, device=logits.device)
     for members in groups.values():
-        at = torch.tensor(members, dtype=torch.int64, device=logits.device)
+        at = upload(members, torch.int64, logits.device)
         out.index_copy_(0, at, _pick_alike(logits.index_select(0, at), [samplers[i] for i in members], history))
     return out
 
