@@ -184,6 +184,45 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
             acc[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc[c & 1], 0, 0, 0);
             if (SWIGLU) accu[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu[c & 1], 0, 0, 0);
         }
+    } else if (K % 32 == 0) {
+        // A share that is no whole number of rounds (K = 2,560 or 9,728 over four wavefronts): the same ring.  A
+        // load for a step past the share's end is issued all the same, from the share's last step (no load in a
+        // branch), and in the last round, the only one that holds such steps, zeros go to the matrix cores in
+        // their place (chosen where the fragment is used: choosing where it is loaded would wait for every load
+        // in turn).  The same sums in the same order as the loop below.
+        Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];
+        const int last = max(min(kt_end, k_tiles) - 1, 0);
+#pragma unroll
+        for (int c = 0; c < SK_CHUNK; ++c) {
+            const size_t from = (size_t)min(kt_begin + c, last);
+            wf[c].u = load_stream16(wp + from * 512);
+            if (SWIGLU) uf[c].u = load_stream16(up + from * 512);
+            xf[c].u = *reinterpret_cast<const uint4*>(xp + from * x_step);
+        }
+        int kt = kt_begin;
+        for (; kt + SK_CHUNK < kt_end; kt += SK_CHUNK) {      // every step of these rounds lies inside the share
+#pragma unroll
+            for (int c = 0; c < SK_CHUNK; ++c) {
+                acc[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c].v, xf[c].v, acc[c & 1], 0, 0, 0);
+                if (SWIGLU) accu[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[c].v, xf[c].v, accu[c & 1], 0, 0, 0);
+                const size_t from = (size_t)min(kt + c + SK_CHUNK, last);
+                wf[c].u = load_stream16(wp + from * 512);
+                if (SWIGLU) uf[c].u = load_stream16(up + from * 512);
+                xf[c].u = *reinterpret_cast<const uint4*>(xp + from * x_step);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < SK_CHUNK; ++c) {
+            const bool live = kt + c < kt_end;
+            Frag w, u, xv;
+            w.u = live ? wf[c].u : zero;
+            xv.u = live ? xf[c].u : zero;
+            acc[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.v, xv.v, acc[c & 1], 0, 0, 0);
+            if (SWIGLU) {
+                u.u = live ? uf[c].u : zero;
+                accu[c & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u.v, xv.v, accu[c & 1], 0, 0, 0);
+            }
+        }
     } else
     for (int kt = kt_begin; kt < kt_end; kt += SK_CHUNK) {
         Frag wf[SK_CHUNK], uf[SK_CHUNK], xf[SK_CHUNK];

@@ -637,7 +637,8 @@ def test_gemv_bf16(ops, m, out_dtype):
 
 
 @pytest.mark.parametrize("m", [1, 3, 8, 16])
-@pytest.mark.parametrize("n, k", [(37, 584), (100, 96), (4096, 4096), (50, 12288), (320, 104)])
+@pytest.mark.parametrize("n, k", [(37, 584), (100, 96), (4096, 4096), (50, 12288), (320, 104),
+                                  (96, 2560), (48, 9728)])       # K whose share of a wavefront is no whole round of 8 steps
 def test_gemm_skinny_packed_bf16(ops, m, n, k):
     rng = np.random.default_rng(m + n)
     x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
