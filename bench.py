@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the Qwen3-8B-shaped model on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|32b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--model 8b|0.6b|1.7b|4b|14b|32b]
 
 The default run has the layer sizes of Qwen3-8B with random weights
 (N(0, 0.02), norm gains 1 + N(0, 0.1), seed 2), a batch of 8 and prompts of 2,048 tokens in a
@@ -39,8 +39,16 @@ QWEN3_0_6B = dict(QWEN3_8B, hidden_size=1024, intermediate_size=3072, num_hidden
                   num_key_value_heads=8, tie_word_embeddings=True)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
                  num_key_value_heads=8)
+# (and the three published sizes between them, for `--model`: not part of the default run)
+QWEN3_1_7B = dict(QWEN3_8B, hidden_size=2048, intermediate_size=6144, num_hidden_layers=28, num_attention_heads=16,
+                  num_key_value_heads=8, tie_word_embeddings=True)
+QWEN3_4B = dict(QWEN3_8B, hidden_size=2560, intermediate_size=9728, num_hidden_layers=36, num_attention_heads=32,
+                num_key_value_heads=8, tie_word_embeddings=True)
+QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40,
+                 num_key_value_heads=8)
 MODELS = {"8b": ("Qwen3-8B shapes", QWEN3_8B, 2), "0.6b": ("Qwen3-0.6B shapes", QWEN3_0_6B, 3),
-          "32b": ("Qwen3-32B shapes", QWEN3_32B, 4)}           # name, sizes, seed of the random weights
+          "32b": ("Qwen3-32B shapes", QWEN3_32B, 4), "1.7b": ("Qwen3-1.7B shapes", QWEN3_1_7B, 5),
+          "4b": ("Qwen3-4B shapes", QWEN3_4B, 6), "14b": ("Qwen3-14B shapes", QWEN3_14B, 7)}   # name, sizes, seed of the random weights
 
 
 def layer_matrix_params(c):

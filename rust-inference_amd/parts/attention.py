@@ -81,7 +81,7 @@ class GroupedQueryAttention(Mixer):
         p = self.prefix
         qkv = torch.cat([weights[p + "q_proj.weight"], weights[p + "k_proj.weight"], weights[p + "v_proj.weight"]], 0)
         self.w_qkv = rt.pack(rt.place_matrix(qkv))
-        self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]))
+        self.w_o = rt.pack(rt.place_matrix(weights[p + "o_proj.weight"]), parts_ok=(p + "o_proj.bias") not in weights)
         self.q_gain = rt.place_gain(weights[p + "q_norm.weight"]) if self.qk_norm else None
         self.k_gain = rt.place_gain(weights[p + "k_norm.weight"]) if self.qk_norm else None
         self.b_qkv = self.b_o = None

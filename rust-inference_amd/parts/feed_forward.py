@@ -33,7 +33,7 @@ class SwiGLU(FeedForward):
         p = self.prefix
         gate_up = rt.place_matrix(torch.cat([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], 0))
         self.w_gate_up = rt.pack(gate_up, swiglu=True)
-        self.w_down = rt.pack(rt.place_matrix(weights[p + "down_proj.weight"]))
+        self.w_down = rt.pack(rt.place_matrix(weights[p + "down_proj.weight"]), parts_ok=True)
 
     def bind_plain(self, weights):
         p = self.prefix

@@ -66,6 +66,9 @@ class PackedWeight:
         # a long K is cut into pieces of 4096 whose float32 sums the next norm adds up: more workgroups
         # stream the weights (768 instead of 256 for 4096 x 12288), and the sum is never rounded to 16 bits
         self.parts = self.k // SPLIT_K if (not swiglu and self.k >= PACKED_LONG_K) else 1
+        # 2 to 16 rows into the residual stream go to the wide kernel (set by Runtime.pack: see there)
+        self.small_wide = False
+        self.small_only = False      # the packed copy was made for that alone: larger steps stay where they were
 
 
 class Runtime:
@@ -131,16 +134,25 @@ class Runtime:
             return ops.as_rows(x)
         return ops.finish_norm(x)
 
-    def pack(self, w: torch.Tensor, swiglu: bool = False, always: bool = False) -> PackedWeight:
+    def pack(self, w: torch.Tensor, swiglu: bool = False, always: bool = False, parts_ok: bool = False) -> PackedWeight:
         """A placed weight, with a packed copy where the packed kernel is the faster one for 2 to 16
-        rows (bfloat16 compute only), or wherever it can be used when the caller says ``always``."""
+        rows (bfloat16 compute only), or wherever it can be used when the caller says ``always``.
+        ``parts_ok``: the product's reader adds stretches of K (the residual stream's next norm).  Then a matrix
+        that the packed kernel serves badly at 2 to 16 rows, one whose row tiles leave most compute units idle in
+        their last round (5,120 rows) or whose long rows it cuts into parts itself (K of 16,384 and more), goes to
+        the wide kernel there, which shares the rows of x through LDS and plans its stretches for the machine
+        (5,120 x 5,120 at 8 rows: 11 us against the library's 19; 5,120 x 25,600: 41 against 51)."""
         n, k = w.shape
         if self.invariant and k % 8:
             raise ShapeError(f"the invariant mode's product takes rows of a multiple of 8 elements, not {k}")
         pays = always or swiglu or self.invariant or _packed_pays(n, k)
-        if self.dtype != torch.bfloat16 or k % 8 or not pays:
+        small_wide = (parts_ok and not swiglu and not self.invariant and k >= WIDE_MIN_K
+                      and (not pays or k >= PACKED_LONG_K))
+        if self.dtype != torch.bfloat16 or k % 8 or not (pays or small_wide):
             return PackedWeight(w, None, swiglu)
-        return PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
+        pw = PackedWeight(w, ops.pack_for_mfma(w, swiglu), swiglu)
+        pw.small_wide, pw.small_only = small_wide, small_wide and not pays
+        return pw
 
     @staticmethod
     def _mid_pays(pw: PackedWeight, m: int, tiled: bool) -> bool:
@@ -167,6 +179,8 @@ class Runtime:
         kernel: whoever makes its rows then makes them as ``ops.TiledRows``."""
         if self.dtype != torch.bfloat16 or pw.packed is None or pw.k % 8 or self.invariant:
             return False
+        if pw.small_only:                                        # a packed copy made for small steps into the stream alone:
+            return parts_ok and 2 < m <= MID_TILED_ROWS          # the wide kernel takes those, nothing else of it
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
         if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu
@@ -196,9 +210,24 @@ class Runtime:
         if self.dtype == torch.bfloat16 and pw.k % 8 == 0:
             later = isinstance(x, ops.NormedLater)
             mine = None
-            if m <= GEMV_MAX_ROWS or (m <= 2 and pw.packed is None):
+            if (max(GEMV_MAX_ROWS, 2 if pw.small_only else 0) < m <= SKINNY_MAX_ROWS and pw.small_wide and parts_ok):
+                # (the parts beat a link to the next norm, as they do for the packed kernel's own; two rows of a
+                # matrix that had no packed copy stay with the kernel of one wavefront a row, which takes the link)
+                x = self.normed_now(x) if later else x
+                waves, parts = _wide_plan(pw.n, pw.k, False)
+                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
+            if (SKINNY_MAX_ROWS // 2 < m <= SKINNY_MAX_ROWS and pw.swiglu and pw.packed is not None and not later
+                    and pw.k >= WIDE_MIN_K):
+                # 9 to 16 rows of a gate|up pair whose input is plain rows (the norm before it was a kernel of its
+                # own): the packed kernel loads every row of x once per 16 rows of weights there (its form that
+                # serves two steps with one load takes 8 rows), the wide one shares them through LDS (16 rows at
+                # Qwen3-8B, 14B and 32B sizes: 33, 64 and 86 us against 35, 67 and 95)
+                waves, _ = _wide_plan(pw.n, pw.k, True)
+                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=True, depth=1, waves=waves,
+                                                 tiled_out=tiled_out and out_dtype == torch.bfloat16)
+            if m <= GEMV_MAX_ROWS or (m <= 2 and (pw.packed is None or pw.small_only)):
                 mine = (pw.w, False)
-            elif m <= SKINNY_MAX_ROWS and pw.packed is not None:
+            elif m <= SKINNY_MAX_ROWS and pw.packed is not None and not pw.small_only:
                 mine = (pw.packed, True)
             if mine is not None:
                 in_parts = mine[1] and parts_ok and pw.parts > 1        # very long rows: parts beat the link
@@ -217,7 +246,7 @@ class Runtime:
                     return ops.gemv_bf16(ops.as_rows(x), pw.w, out_dtype, swiglu=pw.swiglu)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
             if (WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
-                    and pw.k >= WIDE_MIN_K):
+                    and pw.k >= WIDE_MIN_K and not (pw.small_only and m > MID_TILED_ROWS)):
                 # 17 to 64 rows into the residual stream: K in stretches, every stretch a workgroup that shares the tiles of x
                 # through LDS; the stream's next norm adds the stretches' sums
                 x = self.normed_now(x) if later else x
