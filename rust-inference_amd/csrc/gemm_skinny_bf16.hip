@@ -106,12 +106,66 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
 
     floatx4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, accu[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     if (PAIRED) {
-        // (the host launches this form only where the ring's conditions hold)
+        // (the host launches this form only where the ring's conditions hold, or where every wavefront's share is a
+        // whole number of pairs of steps)
         constexpr int PC = SK_CHUNK / 2;                     // pairs of steps in flight: as many weights as the ring below
         const int sub = i >> 3;                              // which step of a pair this lane's piece of x belongs to
         const bf16_t* xq = x_tiled ? x + (size_t)(jg * 16 + (i & 7)) * 8 + (size_t)sub * 512
                                    : x + (size_t)((i & 7) < M ? (i & 7) : 0) * K + jg * 8 + sub * 32;
         Frag wa[PC], wb[PC], ua[PC], ub[PC], xf[PC];
+        if (!ring) {
+            // A share that is a whole number of pairs but no whole number of rounds (the host sees to the pairs):
+            // loads for pairs past the share's end come from its last pair, and in the last round zeros go to the
+            // matrix cores in their place, as in the ring for such shares below.
+            const int last = max(kt_end - 2, 0);
+#pragma unroll
+            for (int c = 0; c < PC; ++c) {
+                const size_t at = (size_t)min(kt_begin + 2 * c, last);
+                wa[c].u = load_stream16(wp + at * 512);
+                wb[c].u = load_stream16(wp + (at + 1) * 512);
+                if (SWIGLU) {
+                    ua[c].u = load_stream16(up + at * 512);
+                    ub[c].u = load_stream16(up + (at + 1) * 512);
+                }
+                xf[c].u = *reinterpret_cast<const uint4*>(xq + at * x_step);
+            }
+            int kt = kt_begin;
+            for (; kt + SK_CHUNK < kt_end; kt += SK_CHUNK) {
+#pragma unroll
+                for (int c = 0; c < PC; ++c) {
+                    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[c].v, xf[c].v, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[c].v, xf[c].v, acc[1], 0, 0, 0);
+                    if (SWIGLU) {
+                        accu[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ua[c].v, xf[c].v, accu[0], 0, 0, 0);
+                        accu[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ub[c].v, xf[c].v, accu[1], 0, 0, 0);
+                    }
+                    const size_t next = (size_t)min(kt + 2 * c + SK_CHUNK, last);
+                    wa[c].u = load_stream16(wp + next * 512);
+                    wb[c].u = load_stream16(wp + (next + 1) * 512);
+                    if (SWIGLU) {
+                        ua[c].u = load_stream16(up + next * 512);
+                        ub[c].u = load_stream16(up + (next + 1) * 512);
+                    }
+                    xf[c].u = *reinterpret_cast<const uint4*>(xq + next * x_step);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < PC; ++c) {
+                const bool live = kt + 2 * c < kt_end;
+                Frag a, b, xv;
+                a.u = live ? wa[c].u : zero;
+                b.u = live ? wb[c].u : zero;
+                xv.u = live ? xf[c].u : zero;
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, xv.v, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, xv.v, acc[1], 0, 0, 0);
+                if (SWIGLU) {
+                    a.u = live ? ua[c].u : zero;
+                    b.u = live ? ub[c].u : zero;
+                    accu[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, xv.v, accu[0], 0, 0, 0);
+                    accu[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, xv.v, accu[1], 0, 0, 0);
+                }
+            }
+        } else {
 #pragma unroll
         for (int c = 0; c < PC; ++c) {
             const size_t at = (size_t)(kt_begin + 2 * c);
@@ -151,6 +205,7 @@ gemm_skinny_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, co
                 accu[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ua[c].v, xf[c].v, accu[0], 0, 0, 0);
                 accu[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ub[c].v, xf[c].v, accu[1], 0, 0, 0);
             }
+        }
         }
     } else if (ring) {
         // Every wavefront's share is a whole number of rounds of SK_CHUNK steps and K a multiple of 32: the
@@ -327,8 +382,9 @@ static void launch_packed(void* out, int out_dtype, const bf16_t* x, const bf16_
     const int part_tiles = (k_tiles + parts - 1) / parts;
     const int tiles_per_wave = (part_tiles + WAVES - 1) / WAVES;
     dim3 grid(row_tiles, parts);
-    // the ring's conditions (the kernel works them out the same way) and at most 8 rows: two steps to a load of x
-    const bool paired = m <= 8 && k % 32 == 0 && tiles_per_wave % SK_CHUNK == 0 && part_tiles == tiles_per_wave * WAVES &&
+    // at most 8 rows and every wavefront's share a whole number of pairs of steps: two steps to a load of x (the
+    // kernel works out for itself whether the share is whole rounds of the ring too)
+    const bool paired = m <= 8 && k % 32 == 0 && tiles_per_wave % 2 == 0 && part_tiles == tiles_per_wave * WAVES &&
                         k_tiles % part_tiles == 0;
 #define RI_SKINNY_GO(TO, PAIRED)                                                        \
     gemm_skinny_packed_kernel<WAVES, SWIGLU, TO, PAIRED><<<grid, WAVES * 64, 0, s>>>(   \

@@ -622,12 +622,13 @@ def test_gemm_f32_is_true_32_bit(ops):
 
 @pytest.mark.parametrize("m", [1, 2, 3, 5, 8])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-def test_gemv_bf16(ops, m, out_dtype):
+@pytest.mark.parametrize("k", [584, 2560, 1544, 2048, 9728])      # steps of 512: one and a bit, five, three and a bit, four, nineteen
+def test_gemv_bf16(ops, m, out_dtype, k):
     rng = np.random.default_rng(m)
-    x, w = t(rng.normal(size=(m, 584)), torch.bfloat16), t(rng.normal(size=(37, 584)), torch.bfloat16)
+    x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(37, k)), torch.bfloat16)
     want = f64(x) @ f64(w).T
     close(ops.gemv_bf16(x, w, out_dtype), want, 2e-6 if out_dtype == torch.float32 else 5e-3, "gemv")
-    wgu = t(rng.normal(size=(2 * 45, 584)) * 0.1, torch.bfloat16)
+    wgu = t(rng.normal(size=(2 * 45, k)) * 0.1, torch.bfloat16)
     y = f64(x) @ f64(wgu).T
     close(ops.gemv_bf16(x, wgu, out_dtype, swiglu=True), P.silu(y[:, :45]) * y[:, 45:],
           3e-6 if out_dtype == torch.float32 else 5e-3, "gemv with swiglu")
