@@ -99,10 +99,13 @@ class OutputHead(Head):
             self.packed = self.rt.pack(self.weight, always=True)
         return self.packed
 
-    # Rows of logits up to which the packed copy serves: 2 to 16 the packed kernel; 17 to 32 the wide kernel with
-    # four row tiles a workgroup (151,936 x 4,096 at 17 and 32 rows: 222 and 247 us against the library's 279 and
-    # 274; from 48 rows on the library is ahead, 266 against 279 us, with 39 MB of float32 logits to write).
+    # Rows of logits up to which the packed copy serves: 2 to 8 the packed kernel (one load of x serves two steps of
+    # K there); 9 to 32 the wide kernel with four row tiles a workgroup, which shares the rows of x through LDS
+    # (151,936 x 4,096 at 9, 16, 17 and 32 rows: 204, 213, 222 and 247 us against the packed kernel's 224 and 279
+    # and the library's 250 to 279; x 1,024 at 16 rows 57 against 78; x 5,120: 254 against 382; from 48 rows on the
+    # library is ahead, 266 against 279 us, with 39 MB of float32 logits to write).
     PACKED_MAX_ROWS = 32
+    PAIRED_MAX_ROWS = 8
 
     def forward(self, x):
         rows = x.shape[0]
@@ -111,7 +114,7 @@ class OutputHead(Head):
         if 2 <= rows <= self.PACKED_MAX_ROWS and self.dim % 8 == 0:
             packed = self._packed_copy()
             if packed is not None and packed.packed is not None:
-                if rows <= 16:
+                if rows <= self.PAIRED_MAX_ROWS:
                     return self.rt.linear_packed(x, packed, out_dtype=torch.float32)
                 return ops.gemm_wide_packed_bf16(self.rt.normed_now(x), packed.packed, self.vocab, torch.float32,
                                                  depth=1, waves=4)
