@@ -32,7 +32,9 @@ MID_MAX_BYTES = 20_000_000       # up to this size the packed kernel beats the l
 MID_TILED_ROWS = 32              # and up to this many rows on any matrix when the rows come tiled
 WIDE_MIN_K = 4096                # rows shorter than this leave the wide kernel's stretches too little to do
 WIDE_MIN_ROWS = 17
-WIDE_GATED_FILL = 0.9            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds
+WIDE_GATED_FILL = 0.9            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds,
+WIDE_GATED_ROWS = 48             # and up to this many rows whatever they fill, if the packed kernel of 17 to 64 rows is no match:
+WIDE_GATED_BYTES = 64_000_000    # pairs larger than this (smaller ones, up to 32 tiled rows, are that kernel's)
 SPLIT_K = 4096                   # pieces of a long K (PACKED_LONG_K and more) whose sums the next norm adds
 # Which matrices get a packed copy for 2 to 16 rows (the gate|up matrix always does: its activation rides in
 # the kernel): up to 40 MB always; up to PACKED_MAX_BYTES unless the last round of workgroups (one per 16 rows)
@@ -163,12 +165,16 @@ class Runtime:
         return tiled and m <= MID_TILED_ROWS
 
     @staticmethod
-    def _wide_gated(pw: PackedWeight) -> bool:
-        """Whether the wide kernel takes a gate|up pair at 17 to 64 rows: where its workgroups (of three or
-        four wavefronts, K whole) fill the compute units evenly; else a quarter of the machine idles and the
-        library with its activation kernel is as fast."""
+    def _wide_gated(pw: PackedWeight, m: int) -> bool:
+        """Whether the wide kernel takes a gate|up pair at 17 to 64 rows: up to WIDE_GATED_ROWS rows whenever the
+        pair is too large for the packed kernel of those rows (which takes twice as long for twice the rows);
+        beyond, where its workgroups (of three or four wavefronts, K whole) fill the compute units evenly; else a
+        quarter of the machine idles and the library with its activation kernel is as fast."""
         if pw.packed is None:
             return False
+        size = pw.w.shape[0] * pw.k * 2
+        if m <= WIDE_GATED_ROWS and (size > WIDE_GATED_BYTES or (m > MID_TILED_ROWS and size > MID_MAX_BYTES)):
+            return True
         waves, parts = _wide_plan(pw.n, pw.k, True)
         groups = -(-(-(-pw.n // 16)) // waves) * parts
         cus = _compute_units()
@@ -183,7 +189,7 @@ class Runtime:
             return parts_ok and 2 < m <= MID_TILED_ROWS          # the wide kernel takes those, nothing else of it
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
-        if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and (self._wide_gated(pw) if pw.swiglu
+        if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and (self._wide_gated(pw, m) if pw.swiglu
                                                    else parts_ok and pw.k >= WIDE_MIN_K):
             return True                                          # the wide kernel (where the reader adds its parts)
         return SKINNY_MAX_ROWS < m <= MID_MAX_ROWS and self._mid_pays(pw, m, True)
@@ -252,7 +258,7 @@ class Runtime:
                 x = self.normed_now(x) if later else x
                 waves, parts = _wide_plan(pw.n, pw.k, False)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
-            if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw):
+            if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw, m):
                 x = self.normed_now(x) if later else x
                 waves, _ = _wide_plan(pw.n, pw.k, True)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=True, depth=1, waves=waves,
