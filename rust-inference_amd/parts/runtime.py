@@ -29,7 +29,8 @@ GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
 MID_MAX_ROWS = 64
 MID_MAX_BYTES = 20_000_000       # up to this size the packed kernel beats the library at 17 to 64 plain rows
-MID_TILED_ROWS = 32              # and up to this many rows on any matrix when the rows come tiled
+MID_TILED_ROWS = 32              # and up to this many rows when the rows come tiled,
+MID_TILED_BYTES = 64_000_000     # on matrices up to this size (7168 x 5120 draws level with the library, 10240 x 5120 loses: 28 us to 20)
 WIDE_MIN_K = 4096                # rows shorter than this leave the wide kernel's stretches too little to do
 WIDE_MIN_ROWS = 17
 WIDE_GATED_FILL = 0.9            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds,
@@ -160,9 +161,10 @@ class Runtime:
     def _mid_pays(pw: PackedWeight, m: int, tiled: bool) -> bool:
         """Whether the packed kernel for 17 to 64 rows beats the library's product (and, for gate|up, its
         activation kernel) on this matrix."""
-        if pw.w.shape[0] * pw.k * 2 <= MID_MAX_BYTES:
+        size = pw.w.shape[0] * pw.k * 2
+        if size <= MID_MAX_BYTES:
             return True
-        return tiled and m <= MID_TILED_ROWS
+        return tiled and m <= MID_TILED_ROWS and size <= MID_TILED_BYTES
 
     @staticmethod
     def _wide_gated(pw: PackedWeight, m: int) -> bool:
