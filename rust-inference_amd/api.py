@@ -30,10 +30,13 @@ def as_dtype(dtype) -> torch.dtype:
 
 
 class Model:
-    """A loaded model with a cache sized for ``max_batch`` sequences of ``max_seq_len`` tokens."""
+    """A loaded model with a cache sized for ``max_batch`` sequences of ``max_seq_len`` tokens.
+    ``graph_after``: decode steps of one batch size run that many times with host launches before their graph is
+    captured (capturing costs 3 to 5 steps' time, and a batch whose sequences stop at different times passes
+    through many sizes); 0, the default, captures at the first step of a size."""
 
     def __init__(self, decoder, max_batch: int = 8, max_seq_len: int = 4096, max_tokens: int | None = None,
-                 use_graphs: bool = True, plain: bool = False):
+                 use_graphs: bool = True, plain: bool = False, graph_after: int = 0):
         self.decoder = decoder
         self.config = getattr(decoder, "config", None)
         per_seq = -(-max_seq_len // PAGE_SIZE) * PAGE_SIZE
@@ -42,7 +45,7 @@ class Model:
             self.cache = self.engine.cache
         else:
             self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
-            self.engine = Engine(decoder, self.cache, use_graphs=use_graphs)
+            self.engine = Engine(decoder, self.cache, use_graphs=use_graphs, capture_after=graph_after)
 
     @classmethod
     def load(cls, model_dir: str, dtype="bfloat16", device="cuda:0", batch_invariant: bool = False,

@@ -118,10 +118,18 @@ class Engine:
     a decode step cost more than its kernels otherwise.  Page tables then have the cache's full
     width and the attention grid is sized for the bound; the results are the same."""
 
-    def __init__(self, model, cache, use_graphs: bool = False):
+    def __init__(self, model, cache, use_graphs: bool = False, capture_after: int = 0):
         self.model, self.cache = model, cache
         self.device = model.rt.device
         self.use_graphs = use_graphs
+        # Decode steps of a batch size and bound run this many times with host launches before their graph is
+        # captured.  Capturing costs what 3 to 5 replays take (6 ms at Qwen3-0.6B sizes, 10 to 17 at Qwen3-8B
+        # sizes), and a batch whose sequences end at different times passes through every size below its first,
+        # some for a step or two; a replay saves a small model half of a step with host launches (1.3 against 2.4
+        # ms) and a large one a few per cent (3.35 against 3.5), so only a large model's short-lived sizes are
+        # better left without a graph.  0: capture at the first step of a size.
+        self.capture_after = int(capture_after)
+        self._seen: dict[tuple[int, int], int] = {}
         self._staging = None
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}       # in order of last use
         self.max_graphs = MAX_GRAPHS
@@ -216,6 +224,15 @@ class Engine:
         slots = np.fromiter((e.slot for e in entries), dtype=np.int32, count=batch)
         bound = _decode_bound(self.cache, self.cache.longest(slots) + 1)
         dg = self._graphs.pop((batch, bound), None)
+        if dg is None and self.capture_after > 0:
+            if len(self._seen) > 8 * max(1, self.max_graphs):
+                self._seen.clear()
+            seen = self._seen[(batch, bound)] = self._seen.get((batch, bound), 0) + 1
+            if seen <= self.capture_after:                   # not yet worth a graph: the step with host launches
+                ctx = self.build_context(entries)
+                logits = self.model.forward(ctx, self.cache)
+                self.cache.commit(ctx.slot_list, ctx.new_counts)
+                return logits
         if dg is not None:
             self._graphs[(batch, bound)] = dg                # the most recently used sits last
         else:

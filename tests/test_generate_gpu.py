@@ -72,7 +72,7 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name, lengths, st
     from rust_inference_amd import Model
     cfg, _ = read_model_f64(model_dirs[name])
     prompts = prompts_for(cfg, lengths, 3)
-    model = Model.load(model_dirs[name], dtype=dtype_name, max_batch=4, max_seq_len=96, use_graphs=use_graphs)
+    model = Model.load(model_dirs[name], dtype=dtype_name, max_batch=4, max_seq_len=96, use_graphs=use_graphs, graph_after=0)
     res = model.generate(prompts, max_new_tokens=steps)
     assert_same_tokens(res.tokens, plain_greedy_with_margins(model_dirs[name], prompts, steps), dtype_name,
                        model_dirs[name], prompts)
@@ -93,7 +93,7 @@ def test_batch_invariant_generation_gives_a_request_the_same_tokens_in_any_batch
     outs = {}
     for graphs in (False, True):
         model = Model.load(model_dirs["D"], dtype="bfloat16", batch_invariant=True, max_batch=7, max_seq_len=128,
-                           use_graphs=graphs)
+                           use_graphs=graphs, graph_after=0)
         outs[graphs, "together"] = model.generate(prompts, max_new_tokens=24, sampling=sampling).tokens
         outs[graphs, "in fours"] = model.generate(prompts, max_new_tokens=24, sampling=sampling, max_batch=4).tokens
         outs[graphs, "alone"] = [model.generate([p], max_new_tokens=24, temperature=1.5, seed=100 + i).tokens[0]
@@ -117,7 +117,7 @@ def test_batches_of_tens_of_sequences(model_dirs, requests):
     stop = [int(t) for t in rng.integers(0, cfg["vocab_size"], 12)]             # a few sequences end on them
     outs = []
     for graphs in (False, True):
-        model = Model.load(model_dirs["D"], dtype="bfloat16", max_batch=requests, max_seq_len=96, use_graphs=graphs)
+        model = Model.load(model_dirs["D"], dtype="bfloat16", max_batch=requests, max_seq_len=96, use_graphs=graphs, graph_after=0)
         res = model.generate(prompts, max_new_tokens=12, stop_token_ids=stop)
         model.cache.check_consistent()
         assert model.cache.slots.free_count == requests
@@ -192,6 +192,32 @@ def test_an_engine_keeps_a_bounded_number_of_graphs(model_dirs):
             live = slots if step % 2 == 0 else slots[:2]
             rows.append(eng.step([StepEntry(s, [(5 * step + s) % 300], "last") for s in live]).clone())
             assert len(eng._graphs) <= 1
+        outs.append(rows)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
+def test_a_graph_is_captured_after_a_batch_size_has_been_used_a_few_times(model_dirs):
+    """``capture_after=3``: three steps of a batch size run with host launches, the fourth captures its graph; a size
+    that is used twice never gets one.  The logits are those of an engine that captures at once, bit for bit."""
+    import torch
+    from rust_inference_amd.engine import Engine, StepEntry
+    from rust_inference_amd.parts import load_model
+    model = load_model(model_dirs["B"], torch.float32)
+    cfg, _ = read_model_f64(model_dirs["B"])
+    prompts = prompts_for(cfg, [33, 2, 40], 5)
+    outs = []
+    for after in (0, 3):
+        eng = Engine(model, model.new_cache(max_tokens=3 * 96, num_slots=3, max_seq_len=96), use_graphs=True,
+                     capture_after=after)
+        slots = [eng.cache.acquire() for _ in prompts]
+        eng.step([StepEntry(s, p, "last") for s, p in zip(slots, prompts)])
+        rows = []
+        for step in range(8):
+            live = slots if step < 6 else slots[:2]              # six steps of three sequences, two of two
+            rows.append(eng.step([StepEntry(s, [(5 * step + s) % 300], "last") for s in live]).clone())
+            if after:
+                assert sorted(b for b, _ in eng._graphs) == ([3] if step >= 3 else [])
         outs.append(rows)
     for a, b in zip(*outs):
         assert torch.equal(a, b)

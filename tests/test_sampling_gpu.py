@@ -165,7 +165,7 @@ def test_a_repetition_penalty_gives_the_same_tokens_with_the_loop_running_ahead(
     kw = dict(max_new_tokens=24, temperature=0.9, top_k=30, repetition_penalty=1.4, seed=11)
     outs = {}
     for graphs in (True, False):
-        model = Model.load(model_dirs["A"], dtype=dtype_name, max_batch=4, max_seq_len=64, use_graphs=graphs)
+        model = Model.load(model_dirs["A"], dtype=dtype_name, max_batch=4, max_seq_len=64, use_graphs=graphs, graph_after=0)
         outs[graphs] = [model.generate(prompts, ignore_eos=True, **kw)]
         if dtype_name == "float32":
             outs[graphs].append(model.generate(prompts, stop_token_ids=[int(t) for t in outs[graphs][0].tokens[1][3:9]], **kw))
@@ -174,7 +174,7 @@ def test_a_repetition_penalty_gives_the_same_tokens_with_the_loop_running_ahead(
         assert a.tokens == b.tokens and a.finish_reasons == b.finish_reasons
     if dtype_name == "float32":
         assert "stop" in outs[True][1].finish_reasons
-    plain = Model.load(model_dirs["A"], dtype=dtype_name, max_batch=4, max_seq_len=64, use_graphs=True)
+    plain = Model.load(model_dirs["A"], dtype=dtype_name, max_batch=4, max_seq_len=64, use_graphs=True, graph_after=0)
     assert plain.generate(prompts, ignore_eos=True, **dict(kw, repetition_penalty=1.0)).tokens != outs[True][0].tokens
 
 
