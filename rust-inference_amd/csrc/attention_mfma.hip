@@ -943,16 +943,21 @@ attn_decode_stream_kernel(bf16_t* __restrict__ out, float* __restrict__ ws, cons
 #define STREAM_MIN_PER_CU 2
 #define STREAM_MIN_CHUNKS 8
 #define STREAM_JOINED_FROM 64
-// Eight wavefronts a workgroup and one run a sequence: where the step has one workgroup for every compute unit and
-// few more (up to an eighth: a second round on some units, or half the units idle, loses more than the join costs),
-// for sequences of up to STREAM_WIDE_MAX_CHUNKS chunks.
+// Eight wavefronts a workgroup and one run a sequence: where the step has a workgroup for four fifths of the compute
+// units or more but for none a second one (a second round on a few units doubles the kernel's time, and with half the
+// units idle the others pull no faster), for sequences of up to STREAM_WIDE_MAX_CHUNKS chunks.
 #ifndef STREAM_WIDE_MAX_CHUNKS
 #define STREAM_WIDE_MAX_CHUNKS 16
+#endif
+#ifndef STREAM_WIDE_BELOW
+#define STREAM_WIDE_BELOW 5       // from this share of the compute units below their number
+#define STREAM_WIDE_ABOVE 0       // to this share above it (0: to their number itself)
 #endif
 static bool stream_wide(int seqs, int kv_heads, int max_chunks) {
     const long rows = (long)seqs * kv_heads;
     const long cus = ri_compute_units();
-    return rows >= cus && rows <= cus + cus / 8 && rows < STREAM_MIN_PER_CU * cus && max_chunks <= STREAM_WIDE_MAX_CHUNKS;
+    const long lo = cus - (STREAM_WIDE_BELOW ? cus / STREAM_WIDE_BELOW : 0), hi = cus + (STREAM_WIDE_ABOVE ? cus / STREAM_WIDE_ABOVE : 0);
+    return rows >= lo && rows <= hi && rows < STREAM_MIN_PER_CU * cus && max_chunks <= STREAM_WIDE_MAX_CHUNKS;
 }
 
 static int stream_splits(int seqs, int kv_heads, int max_chunks) {

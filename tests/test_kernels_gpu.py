@@ -432,16 +432,16 @@ WIDE_LENS = [1, 32, 33, 256, 257, 512, 700, 5, 1025, 1200, 1199, 31, 64, 1024, 3
 @pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 100), (32, 8, 128, None),
                                                          (16, 8, 128, 300), (8, 8, 64, None)])
 def test_mfma_decode_attention_streams_short_sequences_with_eight_wavefronts(ops, heads, kv_heads, dh, window):
-    """Thirty-two sequences of eight kv heads and up to 1,200 keys: a run for every compute unit and few more, and
+    """Thirty-two sequences of eight kv heads and up to 1,200 keys: a run for every compute unit and none a second, and
     no sequence longer than sixteen chunks, is walked in one run by workgroups of eight wavefronts; some of the
     sequences have fewer pages than wavefronts."""
     if ops.compute_units() != 256:
         pytest.skip("the rule is written for the machine's size")
     rng = np.random.default_rng(78)
     assert ops.decode_attention_runs(len(WIDE_LENS), kv_heads, max(WIDE_LENS) + 300) == 1
-    assert ops.decode_attention_runs(len(WIDE_LENS) - 1, kv_heads, max(WIDE_LENS) + 300) == 0
+    assert ops.decode_attention_runs(len(WIDE_LENS) - 7, kv_heads, max(WIDE_LENS) + 300) == 0
     assert ops.decode_attention_runs(len(WIDE_LENS), kv_heads, 4097) == 0
-    assert ops.decode_attention_runs(len(WIDE_LENS) + 5, kv_heads, max(WIDE_LENS) + 300) == 0
+    assert ops.decode_attention_runs(len(WIDE_LENS) + 1, kv_heads, max(WIDE_LENS) + 300) == 0
 
     def boost(qkv, k, kp, table):
         head = 3 * (heads // kv_heads)                                 # sequence 9, kv head 3: its first query head
