@@ -33,6 +33,8 @@ MID_TILED_ROWS = 32              # and up to this many rows when the rows come t
 MID_TILED_BYTES = 64_000_000     # on matrices up to this size (7168 x 5120 draws level with the library, 10240 x 5120 loses: 28 us to 20)
 WIDE_MIN_K = 4096                # rows shorter than this leave the wide kernel's stretches too little to do
 WIDE_MIN_ROWS = 17
+SMALL_ONLY_ROWS = 48             # a matrix packed for small steps alone stays on the wide kernel up to this many rows
+# (5,120 x 8,192 at 32 / 48 / 64 rows: 20 / 24 / 29 us against the library's 19 to 34 / 30 / 23; 5,120 x 5,120: 15 / 18 / 21 against 19 / 20 / 19)
 WIDE_GATED_FILL = 0.9            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds,
 WIDE_GATED_ROWS = 48             # and up to this many rows whatever they fill, if the packed kernel of 17 to 64 rows is no match:
 WIDE_GATED_BYTES = 64_000_000    # pairs larger than this (smaller ones, up to 32 tiled rows, are that kernel's)
@@ -188,7 +190,7 @@ class Runtime:
         if self.dtype != torch.bfloat16 or pw.packed is None or pw.k % 8 or self.invariant:
             return False
         if pw.small_only:                                        # a packed copy made for small steps into the stream alone:
-            return parts_ok and 2 < m <= MID_TILED_ROWS          # the wide kernel takes those, nothing else of it
+            return parts_ok and 2 < m <= SMALL_ONLY_ROWS         # the wide kernel takes those, nothing else of it
         if GEMV_MAX_ROWS < m <= SKINNY_MAX_ROWS:
             return True
         if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and (self._wide_gated(pw, m) if pw.swiglu
@@ -254,7 +256,7 @@ class Runtime:
                     return ops.gemv_bf16(ops.as_rows(x), pw.w, out_dtype, swiglu=pw.swiglu)
                 return ops.gemm_skinny_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=pw.swiglu, tiled_out=tiles)
             if (WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
-                    and pw.k >= WIDE_MIN_K and not (pw.small_only and m > MID_TILED_ROWS)):
+                    and pw.k >= WIDE_MIN_K and not (pw.small_only and m > SMALL_ONLY_ROWS)):
                 # 17 to 64 rows into the residual stream: K in stretches, every stretch a workgroup that shares the tiles of x
                 # through LDS; the stream's next norm adds the stretches' sums
                 x = self.normed_now(x) if later else x
