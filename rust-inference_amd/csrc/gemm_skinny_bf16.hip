@@ -473,8 +473,8 @@ gemm_mid_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         x_ok[rt] = rt * 16 + i < M;
-        // (RT may be more tiles than x has: 33 to 48 rows are three tiles and run with RT = 4.  A tile beyond
-        // the last is never read: the loop that asks for every fragment reads the last tile again instead.)
+        // (RT may be more tiles than x has: up to 16 rows are one tile and run with RT = 2.  A tile beyond the
+        // last is never read: the loop that asks for every fragment reads the last tile again instead.)
         xp[rt] = (tiled & TILED_X) ? x + ((size_t)min(rt, (M - 1) >> 4) * k_tiles * 64 + lane) * 8
                                    : x + (size_t)(x_ok[rt] ? rt * 16 + i : 0) * K + jg * 8;
     }
@@ -595,6 +595,9 @@ extern "C" int ri_gemm_mid_packed_bf16(void* out, int out_dtype, const void* x, 
     if (m <= 32) {
         if (swiglu) { if (eight) RI_MID_CASE(8, true, 2); else RI_MID_CASE(4, true, 2); }
         else        { if (eight) RI_MID_CASE(8, false, 2); else RI_MID_CASE(4, false, 2); }
+    } else if (m <= 48) {
+        if (swiglu) { if (eight) RI_MID_CASE(8, true, 3); else RI_MID_CASE(4, true, 3); }
+        else        { if (eight) RI_MID_CASE(8, false, 3); else RI_MID_CASE(4, false, 3); }
     } else {
         if (swiglu) { if (eight) RI_MID_CASE(8, true, 4); else RI_MID_CASE(4, true, 4); }
         else        { if (eight) RI_MID_CASE(8, false, 4); else RI_MID_CASE(4, false, 4); }

@@ -113,18 +113,19 @@ def test_the_forms_that_a_large_step_chooses_on_a_machine_made_small(runs, units
     _passed(runs[units], tests)
 
 
-# The product for 17 to 64 rows once read a tile of x that its buffer does not have (33 to 48 rows are three
-# tiles of 16 and run with code built for four; the loads that are issued whatever the indices are read the
+# The product for 17 to 64 rows once read a tile of x that its buffer does not have (33 to 48 rows were three
+# tiles of 16 and ran with code built for four; the loads that are issued whatever the indices are read the
 # fourth): a kilobyte per step past the end of the buffer, which on the GPU faulted once in many runs.  The
-# address is pulled back to the last tile now; with the old expression put back the emulated run must end at
-# the guard page and say where.
+# address is pulled back to the last tile now (and 33 to 48 rows have code for three); the kernel still runs with
+# more tiles than x has where a step of up to 16 rows takes it, and with the old expression put back such a run
+# must end at the guard page and say where.
 OLD_MID = {"gemm_skinny_bf16.hip": ("min(rt, (M - 1) >> 4)", "rt")}
 PROBE = """
 import sys
 sys.path.insert(0, {here!r})
 import torch, emulated
 ops = emulated.ops(patches={patches!r})
-m, n, k = 40, 48, 1024
+m, n, k = 10, 48, 1024
 w = (torch.randn(n, k) * 0.1).bfloat16()
 x = ops.TiledRows.empty(m, k, "cpu")
 x.data.zero_()

@@ -746,7 +746,7 @@ def test_products_linked_to_norms(ops, packed, m, hidden, k, inter):
     close(chained.ssq.sum(1), (f64(residual) ** 2).sum(1), 1e-5, "sums of squares, second link")
 
 
-@pytest.mark.parametrize("m", [1, 17, 32, 33, 50, 64])
+@pytest.mark.parametrize("m", [1, 17, 32, 33, 41, 48, 50, 64])
 @pytest.mark.parametrize("n, k", [(37, 72), (1000, 1024), (584, 12288)])
 def test_packed_product_of_17_to_64_rows(ops, m, n, k):
     rng = np.random.default_rng(m + n)
