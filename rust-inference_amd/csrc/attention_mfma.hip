@@ -593,6 +593,39 @@ attn_decode_mfma_kernel(float* __restrict__ ws, const bf16_t* __restrict__ qkv, 
 #define JOIN_SERIAL 16
 #define JOIN_PARTS 8
 
+// G chunks of a run from `cb` on, all their loads asked for before any is used: the largest maximum, and the
+// chunks' results added in chunk order with the run's maximum `m`.
+template <int DH, int G>
+__device__ __forceinline__ void join_max(const float* __restrict__ base, int cb, int c1, float& m) {
+    float mc[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) mc[i] = base[min(cb + i, c1) * (DH + 2) + DH];
+#pragma unroll
+    for (int i = 0; i < G; ++i)
+        if (cb + i <= c1) m = fmaxf(m, mc[i]);
+}
+
+template <int DH, int G>
+__device__ __forceinline__ void join_sum(const float* __restrict__ base, int cb, int c1, int d, float m, float& acc,
+                                         float& l) {
+    float o[G], mc[G], lc[G];
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+        const float* at = base + min(cb + i, c1) * (DH + 2);
+        o[i] = at[d];
+        mc[i] = at[DH];
+        lc[i] = at[DH + 1];
+    }
+#pragma unroll
+    for (int i = 0; i < G; ++i) {
+        if (cb + i <= c1) {
+            const float f = mc[i] == -INFINITY ? 0.f : exp2f(mc[i] - m);
+            acc += o[i] * f;
+            l += lc[i] * f;
+        }
+    }
+}
+
 template <int DH, int PB>
 __global__ void __launch_bounds__(DH * PB)
 attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, const int32_t* __restrict__ tok_pos,
@@ -611,16 +644,18 @@ attn_decode_join_kernel(bf16_t* __restrict__ out, const float* __restrict__ ws, 
     const float* base = ws + ((long)b * heads + h) * max_chunks * (DH + 2);
     for (int p = tp; p < parts; p += PB) {
         const int c0 = c_lo + p * per, c1 = min(c_hi, c0 + per - 1);
+        // Sixteen chunks' loads are asked for at once while the run has sixteen more, then four at a time, each
+        // from an address pulled back into the run, and what lies past the run's end is left out where it would
+        // be used: a loop that fetches a chunk and then uses it makes a trip to memory for every chunk.  The
+        // sums are the same operations in the same order as such a loop's.
         float m = -INFINITY;
-        for (int c = c0; c <= c1; ++c) m = fmaxf(m, base[c * (DH + 2) + DH]);
+        int cb = c0;
+        for (; cb + JOIN_SERIAL - 1 <= c1; cb += JOIN_SERIAL) join_max<DH, JOIN_SERIAL>(base, cb, c1, m);
+        for (; cb <= c1; cb += 4) join_max<DH, 4>(base, cb, c1, m);
         float acc = 0.f, l = 0.f;
-#pragma unroll 4
-        for (int c = c0; c <= c1; ++c) {                            // always in chunk order
-            const float mc = base[c * (DH + 2) + DH];
-            const float f = mc == -INFINITY ? 0.f : exp2f(mc - m);
-            acc += base[c * (DH + 2) + d] * f;
-            l += base[c * (DH + 2) + DH + 1] * f;
-        }
+        cb = c0;                                                    // always in chunk order
+        for (; cb + JOIN_SERIAL - 1 <= c1; cb += JOIN_SERIAL) join_sum<DH, JOIN_SERIAL>(base, cb, c1, d, m, acc, l);
+        for (; cb <= c1; cb += 4) join_sum<DH, 4>(base, cb, c1, d, m, acc, l);
         if (parts == 1) {                                           // the whole workgroup is here or nowhere
             out[tiled ? tiled_at(b, h * DH + d, heads * DH / 32) : ((size_t)b * heads + h) * DH + d] = f32_to_bf16(acc / l);
             return;

@@ -406,6 +406,25 @@ def test_mfma_decode_attention_over_thousands_of_keys(ops, window):
         close(out, want, BF16_OUT, f"far key {far}, window {window}")
 
 
+def test_mfma_decode_attention_joins_more_chunks_than_a_run_fetches_at_once(ops):
+    """One kv head and 40,000 keys: 157 chunks, too few workgroups to stream, joined in eight runs of 20 chunks,
+    which a run fetches sixteen at a time.  A key that stands out among the first sixteen chunks of a run, among
+    its last four, and in the sequence's last chunk; beside it a sequence of 20 chunks (runs of three)."""
+    heads, kv_heads, dh = 2, 1, 32
+    lens = [40000, 5000]
+    assert not ops.decode_attention_streams(len(lens), kv_heads, max(lens) + 300)
+    for far in (100, 256 * 18 + 7, 39990):
+        rng = np.random.default_rng(61 + far)
+
+        def boost(qkv, k, kp, table, far=far):
+            kf = f64(kp[table[0, far // 32].item(), 0, far % 32])          # sequence 0, query head 1
+            qkv[0, dh:2 * dh] = 40.0 * kf / np.linalg.norm(kf) ** 2 * np.sqrt(dh)
+        out, want = attention_case(ops, rng, lens, [1] * len(lens), heads, kv_heads, dh, torch.bfloat16, boost=boost,
+                                   kernel="decode")
+        close(out, want, BF16_OUT, f"far key {far}")
+        assert np.abs(want[0, 1]).max() > 0
+
+
 @pytest.mark.parametrize("heads, kv_heads, dh, window", [(16, 8, 32, None), (16, 8, 32, 100), (16, 8, 32, 300),
                                                          (32, 8, 128, None), (32, 8, 128, 300), (8, 8, 64, None)])
 def test_mfma_decode_attention_streams_over_many_sequences(ops, heads, kv_heads, dh, window):
