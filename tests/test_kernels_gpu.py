@@ -841,7 +841,7 @@ def test_streaming_attention_walks_a_run_of_more_pages_than_it_holds_table_entri
     # on: position 39,990 of sequence 5, a key of sequence 9's last pages and one of sequence 20's page 1,024)
     for b, far, head in ((5, 9_000, 2), (5, 39_990, 3), (9, lens[9] - 100, 1), (20, 32_768 + 10, 4)):
         key = kp[table[b, far // 32].item(), head, far % 32].float()
-        qkv[b, head * dh:(head + 1) * dh] = (6.0 * key / key.norm() * dh ** 0.25).to(torch.bfloat16)
+        qkv[b, head * dh:(head + 1) * dh] = (8.0 * key / key.norm() * dh ** 0.25).to(torch.bfloat16)
     pos = t([n - 1 for n in lens], torch.int32)
     cu = t(np.arange(B + 1), torch.int32)
     seq = t(np.arange(B), torch.int32)
