@@ -142,6 +142,8 @@ int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float 
 // neighbouring row tiles, share the tiles of x through LDS.  parts > 1 cuts K into that many stretches whose
 // float32 sums go to out[parts][m][n]; ri_gemm_wide_packed_bf16_plan says how many wavefronts and parts fill
 // the machine most evenly for a matrix (with swiglu: never parts).  tiled as in ri_gemm_skinny_packed_bf16.
+// 65 to 128 rows of x: every wavefront takes two neighbouring row tiles; float32 sums in plain rows, no
+// activation, x in plain rows, depth 1; the plan for that form is asked for with swiglu = 2.
 int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts);
 int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
                              int swiglu, int parts, int tiled, int depth, int waves, void* stream);

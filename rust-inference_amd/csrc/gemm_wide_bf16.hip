@@ -19,6 +19,12 @@
 // few groups of row tiles to give every compute unit work, so K is cut into `parts` stretches (blockIdx.y) whose float32 sums go to out[part][M][N] for a reader
 // that adds them in order (the residual stream's norm, or ri_sum_parts below).  A row's result does not
 // depend on the number of rows: rows beyond M are zero columns, every tile of x has accumulators of its own.
+//
+// 65 to 128 rows (PAIR): five to eight tiles of x, and every wavefront takes two neighbouring row tiles of the
+// matrix, so that a fragment of x read from LDS meets two weight fragments (with one, the LDS reads of eight tiles
+// of x for every kilobyte of weights come close to what LDS delivers) and a workgroup's copy of x serves twice the
+// weights.  A slice of x is then up to 64 KB and the two buffers all of a compute unit's LDS that one workgroup
+// may have: one workgroup a compute unit, K in stretches, float32 sums for a reader that adds them.
 #include "api.h"
 #include "common.h"
 
@@ -34,8 +40,9 @@ union FragW {
 
 __device__ __forceinline__ float silu_wd(float z) { return z / (1.0f + expf(-z)); }
 
-// W: wavefronts of a workgroup, one row tile of the matrix each
-template <int RT, bool SWIGLU, typename TO, int NS, int W>
+// W: wavefronts of a workgroup, one row tile of the matrix each (with SWIGLU a gate tile and its up tile, with
+// PAIR two neighbouring tiles)
+template <int RT, bool SWIGLU, typename TO, int NS, int W, bool PAIR = false>
 __global__ void __launch_bounds__(W * 64)
 gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked, int M,
                         int N, int K, int k_tiles, int part_tiles, int row_tiles, int tiled) {
@@ -44,13 +51,17 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
     __shared__ uint4 xs[2][RT][WD_SLICE][64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nt = blockIdx.x * W + wave;
+    static_assert(!(SWIGLU && PAIR), "the second stream of weights is the up tile or the next row tile");
+    constexpr bool TWO = SWIGLU || PAIR;
+    const int nt = (blockIdx.x * W + wave) * (PAIR ? 2 : 1);
     const bool live_tile = nt < row_tiles;                    // past the edge: works on tile 0 again and stores nothing
     const int kt_begin = blockIdx.y * part_tiles, kt_end = min(k_tiles, kt_begin + part_tiles);
     const int slices = (kt_end - kt_begin + WD_SLICE - 1) / WD_SLICE;
     const int ntc = live_tile ? nt : 0;
     const bf16_t* wp = wpacked + ((size_t)ntc * k_tiles * 64 + lane) * 8;
-    const bf16_t* up = SWIGLU ? wpacked + ((size_t)(row_tiles + ntc) * k_tiles * 64 + lane) * 8 : nullptr;
+    // the second stream: the up tile of the pair, or the next row tile (past the edge: this one again, not stored)
+    const int nt2 = SWIGLU ? row_tiles + ntc : min(ntc + 1, row_tiles - 1);
+    const bf16_t* up = TWO ? wpacked + ((size_t)nt2 * k_tiles * 64 + lane) * 8 : nullptr;
     const bool x_tiled = tiled & TILED_X;
     const int jg = lane >> 4;
 
@@ -91,7 +102,7 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
         for (int c = 0; c < WD_SLICE; ++c) {
             const int kt = min(kt_begin + ss * WD_SLICE + c, kt_last);
             wf[ss][c].u = load_stream16(wp + (size_t)kt * 512);
-            if (SWIGLU) uf[ss][c].u = load_stream16(up + (size_t)kt * 512);
+            if (TWO) uf[ss][c].u = load_stream16(up + (size_t)kt * 512);
         }
     uint4 stage[PER_THREAD];
 #pragma unroll
@@ -118,13 +129,13 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
                     FragW xf;
                     xf.u = xs[buf][rt][c][lane];
                     acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[ss][c].v, xf.v, acc[rt], 0, 0, 0);
-                    if (SWIGLU) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[ss][c].v, xf.v, accu[rt], 0, 0, 0);
+                    if (TWO) accu[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[ss][c].v, xf.v, accu[rt], 0, 0, 0);
                 }
                 // this register's step NS slices on (past the end: the stretch's last tile again, which then
                 // meets zeros of x)
                 const int next = min(kt0 + NS * WD_SLICE + c, kt_last);
                 wf[ss][c].u = load_stream16(wp + (size_t)next * 512);
-                if (SWIGLU) uf[ss][c].u = load_stream16(up + (size_t)next * 512);
+                if (TWO) uf[ss][c].u = load_stream16(up + (size_t)next * 512);
             }
 #pragma unroll
             for (int j = 0; j < PER_THREAD; ++j) stash(j, buf ^ 1, stage[j]);
@@ -147,6 +158,11 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
         for (int r = 0; r < 4; ++r) {
             const int n = nt * 16 + 4 * jg + r;
             if (n >= N) continue;
+            if (PAIR) {                                      // the sums of both row tiles as they are
+                from_f32(out + (size_t)m * width + n, acc[rt][r]);
+                if (n + 16 < N) from_f32(out + (size_t)m * width + n + 16, accu[rt][r]);
+                continue;
+            }
             if (SWIGLU && raw) {
                 from_f32(out + (size_t)m * width + n, acc[rt][r]);
                 from_f32(out + (size_t)m * width + N + n, accu[rt][r]);
@@ -170,13 +186,23 @@ static int wide_parts(int groups, int k_tiles, bool swiglu, int cus) {
     return parts;
 }
 
+// swiglu 2: no activation, but 65 to 128 rows of x, two row tiles a wavefront.  A compute unit then holds one
+// workgroup (its two buffers of x are most of the LDS), so K is cut only while the workgroups stay within the
+// compute units' number: 4096 x 12288 at 96 rows takes 33 us in 8 stretches (256 workgroups), 45 in 4 and 44 in
+// 16; 5120 x 17408 in 54 groups of three wavefronts 66 us in 4 stretches, 78 in 8.
 extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts) {
     const int row_tiles = (n + 15) / 16, k_tiles = (k + 31) / 32;
     const int cus = ri_compute_units();
+    const bool pairs = swiglu == 2;
     double best = -1.0;
     for (int w = 4; w >= 3; --w) {
-        const int groups = (row_tiles + w - 1) / w;
-        const int p = wide_parts(groups, k_tiles, swiglu != 0, cus);
+        const int per = pairs ? 2 * w : w;
+        const int groups = (row_tiles + per - 1) / per;
+        int p = 1;
+        if (pairs)
+            while (p < 16 && groups * p * 2 <= cus && k_tiles / (p * 2) >= 2 * WD_SLICE) p *= 2;
+        else
+            p = wide_parts(groups, k_tiles, swiglu == 1, cus);
         const long wgs = (long)groups * p;
         const double fill = (double)wgs / (double)((wgs + cus - 1) / cus * cus);
         if (fill > best + 1e-9) {
@@ -186,6 +212,15 @@ extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* wave
         }
     }
     return 0;
+}
+
+template <int RT, int W>
+static void launch_wide_pairs(float* out, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts, hipStream_t s) {
+    const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
+    const int part_tiles = ((k_tiles + parts - 1) / parts + WD_SLICE - 1) / WD_SLICE * WD_SLICE;
+    dim3 grid((row_tiles + 2 * W - 1) / (2 * W), parts);
+    gemm_wide_packed_kernel<RT, false, float, 1, W, true><<<grid, W * 64, 0, s>>>(out, x, w, m, n, k, k_tiles, part_tiles,
+                                                                                 row_tiles, 0);
 }
 
 template <int RT, bool SWIGLU, int NS, int W>
@@ -208,7 +243,10 @@ static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t*
 // against 13.6 us and 24.8 against 24.2 us at 64 rows, and the reading norm then adds twice the stretches.)
 extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
                                         int k, int swiglu, int parts, int tiled, int depth, int waves, void* stream) {
-    RI_REQUIRE(m > 0 && m <= 64, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 64", m);
+    RI_REQUIRE(m > 0 && m <= 128, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 128", m);
+    RI_REQUIRE(m <= 64 || (!swiglu && out_dtype == RI_F32 && !tiled && depth == 1),
+               "gemm_wide_packed_bf16: %d rows of x: more than 64 give float32 sums in plain rows from plain rows, "
+               "without the activation, one slice of weights in flight", m);
     RI_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_wide_packed_bf16: n %d, k %d (k must be a multiple of 8)", n, k);
     RI_REQUIRE(out_dtype == RI_F32 || out_dtype == RI_BF16, "gemm_wide_packed_bf16: out dtype %d", out_dtype);
     RI_REQUIRE(parts >= 1 && parts <= 64 && (parts == 1 || out_dtype == RI_F32),
@@ -228,10 +266,20 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
 #define RI_WIDE_CASE(RT)                                                                  \
     if (swiglu) { if (depth == 2) RI_WIDE_GO(RT, true, 2); else RI_WIDE_GO(RT, true, 1); } \
     else        { if (depth == 2) RI_WIDE_GO(RT, false, 2); else RI_WIDE_GO(RT, false, 1); }
-    if (m <= 16)      { RI_WIDE_CASE(1) }
-    else if (m <= 32) { RI_WIDE_CASE(2) }
-    else if (m <= 48) { RI_WIDE_CASE(3) }
-    else              { RI_WIDE_CASE(4) }
+#define RI_WIDE_PAIRS(RT)                                                                      \
+    do {                                                                                        \
+        if (waves == 3) launch_wide_pairs<RT, 3>((float*)out, xb, wb, m, n, k, parts, s);       \
+        else            launch_wide_pairs<RT, 4>((float*)out, xb, wb, m, n, k, parts, s);       \
+    } while (0)
+    if (m <= 16)       { RI_WIDE_CASE(1) }
+    else if (m <= 32)  { RI_WIDE_CASE(2) }
+    else if (m <= 48)  { RI_WIDE_CASE(3) }
+    else if (m <= 64)  { RI_WIDE_CASE(4) }
+    else if (m <= 80)  RI_WIDE_PAIRS(5);
+    else if (m <= 96)  RI_WIDE_PAIRS(6);
+    else if (m <= 112) RI_WIDE_PAIRS(7);
+    else               RI_WIDE_PAIRS(8);
+#undef RI_WIDE_PAIRS
 #undef RI_WIDE_CASE
 #undef RI_WIDE_GO
     RI_LAUNCH_CHECK("gemm_wide_packed_bf16");

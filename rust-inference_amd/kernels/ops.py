@@ -517,12 +517,15 @@ def compute_units() -> int:
     return int(_get("ri_compute_units")())
 
 
-def wide_product_plan(n: int, k: int, swiglu: bool = False) -> tuple[int, int]:
+def wide_product_plan(n: int, k: int, swiglu: bool = False, pairs: bool = False) -> tuple[int, int]:
     """``(waves, parts)``: how many wavefronts a workgroup of ``gemm_wide_packed_bf16`` should have and into how
     many stretches of K it should cut a product with an ``n x k`` matrix so that the compute units are filled
-    evenly (host code only)."""
+    evenly (host code only).  ``pairs``: for 65 to 128 rows of x, where a wavefront takes two row tiles."""
+    if swiglu and pairs:
+        raise ShapeError("more than 64 rows go without the activation")
     waves, parts = ctypes.c_int(0), ctypes.c_int(0)
-    _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), int(swiglu), ctypes.addressof(waves), ctypes.addressof(parts))
+    _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), 2 if pairs else int(swiglu), ctypes.addressof(waves),
+          ctypes.addressof(parts))
     return waves.value, parts.value
 
 
@@ -530,6 +533,7 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
                           parts: int = 1, tiled_out: bool = False, depth: int = 2, waves: int = 4):
     """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by ``pack_for_mfma``,
     the tiles of x shared by a workgroup's wavefronts through LDS: the product for steps of 17 to 64 tokens.
+    65 to 128 plain rows: float32 sums in rows (``parts`` from ``wide_product_plan(..., pairs=True)``), ``depth`` 1.
     ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
     that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
     ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``.  ``waves``: wavefronts (row tiles) a
@@ -539,6 +543,10 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
     want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)
     if tuple(wpacked.shape) != want:
         raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
+    if m > 64:
+        if swiglu or out_dtype != torch.float32 or tiled_out or isinstance(x, TiledRows):
+            raise ShapeError("more than 64 rows: float32 sums in plain rows from plain rows, without the activation")
+        depth = 1
     if parts != 1 and (out_dtype != torch.float32 or tiled_out):
         raise ShapeError("a product in parts has float32 sums in rows")
     if tiled_out and out_dtype != torch.bfloat16:

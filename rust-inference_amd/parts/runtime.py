@@ -11,9 +11,9 @@ from ..kernels import ops
 
 
 @functools.lru_cache(maxsize=None)
-def _wide_plan(n: int, k: int, swiglu: bool) -> tuple[int, int]:
+def _wide_plan(n: int, k: int, swiglu: bool, pairs: bool = False) -> tuple[int, int]:
     """``ops.wide_product_plan``, asked once per matrix size."""
-    return ops.wide_product_plan(n, k, swiglu)
+    return ops.wide_product_plan(n, k, swiglu, pairs)
 
 # Which product kernel runs, by the number of rows of x (bfloat16; the measurements behind every constant
 # here are written up with the design notes, under "Which product kernel serves which step"):
@@ -24,6 +24,8 @@ def _wide_plan(n: int, k: int, swiglu: bool) -> tuple[int, int]:
 #   17-64      the wide kernel (tiles of x shared through LDS) where the reader adds stretches of K or the
 #              gate|up pairs fill the machine; the packed kernel with two or four tiles of x on small matrices
 #              and up to 32 rows of tiled x; else the library.
+#   65-128     the wide kernel with two row tiles a wavefront for matrices of long rows whose reader adds stretches
+#              of K (`down`); else the library.
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
 GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
@@ -33,6 +35,8 @@ MID_TILED_ROWS = 32              # and up to this many rows when the rows come t
 MID_TILED_BYTES = 64_000_000     # on matrices up to this size (7168 x 5120 draws level with the library, 10240 x 5120 loses: 28 us to 20)
 WIDE_MIN_K = 4096                # rows shorter than this leave the wide kernel's stretches too little to do
 WIDE_MIN_ROWS = 17
+PAIRS_MAX_ROWS = 128             # 65 to 128 rows: the wide kernel with two row tiles a wavefront, where the library does badly:
+PAIRS_MIN_K = 8192               # matrices of long rows (and at least twice as long as there are rows: `down`)
 SMALL_ONLY_ROWS = 48             # a matrix packed for small steps alone stays on the wide kernel up to this many rows
 # (5,120 x 8,192 at 32 / 48 / 64 rows: 20 / 24 / 29 us against the library's 19 to 34 / 30 / 23; 5,120 x 5,120: 15 / 18 / 21 against 19 / 20 / 19)
 WIDE_GATED_FILL = 0.9            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds,
@@ -261,6 +265,14 @@ class Runtime:
                 # through LDS; the stream's next norm adds the stretches' sums
                 x = self.normed_now(x) if later else x
                 waves, parts = _wide_plan(pw.n, pw.k, False)
+                return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
+            if (MID_MAX_ROWS < m <= PAIRS_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
+                    and pw.k >= PAIRS_MIN_K and pw.k >= 2 * pw.n):
+                # 65 to 128 rows against a matrix of long rows whose result goes into the residual stream (`down`):
+                # the wide kernel with two row tiles a wavefront, K in stretches that the stream's next norm adds
+                x = self.normed_now(x) if later else x
+                x = x.rows() if isinstance(x, ops.TiledRows) else x
+                waves, parts = _wide_plan(pw.n, pw.k, False, True)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
             if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw, m):
                 x = self.normed_now(x) if later else x

@@ -439,18 +439,19 @@ def test_one_layer_of_the_large_model(tmp_path_factory, dtype_name):
             check_against_plain(folder, got, reqs, dtype_name, f"large layer, {what}, graphs {graphs}")
 
 
-# The layer sizes of the published Qwen3 dense checkpoints other than 8B (name: hidden, intermediate, heads, kv
-# heads): what the kernels' rules choose at each (rows of 1,024 to 25,600 elements, 2 to 8 query heads a kv head,
-# K of 2,560 and 9,728 that the ring of eight steps does not divide).
+# The layer sizes of the published Qwen3 dense checkpoints (name: hidden, intermediate, heads, kv heads): what the
+# kernels' rules choose at each (rows of 1,024 to 25,600 elements, 2 to 8 query heads a kv head, K of 2,560 and
+# 9,728 that the ring of eight steps does not divide).
 PUBLISHED = {"0.6B": (1024, 3072, 16, 8), "1.7B": (2048, 6144, 16, 8), "4B": (2560, 9728, 32, 8),
-             "14B": (5120, 17408, 40, 8), "32B": (5120, 25600, 64, 8)}
+             "8B": (4096, 12288, 32, 8), "14B": (5120, 17408, 40, 8), "32B": (5120, 25600, 64, 8)}
 
 
 @pytest.mark.parametrize("size", list(PUBLISHED))
 def test_one_layer_of_every_published_size(tmp_path, size):
     """One layer and a small vocabulary at each size, bfloat16, through graphs: a request alone with its last
-    tokens one by one (the one-row products), batches of five, twenty and forty-four of unequal lengths (the
-    packed products of 2 to 16 rows, the wide ones of 17 to 32, those of 33 to 64, the library's for the prompts)."""
+    tokens one by one (the one-row products), batches of five, twenty, forty-four and ninety of unequal lengths (the
+    packed products of 2 to 16 rows, the wide ones of 17 to 32, of 33 to 64 and of 65 to 128, the library's for the
+    prompts)."""
     from rust_inference_amd.engine import Engine
     from rust_inference_amd.engine.replay import Replayer
     from rust_inference_amd.parts import load_model
@@ -464,9 +465,10 @@ def test_one_layer_of_every_published_size(tmp_path, size):
     rng = np.random.default_rng(len(size) + hidden)
     model = load_model(folder, torch.bfloat16)
     try:
-        for count, tail in ((1, 12), (5, 6), (20, 5), (44, 4)):
+        for count, tail in ((1, 12), (5, 6), (20, 5), (44, 4), (90, 4)):
+            longest = 140 if count == 1 else 48 if count < 90 else 20
             reqs = {f"{size}_{count}_{i}": [int(t) for t in rng.integers(0, 1000, n)]
-                    for i, n in enumerate(rng.integers(tail + 1, 48 if count > 1 else 140, count))}
+                    for i, n in enumerate(rng.integers(tail + 1, longest, count))}
             steps = (plans.tail_one_by_one(reqs, tail) if count == 1 else
                      plans.unequal_batches([{k: (v, len(v) - int(rng.integers(1, tail + 1))) for k, v in reqs.items()}]))
             cache = model.new_cache(max_tokens=plans.max_live_tokens(steps), num_slots=count, max_seq_len=192)

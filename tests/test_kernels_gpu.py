@@ -725,6 +725,36 @@ def test_wide_packed_product(ops, m, n, k):
         assert torch.equal(whole[m - 1:], ops.gemm_wide_packed_bf16(x[m - 1:].contiguous(), packed, n, torch.float32))
 
 
+@pytest.mark.parametrize("m", [65, 80, 81, 100, 113, 128])
+@pytest.mark.parametrize("n, k", [(37, 72), (1000, 1024), (584, 12288), (4096, 4096), (70, 264), (16, 520)])
+def test_wide_packed_product_of_65_to_128_rows(ops, m, n, k):
+    """Five to eight tiles of x, two row tiles of the matrix a wavefront (an odd number of row tiles leaves the last
+    wavefront one): whole and in parts of K that add up, with three and four wavefronts a workgroup; a row's sums
+    are those of the kernel for up to 64 rows, bit for bit."""
+    rng = np.random.default_rng(m + n + k)
+    x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
+    want = f64(x) @ f64(w).T
+    packed = ops.pack_for_mfma(w)
+    whole = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32)
+    assert whole.shape == (m, n)
+    close(whole, want, 3e-6, "wide product of more than 64 rows")
+    waves, planned = ops.wide_product_plan(n, k, pairs=True)
+    assert waves in (3, 4) and planned >= 1
+    for parts in (2, 3, planned):
+        got = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=parts, waves=waves)
+        assert got.shape == ((parts, m, n) if parts > 1 else (m, n))
+        if parts > 1:
+            close(got.sum(0), want, 3e-6, f"{parts} parts of K")
+        assert torch.equal(got, ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=parts, waves=7 - waves))
+        first = ops.gemm_wide_packed_bf16(x[:64].contiguous(), packed, n, torch.float32, parts=parts, depth=1)
+        last = ops.gemm_wide_packed_bf16(x[m - 1:].contiguous(), packed, n, torch.float32, parts=parts, depth=1)
+        assert torch.equal(got[..., :64, :], first) and torch.equal(got[..., m - 1:, :], last)
+    with pytest.raises(Exception, match="64"):
+        ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16)
+    with pytest.raises(Exception, match="128"):
+        ops.gemm_wide_packed_bf16(t(rng.normal(size=(129, k)), torch.bfloat16), packed, n, torch.float32)
+
+
 @pytest.mark.parametrize("packed, m", [(False, 1), (False, 2), (False, 5), (True, 1), (True, 3), (True, 16)])
 @pytest.mark.parametrize("hidden, k, inter", [(104, 72, 56), (4096, 4096, 1000), (584, 12288, 37)])
 def test_products_linked_to_norms(ops, packed, m, hidden, k, inter):
