@@ -47,6 +47,7 @@ _SIGNATURES = {
     "ri_gemm_wide_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_int, c_void_p],
     "ri_gemm_wide_packed_bf16_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
+    "ri_gemm_wide_pairs_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
     "ri_compute_units": [],
     "ri_sum_parts": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
@@ -517,15 +518,17 @@ def compute_units() -> int:
     return int(_get("ri_compute_units")())
 
 
-def wide_product_plan(n: int, k: int, swiglu: bool = False, pairs: bool = False) -> tuple[int, int]:
+def wide_product_plan(n: int, k: int, swiglu: bool = False, rows: int = 64) -> tuple[int, int]:
     """``(waves, parts)``: how many wavefronts a workgroup of ``gemm_wide_packed_bf16`` should have and into how
     many stretches of K it should cut a product with an ``n x k`` matrix so that the compute units are filled
-    evenly (host code only).  ``pairs``: for 65 to 128 rows of x, where a wavefront takes two row tiles."""
-    if swiglu and pairs:
-        raise ShapeError("more than 64 rows go without the activation")
+    evenly (host code only).  ``rows`` above 64: for that many rows of x, where a wavefront takes two row tiles."""
     waves, parts = ctypes.c_int(0), ctypes.c_int(0)
-    _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), 2 if pairs else int(swiglu), ctypes.addressof(waves),
-          ctypes.addressof(parts))
+    if rows > 64:
+        if swiglu:
+            raise ShapeError("more than 64 rows go without the activation")
+        _call("ri_gemm_wide_pairs_plan", int(rows), int(n), int(k), ctypes.addressof(waves), ctypes.addressof(parts))
+    else:
+        _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), int(swiglu), ctypes.addressof(waves), ctypes.addressof(parts))
     return waves.value, parts.value
 
 
@@ -533,7 +536,8 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
                           parts: int = 1, tiled_out: bool = False, depth: int = 2, waves: int = 4):
     """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by ``pack_for_mfma``,
     the tiles of x shared by a workgroup's wavefronts through LDS: the product for steps of 17 to 64 tokens.
-    65 to 128 plain rows: float32 sums in rows (``parts`` from ``wide_product_plan(..., pairs=True)``), ``depth`` 1.
+    65 to 128 plain rows: float32 sums in rows (``waves`` and ``parts`` from ``wide_product_plan(..., rows=m)``),
+    ``depth`` 1.
     ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
     that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
     ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``.  ``waves``: wavefronts (row tiles) a

@@ -11,9 +11,9 @@ from ..kernels import ops
 
 
 @functools.lru_cache(maxsize=None)
-def _wide_plan(n: int, k: int, swiglu: bool, pairs: bool = False) -> tuple[int, int]:
-    """``ops.wide_product_plan``, asked once per matrix size."""
-    return ops.wide_product_plan(n, k, swiglu, pairs)
+def _wide_plan(n: int, k: int, swiglu: bool, rows: int = 64) -> tuple[int, int]:
+    """``ops.wide_product_plan``, asked once per matrix size (and, above 64 rows, per tile of 16 rows)."""
+    return ops.wide_product_plan(n, k, swiglu, rows)
 
 # Which product kernel runs, by the number of rows of x (bfloat16; the measurements behind every constant
 # here are written up with the design notes, under "Which product kernel serves which step"):
@@ -272,7 +272,7 @@ class Runtime:
                 # the wide kernel with two row tiles a wavefront, K in stretches that the stream's next norm adds
                 x = self.normed_now(x) if later else x
                 x = x.rows() if isinstance(x, ops.TiledRows) else x
-                waves, parts = _wide_plan(pw.n, pw.k, False, True)
+                waves, parts = _wide_plan(pw.n, pw.k, False, -(-m // 16) * 16)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
             if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw, m):
                 x = self.normed_now(x) if later else x

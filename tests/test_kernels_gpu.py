@@ -738,7 +738,7 @@ def test_wide_packed_product_of_65_to_128_rows(ops, m, n, k):
     whole = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32)
     assert whole.shape == (m, n)
     close(whole, want, 3e-6, "wide product of more than 64 rows")
-    waves, planned = ops.wide_product_plan(n, k, pairs=True)
+    waves, planned = ops.wide_product_plan(n, k, rows=m)
     assert waves in (3, 4) and planned >= 1
     for parts in (2, 3, planned):
         got = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=parts, waves=waves)
