@@ -143,9 +143,10 @@ int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float 
 // float32 sums go to out[parts][m][n]; ri_gemm_wide_packed_bf16_plan says how many wavefronts and parts fill
 // the machine most evenly for a matrix (with swiglu: never parts).  tiled as in ri_gemm_skinny_packed_bf16.
 // 65 to 128 rows of x: every wavefront takes two neighbouring row tiles; float32 sums in plain rows, no
-// activation, x in plain rows, depth 1; wavefronts and stretches planned by ri_gemm_wide_pairs_plan.
+// activation, x in plain rows, depth 1.  ri_gemm_wide_stretch_plan: wavefronts and stretches for a product of m
+// rows without the activation.
 int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts);
-int ri_gemm_wide_pairs_plan(int m, int n, int k, int* waves, int* parts);
+int ri_gemm_wide_stretch_plan(int m, int n, int k, int* waves, int* parts);
 int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n, int k,
                              int swiglu, int parts, int tiled, int depth, int waves, void* stream);
 // (depth: 1 or 2 slices of eight weight fragments that a wavefront keeps in flight.  With parts > 1 and swiglu

@@ -204,34 +204,43 @@ extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* wave
     return 0;
 }
 
-// The same for 65 to 128 rows of x, two row tiles a wavefront.  A compute unit then holds one workgroup (its two
-// buffers of x are most of the LDS), so more workgroups than compute units are a second round: K is cut only
-// while they stay within that number (4096 x 12288 at 96 rows takes 33 us in 8 stretches, 256 workgroups, 45 in 4
-// and 44 in 16).  Within that, the product is about as fast as a compute unit fetches its workgroup's bytes (some
-// 30 GB/s, from memory or from the L2 cache alike): the rows of x and the weight rows over one stretch, and its
-// share of the float32 stretches that are written here and read again by whoever adds them.  Of three and four
-// wavefronts and every number of stretches, a power of two or not, the plan takes the one with the fewest such
-// bytes (5120 x 17408 at 128 rows: 40 groups of four wavefronts in 6 stretches 66 us, 54 groups of three in 4
-// stretches 88; 2560 x 9728: 20 groups in 10 stretches 31 us, in 8 stretches 34).
-// (Eight wavefronts, 256 weight rows to a copy of x, were timed too: 4 to 6% ahead at 128 rows of x on the matrices
-// of many long rows, 5120 x 17408 and x 25600 in 12 stretches, 5 to 8% behind at 80 rows, and 13% behind on
-// 4096 x 12288, whose stretches get short.)
-extern "C" int ri_gemm_wide_pairs_plan(int m, int n, int k, int* waves, int* parts) {
+// The plan for a product without the activation by the rows of x too.  Up to 16 rows it is the one above: x is
+// small, and twice the workgroups, two to a compute unit, keep more loads in flight.  From 17 rows on a
+// workgroup's copy of x weighs as much as its weights, and the product is about as fast as a compute unit fetches
+// its workgroups' bytes (some 30 GB/s, from memory or from the L2 cache alike): the rows of x and the weight rows
+// over one stretch, and its share of the float32 stretches that are written here and read again by whoever adds
+// them.  K is cut only while the workgroups stay within the compute units' number (65 to 128 rows, two row tiles
+// a wavefront: a compute unit holds one workgroup then, its two buffers of x are most of the LDS, and more are a
+// second round; 4096 x 12288 at 96 rows takes 33 us in 8 stretches, 256 workgroups, 45 in 4 and 44 in 16; at 64
+// rows 26.5 us in 4 stretches and 29 in 8).  Of three and four wavefronts and every number of stretches, a power
+// of two or not, the plan takes the one with the fewest bytes.  5120 x 17408 at 64 rows: 80 groups of four
+// wavefronts in 3 stretches 43 us, 107 groups of three in 4 stretches, what the plan above says, 56; 2560 x 9728:
+// 40 groups in 6 stretches 17 us, 54 in 8 stretches 21.5; at 128 rows 5120 x 17408 as 40 groups in 6 stretches 66 us,
+// as 54 in 4 stretches 88.  At 4 and 16 rows the same choice makes a decode step at Qwen3-14B and 32B sizes 1.3 to
+// 2.6% longer.
+// (Eight wavefronts, 256 weight rows to a copy of x, were timed too at 65 to 128 rows: 4 to 6% ahead at 128 rows of
+// x on the matrices of many long rows, 5120 x 17408 and x 25600 in 12 stretches, 5 to 8% behind at 80 rows, and 13%
+// behind on 4096 x 12288, whose stretches get short.)
+extern "C" int ri_gemm_wide_stretch_plan(int m, int n, int k, int* waves, int* parts) {
+    if (m <= 16) return ri_gemm_wide_packed_bf16_plan(n, k, 0, waves, parts);
     const int row_tiles = (n + 15) / 16, k_tiles = (k + 31) / 32;
     const int cus = ri_compute_units();
     const int x_rows = (m + 15) / 16 * 16;
     double best = -1.0;
     *waves = 4;
     *parts = 1;
+    const int tiles_a_wave = m > 64 ? 2 : 1;
     for (int w = 4; w >= 3; --w) {
-        const int groups = (row_tiles + 2 * w - 1) / (2 * w);
+        const int groups = (row_tiles + tiles_a_wave * w - 1) / (tiles_a_wave * w);
         const int most = max(1, min(16, cus / groups));
+        const long rounds = (groups + cus - 1) / cus;                   // (more than one only where K stays whole)
         for (int p = 1; p <= most; ++p) {
             const int stretch = ((k_tiles + p - 1) / p + WD_SLICE - 1) / WD_SLICE * WD_SLICE;
             if (p > 1 && stretch < 2 * WD_SLICE) break;
             const int used = (k_tiles + stretch - 1) / stretch;          // stretches that hold any of K
             if (used != p) continue;
-            const double bytes = (double)(x_rows + 32 * w) * stretch * 64.0 + (double)used * m * n * 8.0 / cus;
+            const double bytes = (double)rounds * (x_rows + 16 * tiles_a_wave * w) * stretch * 64.0 +
+                                 (double)used * m * n * 8.0 / cus;
             if (best < 0 || bytes < best * (1.0 - 1e-9)) {
                 best = bytes;
                 *waves = w;

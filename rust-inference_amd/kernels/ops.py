@@ -47,7 +47,7 @@ _SIGNATURES = {
     "ri_gemm_wide_packed_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_int, c_void_p],
     "ri_gemm_wide_packed_bf16_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
-    "ri_gemm_wide_pairs_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
+    "ri_gemm_wide_stretch_plan": [c_int, c_int, c_int, c_void_p, c_void_p],
     "ri_compute_units": [],
     "ri_sum_parts": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "ri_attention_decode_chunks": [c_int],
@@ -520,15 +520,16 @@ def compute_units() -> int:
 
 def wide_product_plan(n: int, k: int, swiglu: bool = False, rows: int = 64) -> tuple[int, int]:
     """``(waves, parts)``: how many wavefronts a workgroup of ``gemm_wide_packed_bf16`` should have and into how
-    many stretches of K it should cut a product with an ``n x k`` matrix so that the compute units are filled
-    evenly (host code only).  ``rows`` above 64: for that many rows of x, where a wavefront takes two row tiles."""
+    many stretches of K it should cut a product of ``rows`` rows with an ``n x k`` matrix (host code only): with the
+    activation K whole and the wavefronts that fill the compute units more evenly; without it, from 17 rows on,
+    what makes a compute unit fetch the fewest bytes."""
     waves, parts = ctypes.c_int(0), ctypes.c_int(0)
-    if rows > 64:
-        if swiglu:
+    if swiglu:
+        if rows > 64:
             raise ShapeError("more than 64 rows go without the activation")
-        _call("ri_gemm_wide_pairs_plan", int(rows), int(n), int(k), ctypes.addressof(waves), ctypes.addressof(parts))
+        _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), 1, ctypes.addressof(waves), ctypes.addressof(parts))
     else:
-        _call("ri_gemm_wide_packed_bf16_plan", int(n), int(k), int(swiglu), ctypes.addressof(waves), ctypes.addressof(parts))
+        _call("ri_gemm_wide_stretch_plan", int(rows), int(n), int(k), ctypes.addressof(waves), ctypes.addressof(parts))
     return waves.value, parts.value
 
 

@@ -12,7 +12,7 @@ from ..kernels import ops
 
 @functools.lru_cache(maxsize=None)
 def _wide_plan(n: int, k: int, swiglu: bool, rows: int = 64) -> tuple[int, int]:
-    """``ops.wide_product_plan``, asked once per matrix size (and, above 64 rows, per tile of 16 rows)."""
+    """``ops.wide_product_plan``, asked once per matrix size and tile of 16 rows."""
     return ops.wide_product_plan(n, k, swiglu, rows)
 
 # Which product kernel runs, by the number of rows of x (bfloat16; the measurements behind every constant
@@ -228,7 +228,7 @@ class Runtime:
                 # (the parts beat a link to the next norm, as they do for the packed kernel's own; two rows of a
                 # matrix that had no packed copy stay with the kernel of one wavefront a row, which takes the link)
                 x = self.normed_now(x) if later else x
-                waves, parts = _wide_plan(pw.n, pw.k, False)
+                waves, parts = _wide_plan(pw.n, pw.k, False, -(-m // 16) * 16)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
             if (SKINNY_MAX_ROWS // 2 < m <= SKINNY_MAX_ROWS and pw.swiglu and pw.packed is not None and not later
                     and pw.k >= WIDE_MIN_K):
@@ -264,7 +264,7 @@ class Runtime:
                 # 17 to 64 rows into the residual stream: K in stretches, every stretch a workgroup that shares the tiles of x
                 # through LDS; the stream's next norm adds the stretches' sums
                 x = self.normed_now(x) if later else x
-                waves, parts = _wide_plan(pw.n, pw.k, False)
+                waves, parts = _wide_plan(pw.n, pw.k, False, -(-m // 16) * 16)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
             if (MID_MAX_ROWS < m <= PAIRS_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
                     and pw.k >= PAIRS_MIN_K and pw.k >= 2 * pw.n):

@@ -691,7 +691,7 @@ def test_wide_packed_product(ops, m, n, k):
     whole = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32)
     close(whole, want, 3e-6, "wide product")
     close(ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16), want, 5e-3, "wide product, bfloat16 out")
-    for parts in (2, 3, ops.wide_product_plan(n, k)[1]):
+    for parts in (2, 3, ops.wide_product_plan(n, k, rows=m)[1]):
         got = ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=parts)
         assert got.shape == ((parts, m, n) if parts > 1 else (m, n))
         if parts > 1:
