@@ -15,7 +15,8 @@
 // the machine's), so the product is as fast as the fullest compute unit: the workgroups should be a multiple
 // of the compute units, all alike.  Three wavefronts instead of four do that for a matrix whose row tiles are
 // a multiple of three times the compute units (768 pairs of gate|up tiles: 256 workgroups of three, where
-// groups of four make 192 and leave a quarter of the machine idle).  A matrix of a few thousand rows has too
+// groups of four make 192 and leave a quarter of the machine idle), five to eight for gate|up matrices of more
+// than four pairs of row tiles a compute unit.  A matrix of a few thousand rows has too
 // few groups of row tiles to give every compute unit work, so K is cut into `parts` stretches (blockIdx.y) whose float32 sums go to out[part][M][N] for a reader
 // that adds them in order (the residual stream's norm, or ri_sum_parts below).  A row's result does not
 // depend on the number of rows: rows beyond M are zero columns, every tile of x has accumulators of its own.
@@ -189,6 +190,17 @@ static int wide_parts(int groups, int k_tiles, bool swiglu, int cus) {
 extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts) {
     const int row_tiles = (n + 15) / 16, k_tiles = (k + 31) / 32;
     const int cus = ri_compute_units();
+    if (swiglu && row_tiles > 4 * cus && row_tiles <= 8 * cus) {
+        // With the activation K stays whole, and pairs of row tiles for more than four wavefronts a compute unit
+        // would be a second round on some of them (groups of three or four: two workgroups on some compute units,
+        // one on others, and the product takes what the fuller ones take).  Up to eight wavefronts a workgroup
+        // bring the groups within the compute units' number again: 1,088 pairs (17408 x 5120) in 218 groups of
+        // five take 61 to 71 us at 24 to 64 rows where 363 groups of three take 74 to 93; 1,600 pairs (25600 x
+        // 5120) in 229 groups of seven 87 to 95 us where 400 groups of four take 97 to 113.
+        *waves = (row_tiles + cus - 1) / cus;
+        *parts = 1;
+        return 0;
+    }
     double best = -1.0;
     for (int w = 4; w >= 3; --w) {
         const int groups = (row_tiles + w - 1) / w;
@@ -274,7 +286,8 @@ static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t*
             (bf16_t*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
 }
 
-// depth: slices of weights a wavefront keeps in flight (1 or 2); waves: wavefronts (row tiles) a workgroup (3 or 4).
+// depth: slices of weights a wavefront keeps in flight (1 or 2); waves: wavefronts (row tiles) a workgroup (3 or 4;
+// with the activation and depth 1 up to 8).
 // (Eight wavefronts on eight row tiles, with K in twice the stretches so that the workgroups stay as many and each
 // fetches half the rows of x, were timed at 17 to 64 rows: at 4096 x 4096 and 4096 x 12288 level or behind, 14.1
 // against 13.6 us and 24.8 against 24.2 us at 64 rows, and the reading norm then adds twice the stretches.)
@@ -291,7 +304,8 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
     RI_REQUIRE(!(tiled & ~(TILED_X | TILED_OUT)) && (!(tiled & TILED_OUT) || (out_dtype == RI_BF16 && parts == 1)),
                "gemm_wide_packed_bf16: layout flags %d (a tiled result is bfloat16 and whole)", tiled);
     RI_REQUIRE(depth == 1 || depth == 2, "gemm_wide_packed_bf16: depth %d", depth);
-    RI_REQUIRE(waves == 3 || waves == 4, "gemm_wide_packed_bf16: %d wavefronts a workgroup (3 or 4)", waves);
+    RI_REQUIRE(waves == 3 || waves == 4 || (waves >= 5 && waves <= 8 && swiglu && depth == 1 && m <= 64),
+               "gemm_wide_packed_bf16: %d wavefronts a workgroup (3 or 4; 5 to 8 too with the activation at depth 1)", waves);
     hipStream_t s = (hipStream_t)stream;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)wpacked;
@@ -308,7 +322,20 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
         if (waves == 3) launch_wide_pairs<RT, 3>((float*)out, xb, wb, m, n, k, parts, s);       \
         else            launch_wide_pairs<RT, 4>((float*)out, xb, wb, m, n, k, parts, s);       \
     } while (0)
-    if (m <= 16)       { RI_WIDE_CASE(1) }
+#define RI_WIDE_MANY(RT)                                                                                     \
+    do {                                                                                                     \
+        if (waves == 5)      launch_wide<RT, true, 1, 5>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s);  \
+        else if (waves == 6) launch_wide<RT, true, 1, 6>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s);  \
+        else if (waves == 7) launch_wide<RT, true, 1, 7>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s);  \
+        else                 launch_wide<RT, true, 1, 8>(out, out_dtype, xb, wb, m, n, k, parts, tiled, s);  \
+    } while (0)
+    if (waves > 4) {
+        if (m <= 16)      RI_WIDE_MANY(1);
+        else if (m <= 32) RI_WIDE_MANY(2);
+        else if (m <= 48) RI_WIDE_MANY(3);
+        else              RI_WIDE_MANY(4);
+    }
+    else if (m <= 16)  { RI_WIDE_CASE(1) }
     else if (m <= 32)  { RI_WIDE_CASE(2) }
     else if (m <= 48)  { RI_WIDE_CASE(3) }
     else if (m <= 64)  { RI_WIDE_CASE(4) }
@@ -317,6 +344,7 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
     else if (m <= 112) RI_WIDE_PAIRS(7);
     else               RI_WIDE_PAIRS(8);
 #undef RI_WIDE_PAIRS
+#undef RI_WIDE_MANY
 #undef RI_WIDE_CASE
 #undef RI_WIDE_GO
     RI_LAUNCH_CHECK("gemm_wide_packed_bf16");

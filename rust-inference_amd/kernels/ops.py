@@ -542,7 +542,7 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
     ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
     that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
     ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``.  ``waves``: wavefronts (row tiles) a
-    workgroup, 3 or 4 (``wide_product_plan``); the sums do not depend on it."""
+    workgroup, 3 or 4, with the activation at ``depth`` 1 up to 8 (``wide_product_plan``); the sums do not depend on it."""
     m, k = x.shape
     row_tiles = -(-n // 16)
     want = (row_tiles * (2 if swiglu else 1), -(-k // 32), 64, 8)

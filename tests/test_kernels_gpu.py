@@ -713,8 +713,17 @@ def test_wide_packed_product(ops, m, n, k):
                        ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, parts=3))
     assert torch.equal(ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, waves=3, tiled_out=True).rows(),
                        ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True))
+    # five to eight wavefronts a workgroup (matrices of more than a thousand pairs of row tiles): the same bits
+    gated = ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, depth=1)
+    for many in (5, 6, 7, 8):
+        assert torch.equal(ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, depth=1, waves=many), gated)
+    assert torch.equal(ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, depth=1, waves=7, tiled_out=True).rows(), gated)
+    with pytest.raises(Exception, match="wavefronts"):
+        ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, waves=5)
     waves, parts = ops.wide_product_plan(n, k, True)
     assert waves in (3, 4) and parts == 1                   # the activation is never left to a second kernel
+    assert ops.wide_product_plan(16 * 4 * ops.compute_units() + 16, k, True) == (5, 1)
+    assert ops.wide_product_plan(16 * 7 * ops.compute_units(), k, True) == (7, 1)
     # rows in the matrix cores' order on either side: the same bits
     tiled = ops.sum_parts(x.float()[None].contiguous(), torch.bfloat16, tiled_out=True)
     assert torch.equal(tiled.rows(), x)
