@@ -721,7 +721,7 @@ def test_wide_packed_product(ops, m, n, k):
     with pytest.raises(Exception, match="wavefronts"):
         ops.gemm_wide_packed_bf16(x, packed, n, torch.float32, waves=5)
     waves, parts = ops.wide_product_plan(n, k, True)
-    assert waves in (3, 4) and parts == 1                   # the activation is never left to a second kernel
+    assert 3 <= waves <= 8 and parts == 1                   # the activation is never left to a second kernel
     assert ops.wide_product_plan(16 * 4 * ops.compute_units() + 16, k, True) == (5, 1)
     assert ops.wide_product_plan(16 * 7 * ops.compute_units(), k, True) == (7, 1)
     # rows in the matrix cores' order on either side: the same bits
