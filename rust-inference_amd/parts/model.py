@@ -90,7 +90,7 @@ class OutputHead(Head):
         return plain.linear(x, self.weight_plain)
 
     def _packed_copy(self):
-        """A second copy of the matrix in the matrix cores' tile order, for steps that want 2 to 32 rows of
+        """A second copy of the matrix in the matrix cores' tile order, for steps that want 2 to 32 or 48 rows of
         logits (a decode step of as many sequences): at 151,936 x 4,096 the packed kernel takes 0.21 ms where
         the library's product takes 0.26 (1% of such a step), for 1.2 GB more memory.  It is made at the first
         such step, so that a model which never runs one (a single slot, or only larger batches) does not pay
@@ -100,18 +100,23 @@ class OutputHead(Head):
         return self.packed
 
     # Rows of logits up to which the packed copy serves: 2 to 8 the packed kernel (one load of x serves two steps of
-    # K there); 9 to 32 the wide kernel with four row tiles a workgroup, which shares the rows of x through LDS
+    # K there); from 9 on the wide kernel with four row tiles a workgroup, which shares the rows of x through LDS
     # (151,936 x 4,096 at 9, 16, 17 and 32 rows: 204, 213, 222 and 247 us against the packed kernel's 224 and 279
     # and the library's 250 to 279; x 1,024 at 16 rows 57 against 78; x 5,120: 254 against 382; from 48 rows on the
-    # library is ahead, 266 against 279 us, with 39 MB of float32 logits to write).
+    # library is ahead, 266 against 279 us, with 39 MB of float32 logits to write).  33 to 48 rows with three tiles of
+    # x, for rows of up to 4,096 elements: eight layers and this matrix at 33 / 40 / 47 sequences are 1.5 / 1.5 / 0.9%
+    # shorter at Qwen3-0.6B sizes, 3.7 / 2.8 / 1.8% at 4B, 1.2 / 0.8 / 0% at 8B; with rows of 5,120 (32B) 0 to 0.7% longer.
     PACKED_MAX_ROWS = 32
+    PACKED_MORE_ROWS = 48            # for rows of up to PACKED_MORE_DIM elements
+    PACKED_MORE_DIM = 4096
     PAIRED_MAX_ROWS = 8
 
     def forward(self, x):
         rows = x.shape[0]
         if self.rt.invariant:
             return self.rt.linear_packed(x, self._packed_copy(), out_dtype=torch.float32)
-        if 2 <= rows <= self.PACKED_MAX_ROWS and self.dim % 8 == 0:
+        most = self.PACKED_MORE_ROWS if self.dim <= self.PACKED_MORE_DIM else self.PACKED_MAX_ROWS
+        if 2 <= rows <= most and self.dim % 8 == 0:
             packed = self._packed_copy()
             if packed is not None and packed.packed is not None:
                 if rows <= self.PAIRED_MAX_ROWS:
