@@ -46,7 +46,7 @@ __device__ __forceinline__ float silu_wd(float z) { return z / (1.0f + expf(-z))
 template <int RT, bool SWIGLU, typename TO, int NS, int W, bool PAIR = false>
 __global__ void __launch_bounds__(W * 64)
 gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ wpacked, int M,
-                        int N, int K, int k_tiles, int part_tiles, int row_tiles, int tiled) {
+                        int N, int K, int k_tiles, int part_tiles, int row_tiles, int tiled, long part_stride) {
     constexpr int FRAGS = RT * WD_SLICE;                     // fragments of x (64 pieces of 16 bytes) in a slice
     constexpr int PER_THREAD = (FRAGS + W - 1) / W;          // of which a wavefront copies this many
     __shared__ uint4 xs[2][RT][WD_SLICE][64];
@@ -150,7 +150,7 @@ gemm_wide_packed_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, cons
     // columns 0..N-1 and the up sums N..2N-1 of rows 2 N wide.
     const bool raw = gridDim.y > 1;
     const int width = (SWIGLU && raw) ? 2 * N : N;
-    out += (size_t)blockIdx.y * M * width;
+    out += (size_t)blockIdx.y * part_stride;          // (M * width, or more where the rows are a slice of a taller result)
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int m = rt * 16 + (lane & 15);
@@ -235,6 +235,10 @@ extern "C" int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* wave
 // behind on 4096 x 12288, whose stretches get short.)
 extern "C" int ri_gemm_wide_stretch_plan(int m, int n, int k, int* waves, int* parts) {
     if (m <= 16) return ri_gemm_wide_packed_bf16_plan(n, k, 0, waves, parts);
+    if (m > 128) {                                            // two passes: the plan for the taller one
+        const int tiles = (m + 15) / 16, passes = (tiles + 7) / 8;
+        m = (tiles + passes - 1) / passes * 16;
+    }
     const int row_tiles = (n + 15) / 16, k_tiles = (k + 31) / 32;
     const int cus = ri_compute_units();
     const int x_rows = (m + 15) / 16 * 16;
@@ -264,12 +268,13 @@ extern "C" int ri_gemm_wide_stretch_plan(int m, int n, int k, int* waves, int* p
 }
 
 template <int RT, int W>
-static void launch_wide_pairs(float* out, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts, hipStream_t s) {
+static void launch_wide_pairs(float* out, const bf16_t* x, const bf16_t* w, int m, int n, int k, int parts, long part_stride,
+                              hipStream_t s) {
     const int k_tiles = (k + 31) / 32, row_tiles = (n + 15) / 16;
     const int part_tiles = ((k_tiles + parts - 1) / parts + WD_SLICE - 1) / WD_SLICE * WD_SLICE;
     dim3 grid((row_tiles + 2 * W - 1) / (2 * W), parts);
     gemm_wide_packed_kernel<RT, false, float, 1, W, true><<<grid, W * 64, 0, s>>>(out, x, w, m, n, k, k_tiles, part_tiles,
-                                                                                 row_tiles, 0);
+                                                                                 row_tiles, 0, part_stride);
 }
 
 template <int RT, bool SWIGLU, int NS, int W>
@@ -280,10 +285,10 @@ static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t*
     dim3 grid((row_tiles + W - 1) / W, parts);
     if (out_dtype == RI_F32)
         gemm_wide_packed_kernel<RT, SWIGLU, float, NS, W><<<grid, W * 64, 0, s>>>(
-            (float*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
+            (float*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled, (long)m * (SWIGLU && parts > 1 ? 2 * n : n));
     else
         gemm_wide_packed_kernel<RT, SWIGLU, bf16_t, NS, W><<<grid, W * 64, 0, s>>>(
-            (bf16_t*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled);
+            (bf16_t*)out, x, w, m, n, k, k_tiles, part_tiles, row_tiles, tiled, (long)m * n);
 }
 
 // depth: slices of weights a wavefront keeps in flight (1 or 2); waves: wavefronts (row tiles) a workgroup (3 or 4;
@@ -293,7 +298,7 @@ static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t*
 // against 13.6 us and 24.8 against 24.2 us at 64 rows, and the reading norm then adds twice the stretches.)
 extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
                                         int k, int swiglu, int parts, int tiled, int depth, int waves, void* stream) {
-    RI_REQUIRE(m > 0 && m <= 128, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 128", m);
+    RI_REQUIRE(m > 0 && m <= 256, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 256", m);
     RI_REQUIRE(m <= 64 || (!swiglu && out_dtype == RI_F32 && !tiled && depth == 1),
                "gemm_wide_packed_bf16: %d rows of x: more than 64 give float32 sums in plain rows from plain rows, "
                "without the activation, one slice of weights in flight", m);
@@ -317,10 +322,10 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
 #define RI_WIDE_CASE(RT)                                                                  \
     if (swiglu) { if (depth == 2) RI_WIDE_GO(RT, true, 2); else RI_WIDE_GO(RT, true, 1); } \
     else        { if (depth == 2) RI_WIDE_GO(RT, false, 2); else RI_WIDE_GO(RT, false, 1); }
-#define RI_WIDE_PAIRS(RT)                                                                      \
-    do {                                                                                        \
-        if (waves == 3) launch_wide_pairs<RT, 3>((float*)out, xb, wb, m, n, k, parts, s);       \
-        else            launch_wide_pairs<RT, 4>((float*)out, xb, wb, m, n, k, parts, s);       \
+#define RI_WIDE_PAIRS(RT)                                                                                  \
+    do {                                                                                                    \
+        if (waves == 3) launch_wide_pairs<RT, 3>(po, px, wb, rows, n, k, parts, (long)m * n, s);            \
+        else            launch_wide_pairs<RT, 4>(po, px, wb, rows, n, k, parts, (long)m * n, s);            \
     } while (0)
 #define RI_WIDE_MANY(RT)                                                                                     \
     do {                                                                                                     \
@@ -339,10 +344,26 @@ extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x,
     else if (m <= 32)  { RI_WIDE_CASE(2) }
     else if (m <= 48)  { RI_WIDE_CASE(3) }
     else if (m <= 64)  { RI_WIDE_CASE(4) }
-    else if (m <= 80)  RI_WIDE_PAIRS(5);
-    else if (m <= 96)  RI_WIDE_PAIRS(6);
-    else if (m <= 112) RI_WIDE_PAIRS(7);
-    else               RI_WIDE_PAIRS(8);
+    else {
+        // 65 to 128 rows in one pass, up to 256 in two of as many tiles of 16 rows each as can be (the second may
+        // have one less): each pass reads the weights once and writes its rows of every stretch's float32 sums
+        const int tiles = (m + 15) / 16, passes = (tiles + 7) / 8;
+        int r0 = 0;
+        for (int pass = 0; pass < passes; ++pass) {
+            const int pass_tiles = tiles / passes + (pass < tiles % passes ? 1 : 0);
+            const int rows = min(pass_tiles * 16, m - r0);
+            float* po = (float*)out + (size_t)r0 * n;
+            const bf16_t* px = xb + (size_t)r0 * k;
+            switch (pass_tiles) {
+                case 4: RI_WIDE_PAIRS(4); break;
+                case 5: RI_WIDE_PAIRS(5); break;
+                case 6: RI_WIDE_PAIRS(6); break;
+                case 7: RI_WIDE_PAIRS(7); break;
+                default: RI_WIDE_PAIRS(8); break;
+            }
+            r0 += rows;
+        }
+    }
 #undef RI_WIDE_PAIRS
 #undef RI_WIDE_MANY
 #undef RI_WIDE_CASE

@@ -537,8 +537,8 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
                           parts: int = 1, tiled_out: bool = False, depth: int = 2, waves: int = 4):
     """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by ``pack_for_mfma``,
     the tiles of x shared by a workgroup's wavefronts through LDS: the product for steps of 17 to 64 tokens.
-    65 to 128 plain rows: float32 sums in rows (``waves`` and ``parts`` from ``wide_product_plan(..., rows=m)``),
-    ``depth`` 1.
+    65 to 256 plain rows (past 128 in two passes over the weights): float32 sums in rows (``waves`` and ``parts``
+    from ``wide_product_plan(..., rows=m)``), ``depth`` 1.
     ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
     that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
     ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``.  ``waves``: wavefronts (row tiles) a

@@ -25,7 +25,7 @@ def _wide_plan(n: int, k: int, swiglu: bool, rows: int = 64) -> tuple[int, int]:
 #              gate|up pairs fill the machine; the packed kernel with two or four tiles of x on small matrices
 #              and up to 32 rows of tiled x; else the library.
 #   65-128     the wide kernel with two row tiles a wavefront for matrices of long rows whose reader adds stretches
-#              of K (`down`); else the library.
+#              of K (`down`; up to 256 rows for the longest); else the library.
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
 GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
@@ -37,6 +37,7 @@ WIDE_MIN_K = 4096                # rows shorter than this leave the wide kernel'
 WIDE_MIN_ROWS = 17
 PAIRS_MAX_ROWS = 128             # 65 to 128 rows: the wide kernel with two row tiles a wavefront, where the library does badly:
 PAIRS_MIN_K = 8192               # matrices of long rows (and at least twice as long as there are rows: `down`)
+PAIRS_MORE_ROWS = 256            # and in two passes up to this many rows where the rows have PACKED_LONG_K elements and more
 SMALL_ONLY_ROWS = 64             # a matrix packed for small steps alone stays on the wide kernel up to this many rows
 # (5,120 x 8,192 at 32 / 48 / 64 rows: 20 / 24 / 29 us against the library's 19 to 34 / 30 / 23; 5,120 x 5,120: 15 / 18 / 21 against 19 / 20 / 19;
 # with three stretches of 80 groups of four wavefronts 24 and 18 us at 64 rows: a step of 49 to 64 sequences 1 to 1.6% shorter at those sizes)
@@ -267,10 +268,11 @@ class Runtime:
                 x = self.normed_now(x) if later else x
                 waves, parts = _wide_plan(pw.n, pw.k, False, -(-m // 16) * 16)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
-            if (MID_MAX_ROWS < m <= PAIRS_MAX_ROWS and pw.packed is not None and parts_ok and not pw.swiglu
-                    and pw.k >= PAIRS_MIN_K and pw.k >= 2 * pw.n):
+            if (MID_MAX_ROWS < m <= (PAIRS_MORE_ROWS if pw.k >= PACKED_LONG_K else PAIRS_MAX_ROWS) and pw.packed is not None
+                    and parts_ok and not pw.swiglu and pw.k >= PAIRS_MIN_K and pw.k >= 2 * pw.n):
                 # 65 to 128 rows against a matrix of long rows whose result goes into the residual stream (`down`):
                 # the wide kernel with two row tiles a wavefront, K in stretches that the stream's next norm adds
+                # (the longest rows up to 256 rows of x, in two passes over the weights)
                 x = self.normed_now(x) if later else x
                 x = x.rows() if isinstance(x, ops.TiledRows) else x
                 waves, parts = _wide_plan(pw.n, pw.k, False, -(-m // 16) * 16)

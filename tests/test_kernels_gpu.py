@@ -734,12 +734,12 @@ def test_wide_packed_product(ops, m, n, k):
         assert torch.equal(whole[m - 1:], ops.gemm_wide_packed_bf16(x[m - 1:].contiguous(), packed, n, torch.float32))
 
 
-@pytest.mark.parametrize("m", [65, 80, 81, 100, 113, 128])
+@pytest.mark.parametrize("m", [65, 80, 81, 100, 113, 128, 129, 150, 200, 256])
 @pytest.mark.parametrize("n, k", [(37, 72), (1000, 1024), (584, 12288), (4096, 4096), (70, 264), (16, 520)])
-def test_wide_packed_product_of_65_to_128_rows(ops, m, n, k):
+def test_wide_packed_product_of_65_to_256_rows(ops, m, n, k):
     """Five to eight tiles of x, two row tiles of the matrix a wavefront (an odd number of row tiles leaves the last
-    wavefront one): whole and in parts of K that add up, with three and four wavefronts a workgroup; a row's sums
-    are those of the kernel for up to 64 rows, bit for bit."""
+    wavefront one), past 128 rows in two passes (129 rows: five tiles and four): whole and in parts of K that add up,
+    with three and four wavefronts a workgroup; a row's sums are those of the kernel for up to 64 rows, bit for bit."""
     rng = np.random.default_rng(m + n + k)
     x, w = t(rng.normal(size=(m, k)), torch.bfloat16), t(rng.normal(size=(n, k)), torch.bfloat16)
     want = f64(x) @ f64(w).T
@@ -760,8 +760,8 @@ def test_wide_packed_product_of_65_to_128_rows(ops, m, n, k):
         assert torch.equal(got[..., :64, :], first) and torch.equal(got[..., m - 1:, :], last)
     with pytest.raises(Exception, match="64"):
         ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16)
-    with pytest.raises(Exception, match="128"):
-        ops.gemm_wide_packed_bf16(t(rng.normal(size=(129, k)), torch.bfloat16), packed, n, torch.float32)
+    with pytest.raises(Exception, match="256"):
+        ops.gemm_wide_packed_bf16(t(rng.normal(size=(257, k)), torch.bfloat16), packed, n, torch.float32)
 
 
 @pytest.mark.parametrize("packed, m", [(False, 1), (False, 2), (False, 5), (True, 1), (True, 3), (True, 16)])
