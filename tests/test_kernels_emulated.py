@@ -105,7 +105,7 @@ def test_the_sampler_tests_pass_on_the_cpu_build_between_guard_pages(runs):
     _passed(runs["sampler"], 33)
 
 
-@pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 49)])
+@pytest.mark.parametrize("units, tests", [("sixteen units", 7), ("one unit", 61)])
 def test_the_forms_that_a_large_step_chooses_on_a_machine_made_small(runs, units, tests):
     """tests/small_machine_kernels.py: the emulated runtime reports a few compute units, so that the walk in runs, the
     joins of many pieces and the run of more than 1,024 pages are chosen for one or two heads; with one unit also
