@@ -41,7 +41,7 @@ PAIRS_MORE_ROWS = 256            # and in two passes up to this many rows where 
 SMALL_ONLY_ROWS = 64             # a matrix packed for small steps alone stays on the wide kernel up to this many rows
 # (5,120 x 8,192 at 32 / 48 / 64 rows: 20 / 24 / 29 us against the library's 19 to 34 / 30 / 23; 5,120 x 5,120: 15 / 18 / 21 against 19 / 20 / 19;
 # with three stretches of 80 groups of four wavefronts 24 and 18 us at 64 rows: a step of 49 to 64 sequences 1 to 1.6% shorter at those sizes)
-WIDE_GATED_FILL = 0.8            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds,
+WIDE_GATED_FILL = 0.75            # gate|up goes to the wide kernel where its workgroups fill this share of the rounds,
 WIDE_GATED_ROWS = 48             # and up to this many rows whatever they fill, if the packed kernel of 17 to 64 rows is no match:
 WIDE_GATED_BYTES = 64_000_000    # pairs larger than this (smaller ones, up to 32 tiled rows, are that kernel's)
 SPLIT_K = 4096                   # pieces of a long K (PACKED_LONG_K and more) whose sums the next norm adds
