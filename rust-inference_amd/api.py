@@ -6,6 +6,7 @@ caches, loop {forward, pick, stop?, append}) with its runner's option names
 """
 from __future__ import annotations
 
+import math
 from typing import Sequence
 
 import torch
@@ -29,14 +30,41 @@ def as_dtype(dtype) -> torch.dtype:
         raise ValueError(f"dtype {dtype!r}: expected bfloat16 or float32") from None
 
 
+# A graph of a batch size is worth capturing at once where launching a step's kernels from the host takes as long as
+# the step: a small model.  Where the step's weights take longer to read than its kernels to launch, host launches
+# cost a few per cent and the capture what several steps take, so a size that lives for a step or two is better left
+# without one.  The two times are estimated from what is known before any step has run: the weights' bytes at 5 TB/s,
+# and seven launches a layer at 8 us.  Measured through generate(), ms for the whole call, capture at the first step :
+# after the third: 200 prompts whose sequences stop at random steps (a hundred batch sizes) on three layers of
+# Qwen3-14B sizes 365 : 268, on Qwen3-0.6B 642 : 693; 64 prompts on twelve layers of Qwen3-8B sizes 655 : 578, 16
+# prompts there 316 : 308, 16 prompts on Qwen3-0.6B 541 : 545.
+_WEIGHTS_BYTES_PER_SECOND = 5e12
+_LAUNCH_SECONDS, _LAUNCHES_PER_LAYER = 8e-6, 7
+_DEFERRED_CAPTURE = 3
+
+
+def capture_after_for(decoder) -> int:
+    """How many steps of a batch size should run with host launches before their graph is captured, for this model."""
+    try:
+        width = 2 if decoder.rt.dtype == torch.bfloat16 else 4
+        elements = sum(math.prod(spec.shape) for spec in decoder.tensors().values())
+        layers = len(decoder.schedule)
+    except Exception:
+        return 0
+    reading = elements * width / _WEIGHTS_BYTES_PER_SECOND
+    launching = layers * _LAUNCHES_PER_LAYER * _LAUNCH_SECONDS
+    return _DEFERRED_CAPTURE if reading > launching else 0
+
+
 class Model:
     """A loaded model with a cache sized for ``max_batch`` sequences of ``max_seq_len`` tokens.
     ``graph_after``: decode steps of one batch size run that many times with host launches before their graph is
     captured (capturing costs 3 to 5 steps' time, and a batch whose sequences stop at different times passes
-    through many sizes); 0, the default, captures at the first step of a size."""
+    through many sizes); 0 captures at the first step of a size; None, the default, chooses by the model's size
+    (``capture_after_for``)."""
 
     def __init__(self, decoder, max_batch: int = 8, max_seq_len: int = 4096, max_tokens: int | None = None,
-                 use_graphs: bool = True, plain: bool = False, graph_after: int = 0):
+                 use_graphs: bool = True, plain: bool = False, graph_after: int | None = None):
         self.decoder = decoder
         self.config = getattr(decoder, "config", None)
         per_seq = -(-max_seq_len // PAGE_SIZE) * PAGE_SIZE
@@ -45,6 +73,8 @@ class Model:
             self.cache = self.engine.cache
         else:
             self.cache = decoder.new_cache(max_tokens or per_seq * max_batch, max_batch, max_seq_len)
+            if graph_after is None:
+                graph_after = capture_after_for(decoder) if use_graphs else 0
             self.engine = Engine(decoder, self.cache, use_graphs=use_graphs, capture_after=graph_after)
 
     @classmethod

@@ -376,3 +376,21 @@ def test_every_request_may_sample_in_its_own_way():
     assert len({tuple(t) for t in mixed}) > 1
     with pytest.raises(ShapeError, match="sampling parameters"):
         generate(Peaked(), prompts, max_new_tokens=2, sampling=kinds[:2])
+
+
+def test_whether_a_graph_waits_for_a_batch_size_to_come_back_goes_by_the_models_size():
+    """Capturing at a size's first step pays where launching a step costs what the step costs (a small model); a
+    model whose weights take longer to read than its kernels to launch captures a size only when it has come back."""
+    import types
+    import bench
+    from rust_inference_amd.api import capture_after_for
+    from rust_inference_amd.config import config_from_dict
+    from rust_inference_amd.parts.model import DecoderModel
+    waits = {}
+    for which, (_, shapes, _) in bench.MODELS.items():
+        arch, cfg = config_from_dict(dict(shapes))
+        model = DecoderModel(arch.build_spec(cfg))
+        model.rt = types.SimpleNamespace(dtype=torch.bfloat16)
+        waits[which] = capture_after_for(model)
+    assert waits == {"0.6b": 0, "1.7b": 0, "4b": 0, "8b": 3, "14b": 3, "32b": 3}
+    assert capture_after_for(object()) == 0                 # nothing known about it: as before
