@@ -143,7 +143,8 @@ int ri_finish_norm(void* out, const void* xg, const float* ssq, int n_in, float 
 // float32 sums go to out[parts][m][n]; ri_gemm_wide_packed_bf16_plan says how many wavefronts and parts fill
 // the machine most evenly for a matrix (with swiglu: never parts).  tiled as in ri_gemm_skinny_packed_bf16.
 // 65 to 128 rows of x: every wavefront takes two neighbouring row tiles; float32 sums in plain rows, no
-// activation, x in plain rows, depth 1.  129 to 256 rows: two such passes.  ri_gemm_wide_stretch_plan: wavefronts and stretches for a product of m
+// activation, x in plain rows, depth 1.  129 to 256 rows: two such passes.  With the activation 65 to 128 rows
+// are taken with five to eight wavefronts a workgroup (K whole, plain rows in and out, depth 1).  ri_gemm_wide_stretch_plan: wavefronts and stretches for a product of m
 // rows without the activation.
 int ri_gemm_wide_packed_bf16_plan(int n, int k, int swiglu, int* waves, int* parts);
 int ri_gemm_wide_stretch_plan(int m, int n, int k, int* waves, int* parts);

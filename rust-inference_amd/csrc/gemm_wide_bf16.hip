@@ -299,6 +299,33 @@ static void launch_wide(void* out, int out_dtype, const bf16_t* x, const bf16_t*
 extern "C" int ri_gemm_wide_packed_bf16(void* out, int out_dtype, const void* x, const void* wpacked, int m, int n,
                                         int k, int swiglu, int parts, int tiled, int depth, int waves, void* stream) {
     RI_REQUIRE(m > 0 && m <= 256, "gemm_wide_packed_bf16: %d rows of x, this kernel takes 1 to 256", m);
+    if (m > 64 && m <= 128 && swiglu) {
+        // 65 to 128 rows with the activation, for the matrices that take five to eight wavefronts a workgroup: five to
+        // eight tiles of x, K whole, a gate tile and its up tile a wavefront (17408 x 5120 pairs at 65 / 96 / 128 rows:
+        // 76 / 88 / 98 us against the library's and its activation kernel's 102 / 103 / 108; 25600 x 5120: 95 / 103 / 121
+        // against 113 / 116 / 125; with three or four wavefronts, 12288 x 4096 and 9728 x 2560, it is ahead up to 80
+        // rows only, 54 and 32 us against 56 to 58 and 34, and loses beyond: 74 and 50 against 57 and 35 at 128)
+        RI_REQUIRE(depth == 1 && parts == 1 && !tiled && waves >= 5 && waves <= 8,
+                   "gemm_wide_packed_bf16: %d rows with the activation: depth 1, K whole, plain rows, 5 to 8 wavefronts", m);
+        hipStream_t s2 = (hipStream_t)stream;
+        const bf16_t* xb2 = (const bf16_t*)x;
+        const bf16_t* wb2 = (const bf16_t*)wpacked;
+#define RI_WIDE_TALL_W(RT, W) launch_wide<RT, true, 1, W>(out, out_dtype, xb2, wb2, m, n, k, 1, 0, s2)
+#define RI_WIDE_TALL(RT)                                                                           \
+    do {                                                                                           \
+        switch (waves) {                                                                           \
+            case 5: RI_WIDE_TALL_W(RT, 5); break;                                                  \
+            case 6: RI_WIDE_TALL_W(RT, 6); break;                                                  \
+            case 7: RI_WIDE_TALL_W(RT, 7); break;                                                  \
+            default: RI_WIDE_TALL_W(RT, 8); break;                                                 \
+        }                                                                                          \
+    } while (0)
+        if (m <= 80) RI_WIDE_TALL(5); else if (m <= 96) RI_WIDE_TALL(6); else if (m <= 112) RI_WIDE_TALL(7); else RI_WIDE_TALL(8);
+#undef RI_WIDE_TALL
+#undef RI_WIDE_TALL_W
+        RI_LAUNCH_CHECK("gemm_wide_packed_bf16");
+        return 0;
+    }
     RI_REQUIRE(m <= 64 || (!swiglu && out_dtype == RI_F32 && !tiled && depth == 1),
                "gemm_wide_packed_bf16: %d rows of x: more than 64 give float32 sums in plain rows from plain rows, "
                "without the activation, one slice of weights in flight", m);

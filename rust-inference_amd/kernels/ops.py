@@ -538,7 +538,8 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
     """``x @ w.T`` for up to 64 bfloat16 rows (a tensor or ``TiledRows``) with ``w`` packed by ``pack_for_mfma``,
     the tiles of x shared by a workgroup's wavefronts through LDS: the product for steps of 17 to 64 tokens.
     65 to 256 plain rows (past 128 in two passes over the weights): float32 sums in rows (``waves`` and ``parts``
-    from ``wide_product_plan(..., rows=m)``), ``depth`` 1.
+    from ``wide_product_plan(..., rows=m)``), ``depth`` 1; with ``swiglu`` 65 to 128 plain rows where the plan says
+    five to eight wavefronts, K whole.
     ``parts > 1``: K in that many stretches, the result their float32 sums ``[parts, M, n]`` for a reader
     that adds them (with ``swiglu`` ``[parts, M, 2 n]``, gate sums then up sums, the activation left to
     ``sum_parts``).  ``tiled_out``: the bfloat16 result as ``TiledRows``.  ``waves``: wavefronts (row tiles) a
@@ -549,8 +550,9 @@ def gemm_wide_packed_bf16(x, wpacked: torch.Tensor, n: int, out_dtype=torch.bflo
     if tuple(wpacked.shape) != want:
         raise ShapeError(f"packed weight is {list(wpacked.shape)}, a product with n {n}, k {k} wants {list(want)}")
     if m > 64:
-        if swiglu or out_dtype != torch.float32 or tiled_out or isinstance(x, TiledRows):
-            raise ShapeError("more than 64 rows: float32 sums in plain rows from plain rows, without the activation")
+        if tiled_out or isinstance(x, TiledRows) or (not swiglu and out_dtype != torch.float32) or (swiglu and (parts != 1 or m > 128)):
+            raise ShapeError("more than 64 rows: plain rows in and out; float32 sums without the activation, "
+                             "or up to 128 rows with it and K whole")
         depth = 1
     if parts != 1 and (out_dtype != torch.float32 or tiled_out):
         raise ShapeError("a product in parts has float32 sums in rows")

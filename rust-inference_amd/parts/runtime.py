@@ -25,7 +25,7 @@ def _wide_plan(n: int, k: int, swiglu: bool, rows: int = 64) -> tuple[int, int]:
 #              gate|up pairs fill the machine; the packed kernel with two or four tiles of x on small matrices
 #              and up to 32 rows of tiled x; else the library.
 #   65-128     the wide kernel with two row tiles a wavefront for matrices of long rows whose reader adds stretches
-#              of K (`down`; up to 256 rows for the longest); else the library.
+#              of K (`down`; up to 256 rows for the longest), and for the largest gate|up pairs; else the library.
 #   more       the vendor library (the reference hands every product to one: src/cuda/mod.rs:186-232).
 GEMV_MAX_ROWS = 1
 SKINNY_MAX_ROWS = 16
@@ -277,6 +277,13 @@ class Runtime:
                 x = x.rows() if isinstance(x, ops.TiledRows) else x
                 waves, parts = _wide_plan(pw.n, pw.k, False, -(-m // 16) * 16)
                 return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, torch.float32, parts=parts, depth=1, waves=waves)
+            if MID_MAX_ROWS < m <= PAIRS_MAX_ROWS and pw.swiglu and pw.packed is not None:
+                # 65 to 128 rows of the largest gate|up pairs (those that take five to eight wavefronts a workgroup)
+                waves, _ = _wide_plan(pw.n, pw.k, True)
+                if waves > 4:
+                    x = self.normed_now(x) if later else x
+                    x = x.rows() if isinstance(x, ops.TiledRows) else x
+                    return ops.gemm_wide_packed_bf16(x, pw.packed, pw.n, out_dtype, swiglu=True, depth=1, waves=waves)
             if WIDE_MIN_ROWS <= m <= MID_MAX_ROWS and pw.swiglu and self._wide_gated(pw, m):
                 x = self.normed_now(x) if later else x
                 waves, _ = _wide_plan(pw.n, pw.k, True)

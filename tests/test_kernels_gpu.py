@@ -758,6 +758,17 @@ def test_wide_packed_product_of_65_to_256_rows(ops, m, n, k):
         first = ops.gemm_wide_packed_bf16(x[:64].contiguous(), packed, n, torch.float32, parts=parts, depth=1)
         last = ops.gemm_wide_packed_bf16(x[m - 1:].contiguous(), packed, n, torch.float32, parts=parts, depth=1)
         assert torch.equal(got[..., :64, :], first) and torch.equal(got[..., m - 1:, :], last)
+    if m <= 128:        # with the activation, five to eight wavefronts a workgroup: the bits of the kernel for 64 rows
+        wgu = t(rng.normal(size=(2 * n, k)) * (4.0 / np.sqrt(k)), torch.bfloat16)
+        y = f64(x) @ f64(wgu).T
+        pgu = ops.pack_for_mfma(wgu, swiglu=True)
+        gated = ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, waves=5)
+        close(gated, P.silu(y[:, :n]) * y[:, n:], 5e-3, "more than 64 rows with the activation")
+        for many in (6, 7, 8):
+            assert torch.equal(ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, waves=many), gated)
+        assert torch.equal(gated[:64], ops.gemm_wide_packed_bf16(x[:64].contiguous(), pgu, n, torch.bfloat16, swiglu=True, depth=1))
+        with pytest.raises(Exception, match="wavefronts"):
+            ops.gemm_wide_packed_bf16(x, pgu, n, torch.bfloat16, swiglu=True, waves=4)
     with pytest.raises(Exception, match="64"):
         ops.gemm_wide_packed_bf16(x, packed, n, torch.bfloat16)
     with pytest.raises(Exception, match="256"):
